@@ -1,0 +1,134 @@
+/*
+ * lce.h -- C ABI of liblce_gfx950.so: fused linear + cross-entropy loss for
+ * AMD MI355X (gfx950), forward and backward.
+ *
+ * The library replaces the device side of the reference operator
+ * (JonasGeiping/linear_cross_entropy_loss).  Citations below are to files of
+ * that repository.
+ *
+ * Conventions
+ *   - All pointers except `lce_problem*` are DEVICE pointers; all work is
+ *     enqueued on `stream` (a hipStream_t passed as void*) and nothing is
+ *     synchronised.  No entry point allocates or frees device memory and the
+ *     library keeps no state between calls: scratch comes in through `ws`.
+ *   - x is (N, H) row-major with row stride ldx; w is the TRANSPOSED weight
+ *     (H, V) row-major with row stride ldw (linear_cross_entropy/ops.py:913);
+ *     y is N contiguous int64 labels (ops.py:210).
+ *   - Supported shapes: N % 512 == 0, H % 256 == 0, V % 4096 == 0,
+ *     n_chunk % 512 == 0 -- the reference's own contract (ops.py:689-691,
+ *     ops.py:905-907).
+ *   - Every function returns LCE_OK (0) or a negative lce_status; nothing
+ *     throws or aborts.
+ */
+#ifndef LCE_H_
+#define LCE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum lce_dtype {
+  LCE_BF16 = 0,
+  LCE_F16 = 1,
+  LCE_F32 = 2
+} lce_dtype;
+
+typedef enum lce_status {
+  LCE_OK = 0,
+  LCE_EINVAL_SHAPE = -1, /* shape outside the supported set (ops.py:43-44, 689-691) */
+  LCE_EINVAL_DTYPE = -2, /* unsupported dtype combination                            */
+  LCE_EINVAL_ARG = -3,   /* null pointer, bad stride, bad scalar                     */
+  LCE_EWORKSPACE = -4,   /* workspace missing or smaller than lce_workspace_bytes    */
+  LCE_EHIP = -5          /* a HIP launch failed; see lce_last_hip_error              */
+} lce_status;
+
+/*
+ * One problem instance.  Mirrors the argument list of
+ * LinearXentImplementation.forward (ops.py:669-679) plus the strides and
+ * dtypes the Triton launches took from the tensors (ops.py:731-734).
+ */
+typedef struct lce_problem {
+  int64_t N;            /* tokens (x flattened to (N, H), ops.py:681)         */
+  int64_t H;            /* in_features                                         */
+  int64_t V;            /* out_features (vocabulary)                           */
+  int64_t ldx;          /* row stride of x, elements                           */
+  int64_t ldw;          /* row stride of w, elements                           */
+  int64_t lddx;         /* row stride of dx, elements (backward only)          */
+  int64_t lddw;         /* row stride of dw, elements (backward only)          */
+  int32_t x_dtype;      /* LCE_BF16 | LCE_F16 | LCE_F32                        */
+  int32_t w_dtype;      /* same as x_dtype, or LCE_F32 (master weight, cast in-kernel) */
+  int32_t dx_dtype;     /* x_dtype or LCE_F32                                  */
+  int32_t dw_dtype;     /* w_dtype or LCE_F32                                  */
+  int64_t ignore_index; /* any int64 (ops.py:674)                              */
+  float logit_scale;    /* > 0 (ops.py:908)                                    */
+  float z_reg;          /* >= 0 (ops.py:909)                                   */
+  int64_t n_chunk;      /* N_chunk_size: scratch bound n_chunk*V*4 bytes (ops.py:677) */
+  int32_t monitoring;   /* 0/1: also produce max / entropy / norm (ops.py:678) */
+  int32_t reserved;
+} lce_problem;
+
+/* Library version: major*10000 + minor*100 + patch. */
+int lce_version(void);
+
+/* Static description of a status code. */
+const char* lce_strerror(int status);
+
+/* Text of the last HIP error seen by this thread ("" if none). */
+const char* lce_last_hip_error(void);
+
+/*
+ * Validates `p` exactly as lce_forward / lce_backward would (no device work).
+ * Replaces the asserts of ops.py:685-691 and the ValueError of ops.py:43-44.
+ */
+int lce_check_problem(const lce_problem* p);
+
+/*
+ * Scratch sizes in bytes for lce_forward and lce_backward on problem `p`.
+ * The backward size never exceeds n_chunk * V * 4 bytes -- the memory bound
+ * the reference documents for N_chunk_size (ops.py:677, 700, 860) -- unless
+ * even the smallest staging unit does not fit, in which case
+ * LCE_EWORKSPACE is returned.
+ */
+int lce_workspace_bytes(const lce_problem* p, size_t* fwd_bytes, size_t* bwd_bytes);
+
+/*
+ * Forward.  Replaces the launch of linear_xent_fwd_prep_bwd_kernel_matmul_t
+ * (ops.py:722-752) and the torch reductions around it (ops.py:705, 753-761,
+ * 793-794, 802), without ever writing logits to memory.
+ *
+ *   lse     out, N floats: logsumexp of the scaled logits of every row
+ *   out5    out, 5 floats: loss, z_reg, logit_max, logit_entropy, logit_norm
+ *           (the 5-tuple of ops.py:802 with the meanings of ops.py:9-17; the
+ *           last three are 0 when monitoring == 0)
+ *   n_valid out, 1 int64: number of labels != ignore_index (ops.py:705)
+ */
+int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_t* y,
+                float* lse, float* out5, int64_t* n_valid,
+                void* ws, size_t ws_bytes, void* stream);
+
+/*
+ * Backward.  Replaces linear_xent_bwd_dispatcher and its dx / dA programs
+ * (ops.py:239-337, 340-456, 544-658, launch at ops.py:763-791) and the
+ * rescaling in LinearXentImplementation.backward (ops.py:804-810).
+ *
+ *   lse, n_valid   as produced by lce_forward on the same inputs
+ *   grad_out       device pointer to 1 float: upstream gradient of the loss
+ *   dx             out, (N, H) in dx_dtype, or NULL to skip
+ *   dw             out, (H, V) in dw_dtype, or NULL to skip
+ *
+ * Gradients are accumulated in fp32 and scaled by grad_out*logit_scale/n_valid
+ * after accumulation (ops.py:332, 443-447).  Rows whose label equals
+ * ignore_index get dx == 0 exactly and contribute exact zeros to dw
+ * (ops.py:314, 422).
+ */
+int lce_backward(const lce_problem* p, const void* x, const void* w, const int64_t* y,
+                 const float* lse, const int64_t* n_valid, const float* grad_out,
+                 void* dx, void* dw, void* ws, size_t ws_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LCE_H_ */

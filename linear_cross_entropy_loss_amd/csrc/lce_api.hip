@@ -1,0 +1,209 @@
+// C ABI of liblce_gfx950.so (declared in include/lce.h): argument checking,
+// scratch planning and the launch sequences.  The host side does what
+// LinearXentImplementation.forward does around its Triton launches
+// (linear_cross_entropy/ops.py:681-802) -- minus every allocation, which is the
+// caller's -- and what its backward does (ops.py:804-810).
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/lce.h"
+#include "lce_internal.h"
+
+namespace {
+
+thread_local char g_hip_error[256] = "";
+
+int hip_fail(hipError_t e, const char* what) {
+  snprintf(g_hip_error, sizeof(g_hip_error), "%s: %s", what, hipGetErrorString(e));
+  return LCE_EHIP;
+}
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+bool is16(int d) { return d == LCE_BF16 || d == LCE_F16; }
+
+int check(const lce_problem* p, bool backward) {
+  if (!p) return LCE_EINVAL_ARG;
+  if (p->N <= 0 || p->H <= 0 || p->V <= 0 || p->n_chunk <= 0) return LCE_EINVAL_SHAPE;
+  if (p->N % 512 || p->H % 256 || p->V % 4096 || p->n_chunk % 512) return LCE_EINVAL_SHAPE;
+  if (p->N > (int64_t)1 << 30 || p->V > (int64_t)1 << 30 || p->H > (int64_t)1 << 20) return LCE_EINVAL_SHAPE;
+  const int xd = p->x_dtype, wd = p->w_dtype;
+  const bool ok = (is16(xd) && (wd == xd || wd == LCE_F32)) || (xd == LCE_F32 && wd == LCE_F32);
+  if (!ok) return LCE_EINVAL_DTYPE;
+  if (!(p->logit_scale > 0.f) || !(p->z_reg >= 0.f)) return LCE_EINVAL_ARG;
+  const int64_t xa = xd == LCE_F32 ? 4 : 8, wa = wd == LCE_F32 ? 4 : 8;  // 16-byte rows
+  if (p->ldx < p->H || p->ldx % xa || p->ldw < p->V || p->ldw % wa) return LCE_EINVAL_ARG;
+  if (backward) {
+    if (p->dx_dtype != xd && p->dx_dtype != LCE_F32) return LCE_EINVAL_DTYPE;
+    if (p->dw_dtype != wd && p->dw_dtype != LCE_F32) return LCE_EINVAL_DTYPE;
+    if (p->lddx < p->H || p->lddx % 4 || p->lddw < p->V || p->lddw % 4) return LCE_EINVAL_ARG;
+  }
+  return LCE_OK;
+}
+
+struct FwdPlan {
+  size_t part_lse, part_max, part_pz, part_sq, tgt, blk, total;
+};
+
+FwdPlan plan_fwd(const lce_problem* p) {
+  FwdPlan f;
+  const size_t part = align_up((size_t)(p->V / lce::kChunkV) * (size_t)p->N * 4);
+  size_t o = 0;
+  f.part_lse = o; o += part;
+  f.part_max = o; if (p->monitoring) o += part;
+  f.part_pz = o; if (p->monitoring) o += part;
+  f.part_sq = o; if (p->monitoring) o += part;
+  f.tgt = o; o += align_up((size_t)p->N * 4);
+  f.blk = o; o += align_up((size_t)(p->N / lce::kMergeRows) * 8 * sizeof(double));
+  f.total = o;
+  return f;
+}
+
+struct BwdPlan {
+  int64_t slabs, vs;
+  size_t dz, dx_acc, total;
+};
+
+// Fewest vocabulary slabs whose staging fits in n_chunk * V * 4 bytes.
+int plan_bwd(const lce_problem* p, BwdPlan* b) {
+  const size_t budget = (size_t)p->n_chunk * (size_t)p->V * 4;
+  for (int64_t s = 1; s <= p->V / 256; ++s) {
+    if (p->V % s) continue;
+    const int64_t vs = p->V / s;
+    if (vs % 256) continue;
+    const size_t dz = align_up((size_t)p->N * (size_t)vs * 2);
+    const size_t acc = s > 1 ? align_up((size_t)p->N * (size_t)p->H * 4) : 0;
+    if (dz + acc <= budget) {
+      b->slabs = s;
+      b->vs = vs;
+      b->dz = 0;
+      b->dx_acc = dz;
+      b->total = dz + acc;
+      return LCE_OK;
+    }
+  }
+  return LCE_EWORKSPACE;
+}
+
+bool misaligned(const void* p) { return ((uintptr_t)p & 15) != 0; }
+
+}  // namespace
+
+extern "C" {
+
+int lce_version(void) { return 100; }
+
+const char* lce_strerror(int status) {
+  switch (status) {
+    case LCE_OK: return "ok";
+    case LCE_EINVAL_SHAPE:
+      return "shape outside the supported set (need N % 512 == 0, H % 256 == 0, V % 4096 == 0, N_chunk_size % 512 == 0)";
+    case LCE_EINVAL_DTYPE:
+      return "unsupported dtype combination (x: bf16/f16/f32; w: x dtype or f32; grads: same dtype or f32)";
+    case LCE_EINVAL_ARG: return "invalid argument (null or misaligned pointer, bad stride, logit_scale <= 0 or z_reg < 0)";
+    case LCE_EWORKSPACE: return "workspace missing or too small for this problem and N_chunk_size";
+    case LCE_EHIP: return "HIP error";
+    default: return "unknown status";
+  }
+}
+
+const char* lce_last_hip_error(void) { return g_hip_error; }
+
+int lce_check_problem(const lce_problem* p) { return check(p, true); }
+
+int lce_workspace_bytes(const lce_problem* p, size_t* fwd_bytes, size_t* bwd_bytes) {
+  int rc = check(p, false);
+  if (rc != LCE_OK) return rc;
+  if (fwd_bytes) *fwd_bytes = plan_fwd(p).total;
+  if (bwd_bytes) {
+    BwdPlan b;
+    rc = plan_bwd(p, &b);
+    if (rc != LCE_OK) return rc;
+    *bwd_bytes = b.total;
+  }
+  return LCE_OK;
+}
+
+int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_t* y, float* lse,
+                float* out5, int64_t* n_valid, void* ws, size_t ws_bytes, void* stream) {
+  int rc = check(p, false);
+  if (rc != LCE_OK) return rc;
+  if (!x || !w || !y || !lse || !out5 || !n_valid) return LCE_EINVAL_ARG;
+  if (misaligned(x) || misaligned(w)) return LCE_EINVAL_ARG;
+  const FwdPlan f = plan_fwd(p);
+  if (!ws || ws_bytes < f.total || misaligned(ws)) return LCE_EWORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  char* base = (char*)ws;
+
+  lce::FwdArgs a;
+  memset(&a, 0, sizeof(a));
+  a.x = x; a.w = w; a.y = y;
+  a.N = p->N; a.H = p->H; a.V = p->V; a.ldx = p->ldx; a.ldw = p->ldw;
+  a.x_dtype = p->x_dtype; a.w_dtype = p->w_dtype;
+  a.ignore_index = p->ignore_index;
+  a.scale = p->logit_scale; a.z_reg = p->z_reg; a.monitoring = p->monitoring ? 1 : 0;
+  a.lse = lse; a.out5 = out5; a.n_valid = n_valid;
+  a.part_lse = (float*)(base + f.part_lse);
+  a.part_max = (float*)(base + f.part_max);
+  a.part_pz = (float*)(base + f.part_pz);
+  a.part_sq = (float*)(base + f.part_sq);
+  a.tgt = (float*)(base + f.tgt);
+  a.blk = (float*)(base + f.blk);
+
+  hipError_t e = lce::launch_fill_f32(a.tgt, a.N, 0.f, s);
+  if (e != hipSuccess) return hip_fail(e, "fill");
+  e = lce::launch_fwd_tiles(a, s);
+  if (e != hipSuccess) return hip_fail(e, "fwd_tiles");
+  e = lce::launch_fwd_reduce(a, s);
+  if (e != hipSuccess) return hip_fail(e, "fwd_reduce");
+  return LCE_OK;
+}
+
+int lce_backward(const lce_problem* p, const void* x, const void* w, const int64_t* y,
+                 const float* lse, const int64_t* n_valid, const float* grad_out, void* dx,
+                 void* dw, void* ws, size_t ws_bytes, void* stream) {
+  int rc = check(p, true);
+  if (rc != LCE_OK) return rc;
+  if (!x || !w || !y || !lse || !n_valid || !grad_out) return LCE_EINVAL_ARG;
+  if (misaligned(x) || misaligned(w) || misaligned(dx) || misaligned(dw)) return LCE_EINVAL_ARG;
+  if (!dx && !dw) return LCE_OK;
+  BwdPlan b;
+  rc = plan_bwd(p, &b);
+  if (rc != LCE_OK) return rc;
+  if (!ws || ws_bytes < b.total || misaligned(ws)) return LCE_EWORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  char* base = (char*)ws;
+
+  lce::BwdArgs a;
+  memset(&a, 0, sizeof(a));
+  a.x = x; a.w = w; a.y = y; a.lse = lse; a.n_valid = n_valid; a.grad_out = grad_out;
+  a.N = p->N; a.H = p->H; a.V = p->V;
+  a.ldx = p->ldx; a.ldw = p->ldw; a.lddx = p->lddx; a.lddw = p->lddw;
+  a.x_dtype = p->x_dtype; a.w_dtype = p->w_dtype; a.dx_dtype = p->dx_dtype; a.dw_dtype = p->dw_dtype;
+  a.ignore_index = p->ignore_index;
+  a.scale = p->logit_scale; a.z_reg = p->z_reg;
+  a.dx = dx; a.dw = dw;
+  a.dz = base + b.dz;
+  a.dx_acc = b.slabs > 1 ? (float*)(base + b.dx_acc) : nullptr;
+  a.vs = b.vs;
+
+  for (int64_t i = 0; i < b.slabs; ++i) {
+    a.v0 = i * b.vs;
+    a.first = i == 0;
+    a.last = i == b.slabs - 1;
+    hipError_t e = lce::launch_bwd_dz(a, s);
+    if (e != hipSuccess) return hip_fail(e, "bwd_dz");
+    if (dx) {
+      e = lce::launch_bwd_dx(a, s);
+      if (e != hipSuccess) return hip_fail(e, "bwd_dx");
+    }
+    if (dw) {
+      e = lce::launch_bwd_dw(a, s);
+      if (e != hipSuccess) return hip_fail(e, "bwd_dw");
+    }
+  }
+  return LCE_OK;
+}
+
+}  // extern "C"

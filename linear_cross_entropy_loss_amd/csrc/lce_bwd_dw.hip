@@ -1,0 +1,76 @@
+// Backward, step 3: dW[h][v] = coef * sum_token x[token][h] * dz[token][v] for
+// the columns of one vocabulary slab (the contraction of
+// linear_cross_entropy/ops.py:424).  K = token, so both operands are read
+// through the LDS transpose path.  Each workgroup owns its dW tile over ALL
+// tokens: the fp32 accumulator never leaves registers, no cross-workgroup
+// reduction exists, and the result is written once in the output dtype after
+// scaling by grad_out * logit_scale / n_valid (ops.py:443-447, 810).
+#include "lce_gemm.h"
+#include "lce_internal.h"
+
+namespace lce {
+
+namespace {
+
+template <class T, class XSrc>
+__global__ __launch_bounds__(kThreads) void bwd_dw_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  typedef typename elem_of<T>::type E;
+  const int tiles_p = (int)(a.vs / kTile), tiles_q = (int)(a.H / kTile);
+  int tp, tq;
+  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
+  const int64_t vl0 = (int64_t)tp * kTile, h0 = (int64_t)tq * kTile;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wp = wave & 1, wq = wave >> 1;
+
+  f32x16_t acc[kNB][kNB];
+  gemm_mainloop<T, E, false, XSrc, false>(
+      acc, reinterpret_cast<const E*>(a.dz) + vl0, a.vs,
+      reinterpret_cast<const XSrc*>(a.x) + h0, a.ldx, (int)(a.N / kBK), lds);
+
+  const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
+#pragma unroll
+  for (int qb = 0; qb < kNB; ++qb) {
+    const int64_t h = h0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+#pragma unroll
+    for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int64_t v = a.v0 + vl0 + wp * kWaveTile + pb * kBlk + 8 * rq + 4 * (lane >> 5);
+        f32x4_t o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = acc[pb][qb][rq * 4 + j] * coef;
+        if (a.dw_dtype == DT_F32) {
+          *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + h * a.lddw + v) = o;
+        } else {
+          u32x2_t b;
+          b[0] = pack2<T>(o[0], o[1]);
+          b[1] = pack2<T>(o[2], o[3]);
+          *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + v) = b;
+        }
+      }
+  }
+}
+
+template <class T, class XSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dw_kernel<T, XSrc>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
+  if (e != hipSuccess) return e;
+  const int grid = (int)((a.vs / kTile) * (a.H / kTile));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s) {
+  typedef elem_of<BF16>::type bf;
+  typedef elem_of<F16>::type hf;
+  if (a.x_dtype == DT_BF16) return launch<BF16, bf>(a, s);
+  if (a.x_dtype == DT_F16) return launch<F16, hf>(a, s);
+  if (a.x_dtype == DT_F32) return launch<BF16, float>(a, s);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace lce

@@ -1,0 +1,79 @@
+// Backward, step 2: dx[token][h] (+)= sum_v dz[token][v] * W[h][v] over one
+// vocabulary slab (the contraction of linear_cross_entropy/ops.py:317).  Both
+// operands are K-contiguous (K = v).  The running sum over slabs is kept in
+// fp32; the factor grad_out * logit_scale / n_valid is applied once, after the
+// last slab, as the reference does after its accumulation (ops.py:332, 810).
+#include "lce_gemm.h"
+#include "lce_internal.h"
+
+namespace lce {
+
+namespace {
+
+template <class T, class WSrc>
+__global__ __launch_bounds__(kThreads) void bwd_dx_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  typedef typename elem_of<T>::type E;
+  const int tiles_p = (int)(a.H / kTile), tiles_q = (int)(a.N / kTile);
+  int tp, tq;
+  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
+  const int64_t h0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wp = wave & 1, wq = wave >> 1;
+
+  f32x16_t acc[kNB][kNB];
+  gemm_mainloop<T, WSrc, true, E, true>(
+      acc, reinterpret_cast<const WSrc*>(a.w) + h0 * a.ldw + a.v0, a.ldw,
+      reinterpret_cast<const E*>(a.dz) + t0 * a.vs, a.vs, (int)(a.vs / kBK), lds);
+
+  const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
+#pragma unroll
+  for (int qb = 0; qb < kNB; ++qb) {
+    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+#pragma unroll
+    for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int64_t h = h0 + wp * kWaveTile + pb * kBlk + 8 * rq + 4 * (lane >> 5);
+        f32x4_t v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = acc[pb][qb][rq * 4 + j];
+        if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + tok * a.H + h);
+        if (!a.last) {
+          *reinterpret_cast<f32x4_t*>(a.dx_acc + tok * a.H + h) = v;
+        } else if (a.dx_dtype == DT_F32) {
+          *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dx) + tok * a.lddx + h) = v * coef;
+        } else {
+          u32x2_t o;
+          o[0] = pack2<T>(v[0] * coef, v[1] * coef);
+          o[1] = pack2<T>(v[2] * coef, v[3] * coef);
+          *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dx) + tok * a.lddx + h) = o;
+        }
+      }
+  }
+}
+
+template <class T, class WSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dx_kernel<T, WSrc>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
+  if (e != hipSuccess) return e;
+  const int grid = (int)((a.H / kTile) * (a.N / kTile));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s) {
+  typedef elem_of<BF16>::type bf;
+  typedef elem_of<F16>::type hf;
+  const bool bf_compute = a.x_dtype == DT_BF16 || a.x_dtype == DT_F32;
+  if (bf_compute && a.w_dtype == DT_BF16) return launch<BF16, bf>(a, s);
+  if (bf_compute && a.w_dtype == DT_F32) return launch<BF16, float>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch<F16, hf>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch<F16, float>(a, s);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace lce

@@ -1,0 +1,263 @@
+// Forward of the fused linear + cross-entropy operator on gfx950.
+//
+// fwd_tiles_kernel computes one 256(v) x 256(token) tile of the scaled logits
+// z = logit_scale * x W with MFMA and reduces it, in registers, to per-token
+// partials over each 128-column slice: logsumexp, and when monitoring is on
+// the slice max, sum softmax*z and sum z^2.  The logit of the target column is
+// written by the one lane that holds it.  No logits reach memory.  (The
+// reference kernel, linear_cross_entropy/ops.py:190-236, computes the same
+// per-tile lse but also stores the fp32 logits, ops.py:216.)
+//
+// fwd_rows_kernel merges the slice partials of each token into its lse and
+// forms the per-token loss terms (ops.py:753-761); fwd_final_kernel sums them
+// in a fixed order into the five scalars of ops.py:802 and the valid-label
+// count of ops.py:705.  All reductions are order-deterministic.
+#include "lce_gemm.h"
+#include "lce_internal.h"
+
+namespace lce {
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+LCE_DEV float fast_exp2(float v) { return __builtin_amdgcn_exp2f(v); }
+LCE_DEV float fast_log(float v) { return __builtin_amdgcn_logf(v) * kLn2; }
+
+template <class T, class XSrc, class WSrc>
+__global__ __launch_bounds__(kThreads) void fwd_tiles_kernel(const FwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int tiles_p = (int)(a.V / kTile), tiles_q = (int)(a.N / kTile);
+  int tp, tq;
+  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
+  const int64_t v0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wp = wave & 1, wq = wave >> 1;
+  const int64_t slice_v0 = v0 + wp * kWaveTile;
+
+  // Column of the target inside this wave's 128-wide slice, or -1.
+  int ycol[kNB];
+#pragma unroll
+  for (int qb = 0; qb < kNB; ++qb) {
+    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+    const int64_t yy = a.y[tok];
+    const int64_t rel = yy - slice_v0;
+    ycol[qb] = (yy != a.ignore_index && rel >= 0 && rel < kWaveTile) ? (int)rel : -1;
+  }
+
+  f32x16_t acc[kNB][kNB];
+  gemm_mainloop<T, WSrc, false, XSrc, true>(
+      acc, reinterpret_cast<const WSrc*>(a.w) + v0, a.ldw,
+      reinterpret_cast<const XSrc*>(a.x) + t0 * a.ldx, a.ldx, (int)(a.H / kBK), lds);
+
+  const float c1 = a.scale * kLog2e;
+  const int64_t slice = slice_v0 / kChunkV;
+#pragma unroll
+  for (int qb = 0; qb < kNB; ++qb) {
+    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+    float m = -INFINITY;
+#pragma unroll
+    for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) m = fmaxf(m, acc[pb][qb][r]);
+    m = fmaxf(m, __shfl_xor(m, 32));
+    m *= a.scale;  // logit_scale > 0, so max commutes with the scaling
+    const float mo = m * kLog2e;
+    float s = 0.f, pz = 0.f, sq = 0.f;
+    if (a.monitoring) {
+#pragma unroll
+      for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = fast_exp2(fmaf(acc[pb][qb][r], c1, -mo));
+          const float z = acc[pb][qb][r] * a.scale;
+          s += e;
+          pz = fmaf(e, z, pz);
+          sq = fmaf(z, z, sq);
+        }
+      pz += __shfl_xor(pz, 32);
+      sq += __shfl_xor(sq, 32);
+    } else {
+#pragma unroll
+      for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s += fast_exp2(fmaf(acc[pb][qb][r], c1, -mo));
+    }
+    s += __shfl_xor(s, 32);
+    if (lane < 32) {
+      const int64_t o = slice * a.N + tok;
+      a.part_lse[o] = m + fast_log(s);
+      if (a.monitoring) {
+        a.part_max[o] = m;
+        a.part_pz[o] = pz / s;
+        a.part_sq[o] = sq;
+      }
+    }
+    const int yl = ycol[qb];
+    if (yl >= 0 && ((yl >> 2) & 1) == (lane >> 5)) {
+      const int want_pb = yl >> 5, want_r = ((yl >> 3) & 3) * 4 + (yl & 3);
+      float zt = 0.f;
+#pragma unroll
+      for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (pb == want_pb && r == want_r) zt = acc[pb][qb][r];
+      a.tgt[tok] = zt * a.scale;
+    }
+  }
+}
+
+// One workgroup = 64 tokens x 4 strided groups of slices.
+__global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
+  __shared__ float sh_m[4][kMergeRows], sh_s[4][kMergeRows], sh_lse[kMergeRows];
+  __shared__ float sh_pz[4][kMergeRows], sh_sq[4][kMergeRows], sh_mx[4][kMergeRows];
+  __shared__ double sh_red[6][kMergeRows];
+  const int r = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int64_t tok = (int64_t)blockIdx.x * kMergeRows + r;
+  const int nslices = (int)(a.V / kChunkV);
+
+  float M = -INFINITY, S = 0.f;
+  for (int c = g; c < nslices; c += 4) {
+    const float l = a.part_lse[(int64_t)c * a.N + tok];
+    const float Mn = fmaxf(M, l);
+    S = S * fast_exp2((M - Mn) * kLog2e) + fast_exp2((l - Mn) * kLog2e);
+    M = Mn;
+  }
+  sh_m[g][r] = M;
+  sh_s[g][r] = S;
+  __syncthreads();
+  if (g == 0) {
+    float Mt = fmaxf(fmaxf(sh_m[0][r], sh_m[1][r]), fmaxf(sh_m[2][r], sh_m[3][r]));
+    float St = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) St += sh_s[i][r] * fast_exp2((sh_m[i][r] - Mt) * kLog2e);
+    const float lse = Mt + fast_log(St);
+    sh_lse[r] = lse;
+    a.lse[tok] = lse;
+  }
+  __syncthreads();
+  const float lse = sh_lse[r];
+  if (a.monitoring) {
+    float pz = 0.f, sq = 0.f, mx = -INFINITY;
+    for (int c = g; c < nslices; c += 4) {
+      const int64_t o = (int64_t)c * a.N + tok;
+      pz = fmaf(a.part_pz[o], fast_exp2((a.part_lse[o] - lse) * kLog2e), pz);
+      sq += a.part_sq[o];
+      mx = fmaxf(mx, a.part_max[o]);
+    }
+    sh_pz[g][r] = pz;
+    sh_sq[g][r] = sq;
+    sh_mx[g][r] = mx;
+  }
+  __syncthreads();
+  if (g == 0) {
+    const bool valid = a.y[tok] != a.ignore_index;
+    const double l = (double)lse;
+    double ent = 0.0, nrm = 0.0, mx = -INFINITY;
+    if (a.monitoring) {
+      const float pz = (sh_pz[0][r] + sh_pz[1][r]) + (sh_pz[2][r] + sh_pz[3][r]);
+      const float sq = (sh_sq[0][r] + sh_sq[1][r]) + (sh_sq[2][r] + sh_sq[3][r]);
+      mx = (double)fmaxf(fmaxf(sh_mx[0][r], sh_mx[1][r]), fmaxf(sh_mx[2][r], sh_mx[3][r]));
+      ent = valid ? (double)(lse - pz) : 0.0;
+      nrm = (double)sqrtf(sq);
+    }
+    sh_red[0][r] = valid ? l - (double)a.tgt[tok] : 0.0;
+    sh_red[1][r] = valid ? l * l : 0.0;
+    sh_red[2][r] = ent;
+    sh_red[3][r] = nrm;
+    sh_red[4][r] = mx;
+    sh_red[5][r] = valid ? 1.0 : 0.0;
+  }
+  __syncthreads();
+  if (threadIdx.x < 6) {
+    const int q = threadIdx.x;
+    double acc = sh_red[q][0];
+    for (int i = 1; i < kMergeRows; ++i) acc = (q == 4) ? fmax(acc, sh_red[q][i]) : acc + sh_red[q][i];
+    reinterpret_cast<double*>(a.blk)[(int64_t)blockIdx.x * 8 + q] = acc;
+  }
+}
+
+__global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
+  __shared__ double sh[6][256];
+  const int nblk = (int)(a.N / kMergeRows);
+  const double* blk = reinterpret_cast<const double*>(a.blk);
+  double v[6] = {0, 0, 0, 0, -INFINITY, 0};
+  for (int b = threadIdx.x; b < nblk; b += 256) {
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+      const double t = blk[(int64_t)b * 8 + q];
+      v[q] = (q == 4) ? fmax(v[q], t) : v[q] + t;
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 6; ++q) sh[q][threadIdx.x] = v[q];
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (threadIdx.x < w) {
+#pragma unroll
+      for (int q = 0; q < 6; ++q) {
+        const double t = sh[q][threadIdx.x + w];
+        sh[q][threadIdx.x] = (q == 4) ? fmax(sh[q][threadIdx.x], t) : sh[q][threadIdx.x] + t;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const double R = sh[5][0];  // 0 valid labels -> 0/0 = NaN, as F.cross_entropy gives
+    const double ce = sh[0][0] / R, zr = sh[1][0] / R;
+    a.out5[0] = (float)(ce + (double)a.z_reg * zr);
+    a.out5[1] = (float)zr;
+    a.out5[2] = a.monitoring ? (float)sh[4][0] : 0.f;
+    a.out5[3] = a.monitoring ? (float)(sh[2][0] / R) : 0.f;
+    a.out5[4] = a.monitoring ? (float)(sh[3][0] / (double)a.N) : 0.f;
+    a.n_valid[0] = (int64_t)R;
+  }
+}
+
+__global__ void fill_f32_kernel(float* p, int64_t n, float v) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = v;
+}
+
+template <class T, class XSrc, class WSrc> hipError_t launch_tiles(const FwdArgs& a, hipStream_t s) {
+  auto kern = fwd_tiles_kernel<T, XSrc, WSrc>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
+  if (e != hipSuccess) return e;
+  const int grid = (int)((a.V / kTile) * (a.N / kTile));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
+  typedef elem_of<BF16>::type bf;
+  typedef elem_of<F16>::type hf;
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_tiles<BF16, bf, bf>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch_tiles<BF16, bf, float>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_tiles<F16, hf, hf>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_tiles<F16, hf, float>(a, s);
+  if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch_tiles<BF16, float, float>(a, s);
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s) {
+  hipLaunchKernelGGL(fwd_rows_kernel, dim3((unsigned)(a.N / kMergeRows)), dim3(256), 0, s, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(fwd_final_kernel, dim3(1), dim3(256), 0, s, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_fill_f32(float* p, int64_t n, float v, hipStream_t s) {
+  if (n <= 0) return hipSuccess;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p, n, v);
+  return hipGetLastError();
+}
+
+}  // namespace lce

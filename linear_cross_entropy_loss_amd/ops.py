@@ -1,0 +1,229 @@
+"""Host side of the fused linear + cross-entropy operator for MI355X.
+
+Mirrors the public interface of the reference's ``linear_cross_entropy/ops.py``:
+
+* ``LinearXentImplementation``  -- ``ops.py:661-810`` (autograd Function, same
+  positional arguments, same 5-tuple, last four outputs non-differentiable)
+* ``linear_cross_entropy``      -- ``ops.py:814-826``
+* ``LinearCrossEntropyLoss``    -- ``ops.py:830-955`` (transposed ``(in, out)``
+  weight, no bias, ``monitoring`` / ``latest_metrics``)
+
+The device work is done by hand-written gfx950 kernels behind the C ABI of
+``liblce_gfx950.so``; torch only supplies device memory and the stream.  Unlike
+the reference, ``forward`` computes only the loss (and saves ``lse``); the
+gradients are computed in ``backward`` by recomputing logit tiles, so backward
+may run any number of times and forward-only use pays no gradient cost.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+
+# Kept for import compatibility with the reference package, which exposes its
+# Triton autotune lists under these names (linear_cross_entropy/__init__.py:1).
+# The gfx950 kernels use one fixed tile configuration; the lists are inert.
+fwd_configs: list = []
+bwd_configs: list = []
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _check_inputs(x, y, At):
+    if not (x.is_cuda and y.is_cuda and At.is_cuda):
+        raise RuntimeError(
+            "linear_cross_entropy needs its tensors on an AMD GPU (device type 'cuda' under ROCm); "
+            "there is no CPU path"
+        )
+    if y.dtype != torch.int64:
+        raise ValueError("labels must be a torch.long tensor")
+    if At.dim() != 2:
+        raise ValueError("weight must be 2-D with shape (in_features, out_features)")
+
+
+class LinearXentImplementation(torch.autograd.Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(
+        ctx,
+        x_in,
+        y,
+        At,
+        ignore_index=-100,
+        z_regularization: float = 0.0,
+        logit_scale: float = 1.0,
+        N_chunk_size: int = 4096,
+        monitoring: bool = True,
+    ):
+        _check_inputs(x_in, y, At)
+        # Under autocast the activations take the autocast dtype; a float32 weight is NOT copied:
+        # the kernels read the fp32 master weight and round it on the way into LDS.
+        if torch.is_autocast_enabled("cuda") and x_in.dtype == torch.float32:
+            x_in = x_in.to(torch.get_autocast_dtype("cuda"))
+        with torch.cuda.device(x_in.device):
+            x = x_in.reshape(-1, x_in.shape[-1])
+            if x.stride(-1) != 1:
+                x = x.contiguous()
+            y1 = y.reshape(-1).contiguous()
+            w = At if At.stride(-1) == 1 else At.contiguous()
+            N, H = x.shape
+            H_A, V = w.shape
+            if H_A != H:
+                raise ValueError(f"weight has in_features={H_A}, input has {H}")
+            if y1.shape != (N,):
+                raise ValueError("labels must have one entry per input row")
+            prob = _lib.make_problem(
+                N, H, V, x.stride(0), w.stride(0), H, V, x.dtype, w.dtype, x.dtype, w.dtype,
+                ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring,
+            )
+            lib = _lib.load()
+            _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")
+            fwd_bytes, _ = _lib.workspace_bytes(prob)
+            dev = x.device
+            ws = torch.empty(fwd_bytes, dtype=torch.uint8, device=dev)
+            lse = torch.empty(N, dtype=torch.float32, device=dev)
+            out5 = torch.empty(5, dtype=torch.float32, device=dev)
+            n_valid = torch.empty(1, dtype=torch.int64, device=dev)
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            rc = lib.lce_forward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(lse), _ptr(out5),
+                                 _ptr(n_valid), _ptr(ws), fwd_bytes, ctypes.c_void_p(stream))
+            _lib.raise_for_status(rc, "lce_forward")
+            del ws
+        ctx.save_for_backward(x, y1, w, lse, n_valid)
+        ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size)
+        ctx.x_shape = x_in.shape
+        loss, z_reg, logit_max, logit_ent, logit_norm = out5.unbind(0)
+        ctx.mark_non_differentiable(z_reg, logit_max, logit_ent, logit_norm)
+        return loss, z_reg, logit_max, logit_ent, logit_norm
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output, void0=None, void1=None, void2=None, void3=None):
+        x, y1, w, lse, n_valid = ctx.saved_tensors
+        ignore_index, z_regularization, logit_scale, N_chunk_size = ctx.lce_cfg
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[2]
+        N, H = x.shape
+        V = w.shape[1]
+        with torch.cuda.device(x.device):
+            dev = x.device
+            dx = torch.empty((N, H), dtype=x.dtype, device=dev) if need_dx else None
+            dw = torch.empty((H, V), dtype=w.dtype, device=dev) if need_dw else None
+            if need_dx or need_dw:
+                prob = _lib.make_problem(
+                    N, H, V, x.stride(0), w.stride(0), H, V, x.dtype, w.dtype, x.dtype, w.dtype,
+                    ignore_index, logit_scale, z_regularization, N_chunk_size, False,
+                )
+                lib = _lib.load()
+                _, bwd_bytes = _lib.workspace_bytes(prob)
+                ws = torch.empty(bwd_bytes, dtype=torch.uint8, device=dev)
+                g = grad_output.detach().to(device=dev, dtype=torch.float32).reshape(1).contiguous()
+                stream = torch.cuda.current_stream(dev).cuda_stream
+                rc = lib.lce_backward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(lse), _ptr(n_valid),
+                                      _ptr(g), _ptr(dx), _ptr(dw), _ptr(ws), bwd_bytes, ctypes.c_void_p(stream))
+                _lib.raise_for_status(rc, "lce_backward")
+                del ws
+        if dx is not None:
+            dx = dx.view(ctx.x_shape)
+        return dx, None, dw, None, None, None, None, None
+
+
+def linear_cross_entropy(
+    x,
+    y,
+    At,
+    ignore_index=-100,
+    z_regularization: float = 0.0,
+    logit_scale: float = 1.0,
+    N_chunk_size: int = 4096,
+    monitoring: bool = False,
+):
+    """Functional form; returns ``(loss, z_reg, logit_max, logit_entropy, logit_norm)``."""
+    return LinearXentImplementation.apply(
+        x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring
+    )
+
+
+class LinearCrossEntropyLoss(torch.nn.Linear):
+    """``loss = cross_entropy(logit_scale * x @ weight, y)`` fused on the GPU.
+
+    An ``nn.Linear`` subclass so that initialisation passes that look for ``nn.Linear`` find it, but the
+    weight is stored transposed, ``(in_features, out_features)``, and there is no bias.
+
+    Args:
+        in_features: hidden size (multiple of 256).
+        out_features: vocabulary size / number of classes (multiple of 4096).
+        ignore_index: label value that is skipped. Default -100.
+        logit_scale: positive factor applied to the logits before the loss. Default 1.0.
+        z_regularization: weight of the ``mean(logsumexp(z)^2)`` penalty. Default 0.0.
+        N_chunk_size: bounds the scratch memory of a call to ``N_chunk_size * out_features * 4`` bytes
+            (multiple of 512; the number of rows of ``x`` must be a multiple of 512). Default 4096.
+        init_method: optional callable applied to the weight instead of the default truncated normal.
+
+    Set ``module.monitoring = True`` to also collect ``logit_norm``, ``logit_max``, ``logit_entropy`` and
+    ``z_value`` into ``module.latest_metrics`` on every forward.
+    """
+
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        device=None,
+        dtype=None,
+        ignore_index: int = -100,
+        logit_scale: float = 1.0,
+        z_regularization: float = 0.0,
+        N_chunk_size: int = 4096,
+        init_method=None,
+    ):
+        factory_kwargs = {"device": device, "dtype": dtype}
+        torch.nn.Module.__init__(self)
+
+        assert in_features % 256 == 0
+        assert out_features % 4096 == 0
+        assert N_chunk_size % 512 == 0
+        assert logit_scale > 0
+        assert z_regularization >= 0
+
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight = torch.nn.Parameter(torch.empty((in_features, out_features), **factory_kwargs))
+
+        self.logit_scale = logit_scale
+        self.ignore_index = ignore_index
+        self.z_regularization = z_regularization
+        self.N_chunk_size = N_chunk_size
+
+        self.monitoring = False
+        self.latest_metrics = {}
+        self.init_method = init_method
+
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        if self.init_method is not None:
+            self.init_method(self.weight)
+        else:
+            std = math.sqrt(1 / self.in_features)
+            torch.nn.init.trunc_normal_(self.weight, mean=0.0, std=std, a=-3 * std, b=3 * std)
+
+    def forward(self, x, y):
+        loss, z_reg, logit_max, logit_ent, logit_norm = LinearXentImplementation.apply(
+            x, y, self.weight, self.ignore_index, self.z_regularization, self.logit_scale,
+            self.N_chunk_size, self.monitoring,
+        )
+        if self.monitoring:
+            self.latest_metrics = {
+                "logit_norm": logit_norm,
+                "logit_max": logit_max,
+                "logit_entropy": logit_ent,
+                "z_value": z_reg,
+            }
+        return loss
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias=False"
