@@ -67,8 +67,22 @@ typedef struct lce_problem {
   float z_reg;          /* >= 0 (ops.py:909)                                   */
   int64_t n_chunk;      /* N_chunk_size: scratch bound n_chunk*V*4 bytes (ops.py:677) */
   int32_t monitoring;   /* 0/1: also produce max / entropy / norm (ops.py:678) */
-  int32_t reserved;
+  int32_t phases;       /* 0 = everything; otherwise a mask of LCE_PHASE_* (profiling aid) */
 } lce_problem;
+
+/*
+ * Profiling aid: a non-zero lce_problem.phases restricts a call to the named
+ * kernels so that each can be bracketed by events.  Results of a restricted
+ * call are only meaningful if the skipped phases ran before on the same
+ * buffers.
+ */
+enum {
+  LCE_PHASE_FWD_TILES = 1,  /* lce_forward: the MFMA tile kernel            */
+  LCE_PHASE_FWD_REDUCE = 2, /* lce_forward: row merge + final reduction     */
+  LCE_PHASE_BWD_DZ = 4,     /* lce_backward: recompute + dz staging         */
+  LCE_PHASE_BWD_DX = 8,     /* lce_backward: dx contraction                 */
+  LCE_PHASE_BWD_DW = 16     /* lce_backward: dW contraction                 */
+};
 
 /* Library version: major*10000 + minor*100 + patch. */
 int lce_version(void);

@@ -151,12 +151,20 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
   a.tgt = (float*)(base + f.tgt);
   a.blk = (float*)(base + f.blk);
 
-  hipError_t e = lce::launch_fill_f32(a.tgt, a.N, 0.f, s);
-  if (e != hipSuccess) return hip_fail(e, "fill");
-  e = lce::launch_fwd_tiles(a, s);
-  if (e != hipSuccess) return hip_fail(e, "fwd_tiles");
-  e = lce::launch_fwd_reduce(a, s);
-  if (e != hipSuccess) return hip_fail(e, "fwd_reduce");
+  const int ph = p->phases ? p->phases : ~0;
+  hipError_t e;
+  if (ph & LCE_PHASE_FWD_TILES) {
+    if (ph & LCE_PHASE_FWD_REDUCE) {  // a tiles-only (profiling) call reuses the zeroed buffer
+      e = lce::launch_fill_f32(a.tgt, a.N, 0.f, s);
+      if (e != hipSuccess) return hip_fail(e, "fill");
+    }
+    e = lce::launch_fwd_tiles(a, s);
+    if (e != hipSuccess) return hip_fail(e, "fwd_tiles");
+  }
+  if (ph & LCE_PHASE_FWD_REDUCE) {
+    e = lce::launch_fwd_reduce(a, s);
+    if (e != hipSuccess) return hip_fail(e, "fwd_reduce");
+  }
   return LCE_OK;
 }
 
@@ -187,18 +195,22 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.dz = base + b.dz;
   a.dx_acc = b.slabs > 1 ? (float*)(base + b.dx_acc) : nullptr;
   a.vs = b.vs;
+  const int ph = p->phases ? p->phases : ~0;
 
   for (int64_t i = 0; i < b.slabs; ++i) {
     a.v0 = i * b.vs;
     a.first = i == 0;
     a.last = i == b.slabs - 1;
-    hipError_t e = lce::launch_bwd_dz(a, s);
-    if (e != hipSuccess) return hip_fail(e, "bwd_dz");
-    if (dx) {
+    hipError_t e;
+    if (ph & LCE_PHASE_BWD_DZ) {
+      e = lce::launch_bwd_dz(a, s);
+      if (e != hipSuccess) return hip_fail(e, "bwd_dz");
+    }
+    if (dx && (ph & LCE_PHASE_BWD_DX)) {
       e = lce::launch_bwd_dx(a, s);
       if (e != hipSuccess) return hip_fail(e, "bwd_dx");
     }
-    if (dw) {
+    if (dw && (ph & LCE_PHASE_BWD_DW)) {
       e = lce::launch_bwd_dw(a, s);
       if (e != hipSuccess) return hip_fail(e, "bwd_dw");
     }

@@ -1,0 +1,167 @@
+"""CPU-side checks: the C-ABI library loads and exports what include/lce.h declares; argument validation and
+scratch planning behave as documented; the Python surface mirrors the reference's.  No compute calls."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from linear_cross_entropy_loss_amd import _lib
+    from linear_cross_entropy_loss_amd.build import build
+
+    build(force=False)
+    return _lib.load()
+
+
+def _prob(**kw):
+    from linear_cross_entropy_loss_amd import _lib
+
+    d = dict(N=512, H=256, V=4096, ldx=256, ldw=4096, lddx=256, lddw=4096, x_dtype=torch.bfloat16,
+             w_dtype=torch.bfloat16, dx_dtype=torch.bfloat16, dw_dtype=torch.bfloat16, ignore_index=-100,
+             logit_scale=1.0, z_reg=0.0, n_chunk=4096, monitoring=False)
+    d.update(kw)
+    return _lib.make_problem(**d)
+
+
+def test_every_declared_symbol_is_exported(lib):
+    from linear_cross_entropy_loss_amd import _lib
+
+    header = open(os.path.join(ROOT, "include", "lce.h")).read()
+    declared = set(re.findall(r"^\s*(?:const\s+char\*|int)\s+(lce_\w+)\s*\(", header, flags=re.M))
+    assert declared == set(_lib.EXPORTS), (declared, _lib.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.lce_version() >= 100
+
+
+def test_struct_layout_matches_header():
+    from linear_cross_entropy_loss_amd import _lib
+
+    header = open(os.path.join(ROOT, "include", "lce.h")).read()
+    body = re.search(r"typedef struct lce_problem \{(.*?)\} lce_problem;", header, flags=re.S).group(1)
+    fields = re.findall(r"^\s*(int64_t|int32_t|float)\s+(\w+);", body, flags=re.M)
+    ctype = {"int64_t": ctypes.c_int64, "int32_t": ctypes.c_int32, "float": ctypes.c_float}
+    assert [(n, ctype[t]) for t, n in fields] == list(_lib.LceProblem._fields_)
+    assert ctypes.sizeof(_lib.LceProblem) == 7 * 8 + 4 * 4 + 8 + 2 * 4 + 8 + 2 * 4
+
+
+def test_shape_contract_is_the_references(lib):
+    from linear_cross_entropy_loss_amd import _lib
+
+    ok = _prob()
+    assert lib.lce_check_problem(ctypes.byref(ok)) == _lib.LCE_OK
+    for bad in (dict(N=500, ldx=256), dict(H=128, ldx=128, lddx=128), dict(V=4000, ldw=4000, lddw=4000),
+                dict(n_chunk=100), dict(N=0)):
+        assert lib.lce_check_problem(ctypes.byref(_prob(**bad))) == _lib.LCE_EINVAL_SHAPE, bad
+    assert lib.lce_check_problem(ctypes.byref(_prob(logit_scale=0.0))) == _lib.LCE_EINVAL_ARG
+    assert lib.lce_check_problem(ctypes.byref(_prob(z_reg=-1.0))) == _lib.LCE_EINVAL_ARG
+    assert lib.lce_check_problem(ctypes.byref(_prob(ldx=250))) == _lib.LCE_EINVAL_ARG
+    assert lib.lce_check_problem(ctypes.byref(_prob(x_dtype=torch.bfloat16, w_dtype=torch.float16))) == _lib.LCE_EINVAL_DTYPE
+    assert lib.lce_check_problem(ctypes.byref(_prob(x_dtype=torch.float32, w_dtype=torch.bfloat16))) == _lib.LCE_EINVAL_DTYPE
+    assert lib.lce_check_problem(ctypes.byref(_prob(w_dtype=torch.float32, dw_dtype=torch.float32))) == _lib.LCE_OK
+    assert lib.lce_check_problem(None) == _lib.LCE_EINVAL_ARG
+
+
+def test_status_maps_to_reference_exceptions(lib):
+    from linear_cross_entropy_loss_amd import _lib
+
+    with pytest.raises(ValueError, match="Provided shape outside the range of valid configs"):
+        _lib.raise_for_status(_lib.LCE_EINVAL_SHAPE, "x")
+    with pytest.raises(ValueError):
+        _lib.raise_for_status(_lib.LCE_EINVAL_DTYPE, "x")
+    with pytest.raises(RuntimeError):
+        _lib.raise_for_status(_lib.LCE_EWORKSPACE, "x")
+    assert b"HIP" in lib.lce_strerror(_lib.LCE_EHIP)
+
+
+@pytest.mark.parametrize("N,H,V,n_chunk", [(16384, 2048, 131072, 4096), (16384, 4096, 131072, 4096),
+                                           (16384, 2048, 262144, 2048), (16384, 2048, 32768, 8192),
+                                           (65536, 8192, 262144, 8192), (512, 256, 4096, 512)])
+def test_backward_scratch_within_n_chunk_bound(N, H, V, n_chunk):
+    from linear_cross_entropy_loss_amd import _lib
+
+    p = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=n_chunk)
+    fwd, bwd = _lib.workspace_bytes(p)
+    assert bwd <= n_chunk * V * 4
+    assert fwd >= (V // 128) * N * 4
+
+
+def test_null_and_small_workspace_are_rejected_without_touching_the_gpu(lib):
+    from linear_cross_entropy_loss_amd import _lib
+
+    p = _prob()
+    one = ctypes.c_void_p(256)  # never dereferenced: validation fails first
+    rc = lib.lce_forward(ctypes.byref(p), one, one, one, one, one, one, None, 0, None)
+    assert rc == _lib.LCE_EWORKSPACE
+    rc = lib.lce_forward(ctypes.byref(p), None, one, one, one, one, one, one, 1 << 30, None)
+    assert rc == _lib.LCE_EINVAL_ARG
+    rc = lib.lce_backward(ctypes.byref(p), one, one, one, one, one, one, one, one, one, 16, None)
+    assert rc == _lib.LCE_EWORKSPACE
+    rc = lib.lce_backward(ctypes.byref(p), one, one, one, one, one, one, ctypes.c_void_p(260), one, one, 1 << 40, None)
+    assert rc == _lib.LCE_EINVAL_ARG  # misaligned dx
+
+
+def test_python_surface_mirrors_reference():
+    import linear_cross_entropy_loss_amd as pkg
+
+    assert pkg.fwd_configs == [] and pkg.bwd_configs == []
+    sig = inspect.signature(pkg.linear_cross_entropy)
+    assert list(sig.parameters) == ["x", "y", "At", "ignore_index", "z_regularization", "logit_scale",
+                                    "N_chunk_size", "monitoring"]
+    assert sig.parameters["ignore_index"].default == -100
+    assert sig.parameters["N_chunk_size"].default == 4096 and sig.parameters["monitoring"].default is False
+    msig = inspect.signature(pkg.LinearCrossEntropyLoss.__init__)
+    assert list(msig.parameters)[1:] == ["in_features", "out_features", "device", "dtype", "ignore_index",
+                                         "logit_scale", "z_regularization", "N_chunk_size", "init_method"]
+
+
+def test_module_contract_on_cpu():
+    from linear_cross_entropy_loss_amd import LinearCrossEntropyLoss
+
+    m = LinearCrossEntropyLoss(256, 4096)
+    assert isinstance(m, torch.nn.Linear)
+    assert tuple(m.weight.shape) == (256, 4096)          # transposed weight
+    assert not hasattr(m, "bias") or m.bias is None or "bias" not in dict(m.named_parameters())
+    assert list(dict(m.named_parameters())) == ["weight"]
+    assert m.ignore_index == -100 and m.monitoring is False and m.latest_metrics == {}
+    std = (1 / 256) ** 0.5
+    assert m.weight.abs().max() <= 3 * std + 1e-6 and abs(m.weight.std().item() - std) < 0.1 * std
+    assert "bias=False" in repr(m)
+    called = []
+    LinearCrossEntropyLoss(256, 4096, init_method=lambda w: (called.append(1), w.data.zero_()))
+    assert called
+    for bad in (dict(in_features=100, out_features=4096), dict(in_features=256, out_features=1000)):
+        with pytest.raises(AssertionError):
+            LinearCrossEntropyLoss(**bad)
+    with pytest.raises(AssertionError):
+        LinearCrossEntropyLoss(256, 4096, N_chunk_size=100)
+    with pytest.raises(AssertionError):
+        LinearCrossEntropyLoss(256, 4096, logit_scale=0.0)
+    sd = m.state_dict()
+    assert list(sd) == ["weight"]
+
+
+def test_cpu_tensors_fail_loudly():
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    x = torch.randn(512, 256)
+    w = torch.randn(256, 4096)
+    y = torch.randint(0, 4096, (512,))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        linear_cross_entropy(x, y, w)
+
+
+def test_product_does_not_import_the_oracle():
+    pkg_dir = os.path.join(ROOT, "linear_cross_entropy_loss_amd")
+    for dirpath, _, files in os.walk(pkg_dir):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, os.path.join(dirpath, f)

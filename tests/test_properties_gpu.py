@@ -1,0 +1,237 @@
+"""GPU tests of masking, determinism, API behaviour and full-size properties of the HIP path."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from helpers import make_inputs, rel_errors
+
+pytestmark = pytest.mark.gpu
+
+
+def _fb(x, y, w, ignore_index=-1, z_reg=0.0, scale=1.0, n_chunk=512, mon=False, g=1.0):
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    xd = x.detach().clone().requires_grad_(True)
+    wd = w.detach().clone().requires_grad_(True)
+    out = linear_cross_entropy(xd, y, wd, ignore_index, z_reg, scale, n_chunk, mon)
+    (out[0] * g).backward()
+    torch.cuda.synchronize()
+    return out, xd.grad, wd.grad
+
+
+def test_masking_is_bit_exact_under_garbage_in_ignored_rows():
+    print("masking bit-exact", flush=True)
+    x, y, w = make_inputs(1024, 256, 8192, torch.bfloat16, seed=21, ignore_frac=0.3, device="cuda")
+    out_a, dx_a, dw_a = _fb(x, y, w, z_reg=1e-3)
+    xg = x.clone()
+    xg[y == -1] = 3.0e4  # finite garbage
+    out_b, dx_b, dw_b = _fb(xg, y, w, z_reg=1e-3)
+    assert torch.equal(out_a[0], out_b[0]) and torch.equal(out_a[1], out_b[1])
+    assert torch.equal(dx_a, dx_b)
+    assert torch.equal(dw_a, dw_b)
+    assert (dx_a[y == -1].view(torch.int16) == 0).all()  # +0.0 bit pattern
+
+
+def test_valid_count_is_exact_and_nonnegative_ignore_index_is_honoured():
+    from linear_cross_entropy_loss_amd import _lib
+
+    print("n_valid exact", flush=True)
+    N, H, V = 2048, 256, 4096
+    x, y, w = make_inputs(N, H, V, torch.float16, seed=22, ignore_frac=0.0, device="cuda")
+    y[::3] = 7  # ignore_index = 7 is a legal column: those rows are ignored, never matched
+    lib = _lib.load()
+    p = _lib.make_problem(N, H, V, H, V, H, V, x.dtype, w.dtype, x.dtype, w.dtype, 7, 1.0, 0.0, 512, False)
+    fwd_b, _ = _lib.workspace_bytes(p)
+    ws = torch.empty(fwd_b, dtype=torch.uint8, device="cuda")
+    lse = torch.empty(N, device="cuda")
+    out5 = torch.empty(5, device="cuda")
+    nv = torch.zeros(1, dtype=torch.int64, device="cuda")
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = lib.lce_forward(ctypes.byref(p), P(x), P(w), P(y), P(lse), P(out5), P(nv), P(ws), fwd_b,
+                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert nv.item() == int((y != 7).sum().item())
+    from oracle import lce_forward_fp64
+
+    ref = lce_forward_fp64(x.cpu().double(), y.cpu(), w.cpu().double(), 7, 0.0, 1.0)
+    assert abs(out5[0].item() - ref.loss.item()) <= 1e-3 * abs(ref.loss.item())
+    assert torch.allclose(lse.cpu().double(), ref.lse, rtol=2e-4, atol=2e-4)
+    _, dx, _ = _fb(x, y, w, ignore_index=7)
+    assert (dx[y == 7] == 0).all()
+
+
+def test_all_labels_ignored_gives_nan_loss():
+    print("all ignored", flush=True)
+    x, y, w = make_inputs(512, 256, 4096, torch.bfloat16, seed=23, device="cuda")
+    y[:] = -1
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    out = linear_cross_entropy(x, y, w, -1)
+    assert math.isnan(out[0].item())
+
+
+def test_runs_are_deterministic_and_backward_can_repeat():
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    print("determinism", flush=True)
+    x, y, w = make_inputs(1024, 512, 8192, torch.bfloat16, seed=24, ignore_frac=0.1, device="cuda")
+    a = _fb(x, y, w, z_reg=1e-4, scale=0.5, mon=True)
+    b = _fb(x, y, w, z_reg=1e-4, scale=0.5, mon=True)
+    for t, u in zip(a[0], b[0]):
+        assert torch.equal(t, u)
+    assert torch.equal(a[1], b[1]) and torch.equal(a[2], b[2])
+    # backward twice on one graph: each call recomputes, nothing is scaled in place
+    xd = x.clone().requires_grad_(True)
+    wd = w.clone().requires_grad_(True)
+    loss = linear_cross_entropy(xd, y, wd, -1, 1e-4, 0.5, 512, False)[0]
+    g1 = torch.autograd.grad(loss, (xd, wd), retain_graph=True)
+    g2 = torch.autograd.grad(loss, (xd, wd))
+    assert torch.equal(g1[0], g2[0]) and torch.equal(g1[1], g2[1])
+    assert torch.equal(g1[0], a[1])
+
+
+def test_upstream_gradient_scales_linearly():
+    print("grad_output linearity", flush=True)
+    # bf16 on purpose: gradients of order 1/N are subnormal in fp16, where scaling by 4 is not exact
+    x, y, w = make_inputs(512, 256, 4096, torch.bfloat16, seed=25, ignore_frac=0.1, device="cuda")
+    _, dx1, dw1 = _fb(x, y, w, g=1.0)
+    _, dx2, dw2 = _fb(x, y, w, g=4.0)  # power of two: exact scaling
+    assert torch.equal(dx2, dx1 * 4) and torch.equal(dw2, dw1 * 4)
+
+
+def test_n_chunk_size_only_changes_scratch_not_results():
+    print("chunk invariance", flush=True)
+    x, y, w = make_inputs(2048, 256, 16384, torch.bfloat16, seed=26, ignore_frac=0.1, device="cuda")
+    ref = _fb(x, y, w, n_chunk=4096)
+    for nc in (512, 1024):
+        got = _fb(x, y, w, n_chunk=nc)
+        assert torch.equal(got[0][0], ref[0][0])
+        # dx is summed over vocabulary slabs in fp32, so a different slab count may move the last bit
+        assert rel_errors(got[1], ref[1])[0] < 1e-2
+        assert torch.equal(got[2], ref[2])  # dW never depends on the slab split
+
+
+def test_module_api_3d_input_monitoring_and_no_grad():
+    from linear_cross_entropy_loss_amd import LinearCrossEntropyLoss
+    from oracle import lce_forward_fp64
+
+    print("module api", flush=True)
+    torch.manual_seed(3)
+    m = LinearCrossEntropyLoss(256, 4096, device="cuda", dtype=torch.float16, ignore_index=-1, logit_scale=0.5,
+                               z_regularization=1e-4, N_chunk_size=512)
+    x = torch.randn(4, 128, 256, device="cuda", dtype=torch.float16, requires_grad=True)
+    y = torch.randint(0, 4096, (4, 128), device="cuda")
+    y[0, :10] = -1
+    loss = m(x, y)
+    assert m.latest_metrics == {}
+    assert loss.dtype == torch.float32 and loss.dim() == 0
+    loss.backward()
+    assert x.grad.shape == x.shape and m.weight.grad.shape == m.weight.shape
+    assert x.grad.dtype == torch.float16 and m.weight.grad.dtype == torch.float16
+    m.monitoring = True
+    with torch.no_grad():
+        loss2 = m(x, y)
+    assert torch.equal(loss2, loss.detach())
+    assert set(m.latest_metrics) == {"logit_norm", "logit_max", "logit_entropy", "z_value"}
+    ref = lce_forward_fp64(x.detach().cpu().double(), y.cpu(), m.weight.detach().cpu().double(), -1, 1e-4, 0.5)
+    assert abs(m.latest_metrics["logit_max"].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item())
+    assert abs(m.latest_metrics["logit_entropy"].item() - ref.logit_entropy.item()) <= 2e-3 * ref.logit_entropy.item()
+    assert abs(m.latest_metrics["logit_norm"].item() - ref.logit_norm.item()) <= 2e-3 * ref.logit_norm.item()
+    assert abs(m.latest_metrics["z_value"].item() - ref.z_reg.item()) <= 1e-3 * ref.z_reg.item()
+    # only dx wanted: weight frozen
+    m.weight.requires_grad_(False)
+    x.grad = None
+    m(x, y).backward()
+    assert x.grad is not None
+
+
+def test_shape_errors_raise_value_error():
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    print("shape errors", flush=True)
+    x = torch.randn(500, 256, device="cuda", dtype=torch.bfloat16)
+    w = torch.randn(256, 4096, device="cuda", dtype=torch.bfloat16)
+    y = torch.randint(0, 4096, (500,), device="cuda")
+    with pytest.raises(ValueError, match="Provided shape outside the range of valid configs"):
+        linear_cross_entropy(x, y, w)
+    with pytest.raises(ValueError):
+        linear_cross_entropy(torch.randn(512, 256, device="cuda", dtype=torch.bfloat16), y[:12], w)
+
+
+def test_autocast_keeps_fp32_master_weight_and_returns_fp32_dw():
+    from linear_cross_entropy_loss_amd import LinearCrossEntropyLoss
+    from oracle import lce_forward_backward_fp64
+
+    print("autocast / fp32 master weight", flush=True)
+    torch.manual_seed(4)
+    m = LinearCrossEntropyLoss(256, 4096, device="cuda", ignore_index=-1, N_chunk_size=512)  # fp32 parameter
+    x = torch.randn(512, 256, device="cuda", requires_grad=True)
+    y = torch.randint(0, 4096, (512,), device="cuda")
+    with torch.autocast("cuda", dtype=torch.float16):
+        loss = m(x, y)
+    loss.backward()
+    assert m.weight.grad.dtype == torch.float32 and x.grad.dtype == torch.float32
+    ref = lce_forward_backward_fp64(x.detach().cpu().double(), y.cpu(), m.weight.detach().cpu().double(), -1)
+    assert abs(loss.item() - ref.loss.item()) <= 1e-3 * ref.loss.item()
+    assert rel_errors(m.weight.grad, ref.dw)[1] <= 2e-2 and rel_errors(x.grad, ref.dx)[1] <= 2e-2
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Full benchmark shape (N=16384, H=2048, V=131072, bf16): size-independent properties plus the fp64 oracle
+# evaluated on the GPU in row chunks.
+# ---------------------------------------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def big():
+    N, H, V = 16384, 2048, 131072
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn(N, H, device="cuda", generator=g).to(torch.bfloat16)
+    std = 1 / math.sqrt(H)
+    w = torch.empty(H, V, device="cuda")
+    torch.nn.init.trunc_normal_(w, std=std, a=-3 * std, b=3 * std, generator=g)
+    w = w.to(torch.bfloat16)
+    y = torch.randint(0, V, (N,), device="cuda", generator=g)
+    y[torch.rand(N, device="cuda", generator=g) < 0.05] = -1
+    return x, y, w
+
+
+def test_full_size_matches_fp64_oracle_on_gpu(big):
+    from oracle import lce_forward_backward_fp64
+
+    print("full size vs fp64 oracle (GPU-evaluated)", flush=True)
+    x, y, w = big
+    out, dx, dw = _fb(x, y, w, n_chunk=4096)
+    ref = lce_forward_backward_fp64(x, y, w, -1, 0.0, 1.0, chunk=512)
+    assert abs(out[0].item() - ref.loss.item()) <= 1e-3 * ref.loss.item()
+    assert abs(out[0].item() - (math.log(131072) + 0.5)) < 0.05  # logits ~ N(0,1): loss ~ log V + 1/2
+    for name, got, want in (("dx", dx, ref.dx), ("dw", dw, ref.dw)):
+        d = got.double() - want
+        emax = (d.abs().max() / want.abs().max()).item()
+        el2 = (d.norm() / want.norm()).item()
+        print(f"  {name}: max-rel {emax:.3e} l2-rel {el2:.3e}", flush=True)
+        assert emax <= 2e-2 and el2 <= 2e-2
+    assert (dx[y == -1] == 0).all()
+    del ref
+    torch.cuda.empty_cache()
+
+
+def test_full_size_properties(big):
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    print("full size properties", flush=True)
+    x, y, w = big
+    V = w.shape[1]
+    # zero weight: every lse is exactly log V, loss = log V
+    out = linear_cross_entropy(x, y, torch.zeros_like(w), -1, 0.0, 1.0, 4096, True)
+    assert abs(out[0].item() - math.log(V)) < 1e-5
+    assert abs(out[3].item() - math.log(V)) < 1e-4 and out[2].item() == 0 and out[4].item() == 0
+    # zero input: dW = 0 exactly
+    _, dx0, dw0 = _fb(torch.zeros_like(x), y, w, n_chunk=4096)
+    assert (dw0 == 0).all()
+    # row-sum invariant (z_reg = 0): sum_v dW[h, v] = 0 up to rounding of the stored 16-bit entries
+    _, dx, dw = _fb(x, y, w, n_chunk=4096)
+    s = dw.float().sum(1).abs().max().item()
+    a = dw.float().abs().sum(1).max().item()
+    assert s <= 2e-3 * a, (s, a)
