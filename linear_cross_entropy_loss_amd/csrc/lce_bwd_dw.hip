@@ -5,7 +5,7 @@
 // tokens: the fp32 accumulator never leaves registers, no cross-workgroup
 // reduction exists, and the result is written once in the output dtype after
 // scaling by grad_out * logit_scale / n_valid (ops.py:443-447, 810).
-#include "lce_gemm.h"
+#include "lce_gemm2.h"
 #include "lce_internal.h"
 
 namespace lce {
@@ -24,7 +24,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dw_kernel(const BwdArgs a) {
   const int wp = wave & 1, wq = wave >> 1;
 
   f32x16_t acc[kNB][kNB];
-  gemm_mainloop<T, E, false, XSrc, false>(
+  gemm_tile<T, E, false, XSrc, false>(
       acc, reinterpret_cast<const E*>(a.dz) + vl0, a.vs,
       reinterpret_cast<const XSrc*>(a.x) + h0, a.ldx, (int)(a.N / kBK), lds);
 

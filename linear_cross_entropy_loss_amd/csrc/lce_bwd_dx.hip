@@ -3,7 +3,7 @@
 // operands are K-contiguous (K = v).  The running sum over slabs is kept in
 // fp32; the factor grad_out * logit_scale / n_valid is applied once, after the
 // last slab, as the reference does after its accumulation (ops.py:332, 810).
-#include "lce_gemm.h"
+#include "lce_gemm2.h"
 #include "lce_internal.h"
 
 namespace lce {
@@ -22,7 +22,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dx_kernel(const BwdArgs a) {
   const int wp = wave & 1, wq = wave >> 1;
 
   f32x16_t acc[kNB][kNB];
-  gemm_mainloop<T, WSrc, true, E, true>(
+  gemm_tile<T, WSrc, true, E, true>(
       acc, reinterpret_cast<const WSrc*>(a.w) + h0 * a.ldw + a.v0, a.ldw,
       reinterpret_cast<const E*>(a.dz) + t0 * a.vs, a.vs, (int)(a.vs / kBK), lds);
 

@@ -7,7 +7,7 @@
 // products (ops.py:314, 422).  The tile is transposed through LDS and written
 // to the row-major staging buffer dz[N][vs] of the current vocabulary slab
 // with 16-byte stores.
-#include "lce_gemm.h"
+#include "lce_gemm2.h"
 #include "lce_internal.h"
 
 namespace lce {
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dz_kernel(const BwdArgs a) {
   }
 
   f32x16_t acc[kNB][kNB];
-  gemm_mainloop<T, WSrc, false, XSrc, true>(
+  gemm_tile<T, WSrc, false, XSrc, true>(
       acc, reinterpret_cast<const WSrc*>(a.w) + v0, a.ldw,
       reinterpret_cast<const XSrc*>(a.x) + t0 * a.ldx, a.ldx, (int)(a.H / kBK), lds);
 

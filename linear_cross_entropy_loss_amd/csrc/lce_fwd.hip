@@ -12,7 +12,7 @@
 // forms the per-token loss terms (ops.py:753-761); fwd_final_kernel sums them
 // in a fixed order into the five scalars of ops.py:802 and the valid-label
 // count of ops.py:705.  All reductions are order-deterministic.
-#include "lce_gemm.h"
+#include "lce_gemm2.h"
 #include "lce_internal.h"
 
 namespace lce {
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(kThreads) void fwd_tiles_kernel(const FwdArgs a) {
   }
 
   f32x16_t acc[kNB][kNB];
-  gemm_mainloop<T, WSrc, false, XSrc, true>(
+  gemm_tile<T, WSrc, false, XSrc, true>(
       acc, reinterpret_cast<const WSrc*>(a.w) + v0, a.ldw,
       reinterpret_cast<const XSrc*>(a.x) + t0 * a.ldx, a.ldx, (int)(a.H / kBK), lds);
 
