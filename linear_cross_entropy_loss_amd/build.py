@@ -37,7 +37,8 @@ def _hipcc() -> str:
 
 def _compile(src: str, objdir: Path) -> Path:
     obj = objdir / (src + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+    extra = os.environ.get("LCE_EXTRA_HIPCC_FLAGS", "").split()
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{r.stderr}")

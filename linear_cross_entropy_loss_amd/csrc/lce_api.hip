@@ -88,6 +88,16 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
 
 bool misaligned(const void* p) { return ((uintptr_t)p & 15) != 0; }
 
+// Compute units of the current device (grid size of the persistent kernels).
+int current_num_cus(int* out) {
+  int dev = 0, n = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return hip_fail(e, "device query");
+  *out = n > 0 ? n : 1;
+  return LCE_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -150,6 +160,8 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
   a.part_sq = (float*)(base + f.part_sq);
   a.tgt = (float*)(base + f.tgt);
   a.blk = (float*)(base + f.blk);
+  rc = current_num_cus(&a.num_cus);
+  if (rc != LCE_OK) return rc;
 
   const int ph = p->phases ? p->phases : ~0;
   hipError_t e;
@@ -195,6 +207,8 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.dz = base + b.dz;
   a.dx_acc = b.slabs > 1 ? (float*)(base + b.dx_acc) : nullptr;
   a.vs = b.vs;
+  rc = current_num_cus(&a.num_cus);
+  if (rc != LCE_OK) return rc;
   const int ph = p->phases ? p->phases : ~0;
 
   for (int64_t i = 0; i < b.slabs; ++i) {

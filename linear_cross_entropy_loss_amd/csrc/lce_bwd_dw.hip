@@ -5,29 +5,20 @@
 // tokens: the fp32 accumulator never leaves registers, no cross-workgroup
 // reduction exists, and the result is written once in the output dtype after
 // scaling by grad_out * logit_scale / n_valid (ops.py:443-447, 810).
-#include "lce_gemm2.h"
+#include "lce_gemm3.h"
 #include "lce_internal.h"
 
 namespace lce {
 
 namespace {
 
-template <class T, class XSrc>
-__global__ __launch_bounds__(kThreads) void bwd_dw_kernel(const BwdArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
+template <class T>
+LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   typedef typename elem_of<T>::type E;
-  const int tiles_p = (int)(a.vs / kTile), tiles_q = (int)(a.H / kTile);
-  int tp, tq;
-  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
   const int64_t vl0 = (int64_t)tp * kTile, h0 = (int64_t)tq * kTile;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
-
-  f32x16_t acc[kNB][kNB];
-  gemm_tile<T, E, false, XSrc, false>(
-      acc, reinterpret_cast<const E*>(a.dz) + vl0, a.vs,
-      reinterpret_cast<const XSrc*>(a.x) + h0, a.ldx, (int)(a.N / kBK), lds);
-
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
@@ -52,6 +43,47 @@ __global__ __launch_bounds__(kThreads) void bwd_dw_kernel(const BwdArgs a) {
   }
 }
 
+template <class T> struct DwProblem {
+  typedef typename elem_of<T>::type E;
+  const BwdArgs& a;
+  int tiles_p, tiles_q;
+  LCE_DEV DwProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.H / kTile)) {}
+  LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
+  LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
+    int tp, tq;
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    p = reinterpret_cast<const E*>(a.dz) + (int64_t)tp * kTile;
+    q = reinterpret_cast<const E*>(a.x) + (int64_t)tq * kTile;
+  }
+  LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
+    int tp, tq;
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    dw_epilogue<T>(a, acc, tp, tq);
+  }
+};
+
+template <class T>
+__global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  DwProblem<T> prob(a);
+  Pipe3<T, false, false, DwProblem<T>> pipe(prob);
+  pipe.run(a.vs, a.ldx, (int)(a.N / kBK), lds);
+}
+
+template <class T, class XSrc>
+__global__ __launch_bounds__(kThreads) void bwd_dw_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  typedef typename elem_of<T>::type E;
+  const int tiles_p = (int)(a.vs / kTile), tiles_q = (int)(a.H / kTile);
+  int tp, tq;
+  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
+  f32x16_t acc[kNB][kNB];
+  gemm_mainloop<T, E, false, XSrc, false>(
+      acc, reinterpret_cast<const E*>(a.dz) + (int64_t)tp * kTile, a.vs,
+      reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile, a.ldx, (int)(a.N / kBK), lds);
+  dw_epilogue<T>(a, acc, tp, tq);
+}
+
 template <class T, class XSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
   auto kern = bwd_dw_kernel<T, XSrc>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -62,13 +94,24 @@ template <class T, class XSrc> hipError_t launch(const BwdArgs& a, hipStream_t s
   return hipGetLastError();
 }
 
+template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dw_persistent_kernel<T>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
+  if (e != hipSuccess) return e;
+  const int64_t tiles = (a.vs / kTile) * (a.H / kTile);
+  const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16) return launch<BF16, bf>(a, s);
-  if (a.x_dtype == DT_F16) return launch<F16, hf>(a, s);
+  if (a.x_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
+  if (a.x_dtype == DT_F16) return launch_persistent<F16>(a, s);
   if (a.x_dtype == DT_F32) return launch<BF16, float>(a, s);
   return hipErrorInvalidValue;
 }

@@ -3,29 +3,20 @@
 // operands are K-contiguous (K = v).  The running sum over slabs is kept in
 // fp32; the factor grad_out * logit_scale / n_valid is applied once, after the
 // last slab, as the reference does after its accumulation (ops.py:332, 810).
-#include "lce_gemm2.h"
+#include "lce_gemm3.h"
 #include "lce_internal.h"
 
 namespace lce {
 
 namespace {
 
-template <class T, class WSrc>
-__global__ __launch_bounds__(kThreads) void bwd_dx_kernel(const BwdArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
+template <class T>
+LCE_DEV void dx_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   typedef typename elem_of<T>::type E;
-  const int tiles_p = (int)(a.H / kTile), tiles_q = (int)(a.N / kTile);
-  int tp, tq;
-  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
   const int64_t h0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
-
-  f32x16_t acc[kNB][kNB];
-  gemm_tile<T, WSrc, true, E, true>(
-      acc, reinterpret_cast<const WSrc*>(a.w) + h0 * a.ldw + a.v0, a.ldw,
-      reinterpret_cast<const E*>(a.dz) + t0 * a.vs, a.vs, (int)(a.vs / kBK), lds);
-
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
@@ -53,6 +44,47 @@ __global__ __launch_bounds__(kThreads) void bwd_dx_kernel(const BwdArgs a) {
   }
 }
 
+template <class T> struct DxProblem {
+  typedef typename elem_of<T>::type E;
+  const BwdArgs& a;
+  int tiles_p, tiles_q;
+  LCE_DEV DxProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.H / kTile)), tiles_q((int)(a_.N / kTile)) {}
+  LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
+  LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
+    int tp, tq;
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    p = reinterpret_cast<const E*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0;
+    q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs;
+  }
+  LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
+    int tp, tq;
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    dx_epilogue<T>(a, acc, tp, tq);
+  }
+};
+
+template <class T>
+__global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  DxProblem<T> prob(a);
+  Pipe3<T, true, true, DxProblem<T>> pipe(prob);
+  pipe.run(a.ldw, a.vs, (int)(a.vs / kBK), lds);
+}
+
+template <class T, class WSrc>
+__global__ __launch_bounds__(kThreads) void bwd_dx_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  typedef typename elem_of<T>::type E;
+  const int tiles_p = (int)(a.H / kTile), tiles_q = (int)(a.N / kTile);
+  int tp, tq;
+  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
+  f32x16_t acc[kNB][kNB];
+  gemm_mainloop<T, WSrc, true, E, true>(
+      acc, reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0, a.ldw,
+      reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs, a.vs, (int)(a.vs / kBK), lds);
+  dx_epilogue<T>(a, acc, tp, tq);
+}
+
 template <class T, class WSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
   auto kern = bwd_dx_kernel<T, WSrc>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -63,15 +95,26 @@ template <class T, class WSrc> hipError_t launch(const BwdArgs& a, hipStream_t s
   return hipGetLastError();
 }
 
+template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dx_persistent_kernel<T>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
+  if (e != hipSuccess) return e;
+  const int64_t tiles = (a.H / kTile) * (a.N / kTile);
+  const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
   const bool bf_compute = a.x_dtype == DT_BF16 || a.x_dtype == DT_F32;
-  if (bf_compute && a.w_dtype == DT_BF16) return launch<BF16, bf>(a, s);
+  if (bf_compute && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
   if (bf_compute && a.w_dtype == DT_F32) return launch<BF16, float>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch<F16, hf>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch<F16, float>(a, s);
   return hipErrorInvalidValue;
 }

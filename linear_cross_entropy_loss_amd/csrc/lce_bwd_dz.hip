@@ -6,8 +6,10 @@
 // 16-bit compute type exactly where the reference casts dz before its dot
 // products (ops.py:314, 422).  The tile is transposed through LDS and written
 // to the row-major staging buffer dz[N][vs] of the current vocabulary slab
-// with 16-byte stores.
-#include "lce_gemm2.h"
+// with 16-byte stores.  With 16-bit operands the kernel is persistent (one
+// workgroup per CU, operand stream pipelined across tiles); with an fp32
+// weight it runs one tile per workgroup and converts on the way into LDS.
+#include "lce_gemm3.h"
 #include "lce_internal.h"
 
 namespace lce {
@@ -15,9 +17,135 @@ namespace lce {
 namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr int kDzRowBytes = kTile * 2 + 16;          // padded LDS row of the dz tile
-constexpr int kDzLds = kTile * kDzRowBytes;          // 135168 bytes
-static_assert(kDzLds >= kMainloopLds, "dz tile reuses the main-loop LDS");
+constexpr int kDzRowBytes = 64 * 2 + 16;             // padded LDS row of one 64-column pass
+constexpr int kLdsBytes = 160 * 1024;                // two main-loop stages + 32 KiB
+static_assert(4 * kWaveTile * kDzRowBytes <= kLdsBytes - kStageBytes, "four wave slices must fit beside one stage");
+
+// Turns the finished logit tile (tp, tq) into dz and writes it out.
+//
+// Each lane owns 4 tokens (columns of the accumulator) x 64 vocabulary entries
+// per token, four consecutive entries per register quad.  A wave stages its own
+// 128(token) x 128(v) sub-tile through a private slice of `scratch` in two
+// passes of 64 columns, so that it leaves the CU as full 128-byte lines; no
+// other wave is involved, hence no workgroup barrier until the very end.
+//   * ignored tokens use lse = +inf, which makes every exp2 an exact +0;
+//   * the "- onehot" is applied by the one lane that owns the target column,
+//     from the fp32 value, after the bulk store (one rounding, as in ops.py:313-314).
+template <class T, bool ZREG>
+LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
+  typedef typename elem_of<T>::type E;
+  const int64_t v0 = a.v0 + (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wp = wave & 1, wq = wave >> 1;
+  const int64_t slice_v0 = v0 + wp * kWaveTile;
+  const float c1 = a.scale * kLog2e;
+  char* mine = scratch + wave * (kWaveTile * kDzRowBytes);
+  E* out = reinterpret_cast<E*>(a.dz) + (t0 + wq * kWaveTile) * a.vs + (int64_t)tp * kTile + wp * kWaveTile;
+
+  // per-token scalars of this lane's four tokens
+  float nlse[kNB], gain[kNB];
+  int ycol[kNB];
+#pragma unroll
+  for (int qb = 0; qb < kNB; ++qb) {
+    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+    const int64_t yy = a.y[tok];
+    const int64_t rel = yy - slice_v0;
+    const bool valid = yy != a.ignore_index;
+    const float l = a.lse[tok];
+    nlse[qb] = valid ? -l * kLog2e : -INFINITY;
+    gain[qb] = 1.f + 2.f * a.z_reg * l;
+    // target column inside this wave's slice, only in the lane half that holds it
+    ycol[qb] = (valid && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == (lane >> 5)) ? (int)rel : -1;
+  }
+
+#pragma unroll
+  for (int ph = 0; ph < 2; ++ph) {
+#pragma unroll
+    for (int qb = 0; qb < kNB; ++qb) {
+      const int row = qb * kBlk + (lane & 31);
+#pragma unroll
+      for (int pp = 0; pp < 2; ++pp) {
+        const int pb = 2 * ph + pp;
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int lcol = pp * kBlk + 8 * rq + 4 * (lane >> 5);  // column inside this pass
+          float d[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            d[j] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][rq * 4 + j], c1, nlse[qb]));
+            if (ZREG) d[j] *= gain[qb];
+          }
+          u32x2_t v;
+          v[0] = pack2<T>(d[0], d[1]);
+          v[1] = pack2<T>(d[2], d[3]);
+          *reinterpret_cast<u32x2_t*>(mine + row * kDzRowBytes + lcol * 2) = v;
+        }
+      }
+      // the target column, if it falls into this pass
+      const int yl = ycol[qb] - ph * 64;
+      if (yl >= 0 && yl < 64) {
+        const int want = (yl >> 5) * 16 + ((yl >> 3) & 3) * 4 + (yl & 3);  // (pp, register) index
+        float zt = 0.f;
+#pragma unroll
+        for (int pp = 0; pp < 2; ++pp)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (want == pp * 16 + r) zt = acc[2 * ph + pp][qb][r];
+        float p = __builtin_amdgcn_exp2f(fmaf(zt, c1, nlse[qb]));
+        if (ZREG) p *= gain[qb];
+        *reinterpret_cast<unsigned short*>(mine + row * kDzRowBytes + yl * 2) = to_bits<T>(p - 1.f);
+      }
+      // keep the register footprint small: an operand tile is in flight across this function
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // read the pass back as 128-byte rows and send it out
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int idx = i * 64 + lane;
+      const int row = idx >> 3, chunk = idx & 7;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * kDzRowBytes + chunk * 16);
+      *reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + ph * 64 + chunk * 8) = v;
+    }
+  }
+  __syncthreads();  // scratch is handed back to the main loop
+}
+
+template <class T>
+LCE_DEV void dz_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
+  if (a.z_reg != 0.f) {
+    dz_epilogue_impl<T, true>(a, acc, tp, tq, scratch);
+  } else {
+    dz_epilogue_impl<T, false>(a, acc, tp, tq, scratch);
+  }
+}
+
+template <class T> struct DzProblem {
+  typedef typename elem_of<T>::type E;
+  const BwdArgs& a;
+  int tiles_p, tiles_q;
+  LCE_DEV DzProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.N / kTile)) {}
+  LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
+  LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
+    int tp, tq;
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    p = reinterpret_cast<const E*>(a.w) + a.v0 + (int64_t)tp * kTile;
+    q = reinterpret_cast<const E*>(a.x) + (int64_t)tq * kTile * a.ldx;
+  }
+  LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
+    int tp, tq;
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    dz_epilogue<T>(a, acc, tp, tq, scratch);
+  }
+};
+
+template <class T>
+__global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  DzProblem<T> prob(a);
+  Pipe3<T, false, true, DzProblem<T>> pipe(prob);
+  pipe.run(a.ldw, a.ldx, (int)(a.H / kBK), lds);
+}
 
 template <class T, class XSrc, class WSrc>
 __global__ __launch_bounds__(kThreads) void bwd_dz_kernel(const BwdArgs a) {
@@ -25,72 +153,31 @@ __global__ __launch_bounds__(kThreads) void bwd_dz_kernel(const BwdArgs a) {
   const int tiles_p = (int)(a.vs / kTile), tiles_q = (int)(a.N / kTile);
   int tp, tq;
   tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
-  const int64_t v0 = a.v0 + (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wp = wave & 1, wq = wave >> 1;
-  const int64_t slice_v0 = v0 + wp * kWaveTile;
-
-  int ycol[kNB];
-  float nlse[kNB], gain[kNB];
-  bool valid[kNB];
-#pragma unroll
-  for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-    const int64_t yy = a.y[tok];
-    const int64_t rel = yy - slice_v0;
-    valid[qb] = yy != a.ignore_index;
-    ycol[qb] = (valid[qb] && rel >= 0 && rel < kWaveTile) ? (int)rel : -1;
-    const float l = a.lse[tok];
-    nlse[qb] = -l * kLog2e;
-    gain[qb] = 1.f + 2.f * a.z_reg * l;
-  }
-
   f32x16_t acc[kNB][kNB];
-  gemm_tile<T, WSrc, false, XSrc, true>(
-      acc, reinterpret_cast<const WSrc*>(a.w) + v0, a.ldw,
-      reinterpret_cast<const XSrc*>(a.x) + t0 * a.ldx, a.ldx, (int)(a.H / kBK), lds);
-
-  const float c1 = a.scale * kLog2e;
-#pragma unroll
-  for (int qb = 0; qb < kNB; ++qb) {
-    const int row = wq * kWaveTile + qb * kBlk + (lane & 31);
-#pragma unroll
-    for (int pb = 0; pb < kNB; ++pb)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int col = pb * kBlk + 8 * rq + 4 * (lane >> 5);  // inside the wave's slice
-        float d[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float p = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][rq * 4 + j], c1, nlse[qb])) * gain[qb];
-          if (col + j == ycol[qb]) p -= 1.f;
-          d[j] = valid[qb] ? p : 0.f;
-        }
-        u32x2_t v;
-        v[0] = pack2<T>(d[0], d[1]);
-        v[1] = pack2<T>(d[2], d[3]);
-        *reinterpret_cast<u32x2_t*>(lds + row * kDzRowBytes + (wp * kWaveTile + col) * 2) = v;
-      }
-  }
-  __syncthreads();
-  typedef typename elem_of<T>::type E;
-  E* out = reinterpret_cast<E*>(a.dz) + t0 * a.vs + (int64_t)tp * kTile;
-#pragma unroll 4
-  for (int i = 0; i < kTile * 32 / kThreads; ++i) {
-    const int idx = i * kThreads + threadIdx.x;
-    const int row = idx >> 5, u = idx & 31;
-    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * kDzRowBytes + u * 16);
-    *reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + u * 8) = v;
-  }
+  gemm_mainloop<T, WSrc, false, XSrc, true>(
+      acc, reinterpret_cast<const WSrc*>(a.w) + a.v0 + (int64_t)tp * kTile, a.ldw,
+      reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx, a.ldx, (int)(a.H / kBK), lds);
+  dz_epilogue<T>(a, acc, tp, tq, lds);
 }
 
 template <class T, class XSrc, class WSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
   auto kern = bwd_dz_kernel<T, XSrc, WSrc>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kDzLds);
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e != hipSuccess) return e;
   const int grid = (int)((a.vs / kTile) * (a.N / kTile));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kDzLds, s, a);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kLdsBytes, s, a);
+  return hipGetLastError();
+}
+
+template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dz_persistent_kernel<T>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (e != hipSuccess) return e;
+  const int64_t tiles = (a.vs / kTile) * (a.N / kTile);
+  const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kLdsBytes, s, a);
   return hipGetLastError();
 }
 
@@ -99,9 +186,9 @@ template <class T, class XSrc, class WSrc> hipError_t launch(const BwdArgs& a, h
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch<BF16, bf, bf>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
   if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch<BF16, bf, float>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch<F16, hf, hf>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch<F16, hf, float>(a, s);
   if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch<BF16, float, float>(a, s);
   return hipErrorInvalidValue;

@@ -12,7 +12,7 @@
 // forms the per-token loss terms (ops.py:753-761); fwd_final_kernel sums them
 // in a fixed order into the five scalars of ops.py:802 and the valid-label
 // count of ops.py:705.  All reductions are order-deterministic.
-#include "lce_gemm2.h"
+#include "lce_gemm3.h"
 #include "lce_internal.h"
 
 namespace lce {
@@ -25,14 +25,15 @@ constexpr float kLn2 = 0.6931471805599453f;
 LCE_DEV float fast_exp2(float v) { return __builtin_amdgcn_exp2f(v); }
 LCE_DEV float fast_log(float v) { return __builtin_amdgcn_logf(v) * kLn2; }
 
-template <class T, class XSrc, class WSrc>
-__global__ __launch_bounds__(kThreads) void fwd_tiles_kernel(const FwdArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int tiles_p = (int)(a.V / kTile), tiles_q = (int)(a.N / kTile);
-  int tp, tq;
-  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
+// Reduces the finished 256(v) x 256(token) accumulator of tile (tp, tq) to the
+// per-slice partials.  Accumulator rows (v) lie along registers and columns
+// (tokens) along lanes, so each lane reduces its own tokens in registers and
+// meets the other half of the vocabulary slice in lane ^ 32.
+template <class T>
+LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   const int64_t v0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
   const int64_t slice_v0 = v0 + wp * kWaveTile;
 
@@ -45,11 +46,6 @@ __global__ __launch_bounds__(kThreads) void fwd_tiles_kernel(const FwdArgs a) {
     const int64_t rel = yy - slice_v0;
     ycol[qb] = (yy != a.ignore_index && rel >= 0 && rel < kWaveTile) ? (int)rel : -1;
   }
-
-  f32x16_t acc[kNB][kNB];
-  gemm_tile<T, WSrc, false, XSrc, true>(
-      acc, reinterpret_cast<const WSrc*>(a.w) + v0, a.ldw,
-      reinterpret_cast<const XSrc*>(a.x) + t0 * a.ldx, a.ldx, (int)(a.H / kBK), lds);
 
   const float c1 = a.scale * kLog2e;
   const int64_t slice = slice_v0 / kChunkV;
@@ -106,6 +102,48 @@ __global__ __launch_bounds__(kThreads) void fwd_tiles_kernel(const FwdArgs a) {
       a.tgt[tok] = zt * a.scale;
     }
   }
+}
+
+// 16-bit x and W: persistent workgroups, pipelined across output tiles.
+template <class T> struct FwdProblem {
+  typedef typename elem_of<T>::type E;
+  const FwdArgs& a;
+  int tiles_p, tiles_q;
+  LCE_DEV FwdProblem(const FwdArgs& a_) : a(a_), tiles_p((int)(a_.V / kTile)), tiles_q((int)(a_.N / kTile)) {}
+  LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
+  LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
+    int tp, tq;
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    p = reinterpret_cast<const E*>(a.w) + (int64_t)tp * kTile;
+    q = reinterpret_cast<const E*>(a.x) + (int64_t)tq * kTile * a.ldx;
+  }
+  LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
+    int tp, tq;
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    fwd_epilogue<T>(a, acc, tp, tq);
+  }
+};
+
+template <class T>
+__global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const FwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  FwdProblem<T> prob(a);
+  Pipe3<T, false, true, FwdProblem<T>> pipe(prob);
+  pipe.run(a.ldw, a.ldx, (int)(a.H / kBK), lds);
+}
+
+// fp32 W (and possibly fp32 x), converted on the way into LDS: one tile per workgroup.
+template <class T, class XSrc, class WSrc>
+__global__ __launch_bounds__(kThreads) void fwd_tiles_kernel(const FwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int tiles_p = (int)(a.V / kTile), tiles_q = (int)(a.N / kTile);
+  int tp, tq;
+  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
+  f32x16_t acc[kNB][kNB];
+  gemm_mainloop<T, WSrc, false, XSrc, true>(
+      acc, reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile, a.ldw,
+      reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx, a.ldx, (int)(a.H / kBK), lds);
+  fwd_epilogue<T>(a, acc, tp, tq);
 }
 
 // One workgroup = 64 tokens x 4 strided groups of slices.
@@ -231,14 +269,25 @@ template <class T, class XSrc, class WSrc> hipError_t launch_tiles(const FwdArgs
   return hipGetLastError();
 }
 
+template <class T> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
+  auto kern = fwd_tiles_persistent_kernel<T>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
+  if (e != hipSuccess) return e;
+  const int64_t tiles = (a.V / kTile) * (a.N / kTile);
+  const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_tiles<BF16, bf, bf>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
   if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch_tiles<BF16, bf, float>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_tiles<F16, hf, hf>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_tiles<F16, hf, float>(a, s);
   if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch_tiles<BF16, float, float>(a, s);
   return hipErrorInvalidValue;

@@ -72,6 +72,16 @@ template <class T> LCE_DEV unsigned short to_bits(float f) {
 template <class T> LCE_DEV unsigned int pack2(float lo, float hi) {
   return (unsigned int)to_bits<T>(lo) | ((unsigned int)to_bits<T>(hi) << 16);
 }
+// threadIdx.x behind an optimisation barrier.  Epilogues that run inside a
+// persistent tile loop derive their per-lane indices from this, so that the
+// compiler recomputes them per tile instead of hoisting them out of the loop
+// and keeping them alive (in scarce vector registers) across the main loop.
+LCE_DEV int opaque_tid() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
 // Bit pattern -> float.  Takes the word by value on purpose: bit-casting a
 // vector element expression directly reads element 0 for every index.
 LCE_DEV float as_f32(unsigned int u) { return __builtin_bit_cast(float, u); }

@@ -1,0 +1,290 @@
+// Persistent, software-pipelined contraction for 16-bit operands.
+//
+// One workgroup per CU walks a list of 256 x 256 output tiles.  The operand
+// fetch is one continuous stream of K tiles that runs THROUGH output-tile
+// boundaries: while the last K tiles of output tile A are being multiplied,
+// the first K tiles of output tile B are already in flight, so B starts
+// without a load bubble and A's epilogue overlaps B's memory latency.
+//
+// Per K tile (64 deep) each wave issues 64 MFMAs and, between them,
+//   * the LDS reads of the next k-step's fragments (double buffered),
+//   * the LDS stores of K tile t+1 (from one of two register staging sets),
+//   * the buffer loads of K tile t+3 (into the set just stored),
+// spread over the k-steps so the four waves, which leave the single barrier
+// in lockstep, never oversubscribe the LDS port.  Staging set and LDS stage are
+// compile-time constants (the loop is unrolled by two); the accumulator of an
+// output tile is started by feeding a zero C operand to its first 16 MFMAs.
+//
+// Across an epilogue only ONE staging set stays in flight (K tile 1 of the next
+// output tile) and no fragments: the last K tile of an output tile issues no
+// loads, and the first K tile of the next one issues two tiles' worth.  That
+// leaves the epilogue most of the register file, so nothing spills.
+//
+// K tiles per output tile (`ktiles`) must be a multiple of 2 and at least 4, so
+// that the first K tile of every output tile lands in LDS stage 0.
+#pragma once
+
+#include "lce_gemm.h"
+
+namespace lce {
+
+struct StageRegs {
+  u32x4_t v[8];  // 8 x 16-byte chunks per thread per operand tile
+};
+
+#define LCE_SG_MFMA 0x008
+#define LCE_SG_VMEM_RD 0x020
+#define LCE_SG_DS_RD 0x100
+#define LCE_SG_DS_WR 0x200
+
+// Operand tiles are fetched with buffer loads: the resource descriptor (in
+// SGPRs) points at the current K tile, each thread contributes one 32-bit byte
+// offset, and the stride between a thread's 8 chunks is a scalar offset, so a
+// load costs one instruction and no vector address arithmetic.
+template <bool KC> struct Stager3 {
+  const char* base;      // uniform: first byte of the K tile being loaded
+  unsigned range;        // uniform: 0x7fffffff, or 0 when the stream has run off the last tile
+  unsigned voff;         // per-thread byte offset of its first chunk
+  unsigned iter_stride;  // uniform: bytes between this thread's consecutive chunks
+  int64_t k_stride;      // bytes between consecutive K tiles
+  int lds_off;           // per-thread byte offset of chunk 0 inside the operand tile
+
+  LCE_DEV void init(int64_t ld) {
+    const int t = threadIdx.x;
+    if (KC) {
+      const int c = t & 7, r = t >> 3;
+      voff = (unsigned)(((int64_t)r * ld + c * 8) * 2);
+      iter_stride = (unsigned)(32 * ld * 2);
+      k_stride = kBK * 2;
+      const int sw = (r & 7) ^ ((r >> 3) & 1);
+      lds_off = r * 128 + ((c ^ sw) << 4);
+    } else {
+      const int c = t & 31, k = t >> 5;
+      voff = (unsigned)(((int64_t)k * ld + c * 8) * 2);
+      iter_stride = (unsigned)(8 * ld * 2);
+      k_stride = (int64_t)kBK * ld * 2;
+      const int j = k & 3;
+      const int mask = ((j & 1) << 7) | ((j >> 1) << 6) | ((j & 1) << 5);
+      lds_off = k * 512 + ((c << 4) ^ mask);
+    }
+  }
+  LCE_DEV void load(StageRegs& r, int i0, int i1) const {
+    // 0x00020000: raw 32-bit data format.  range == 0 turns every load into a
+    // zero-filling no-op (used once the stream is past the last output tile).
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, (int)range, 0x00020000);
+#pragma unroll
+    for (int i = i0; i < i1; ++i)
+      r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, (int)(i * iter_stride), 0);
+  }
+  LCE_DEV void store(const StageRegs& r, char* tile, int i0, int i1) const {
+    constexpr int step = KC ? 32 * 128 : 8 * 512;
+#pragma unroll
+    for (int i = i0; i < i1; ++i) *reinterpret_cast<u32x4_t*>(tile + lds_off + i * step) = r.v[i];
+  }
+};
+
+// What a kernel plugs into the persistent loop.
+//   int  num_tiles()                              output tiles in this launch
+//   void origins(int tile, const void*& p, const void*& q)
+//        first element of the P / Q operand of that output tile:
+//        (row0, k=0) for a KC operand, (k=0, col0) for an MC operand
+//   void epilogue(int tile, acc, char* scratch)
+//        consumes the finished accumulator; may use `scratch`, 96 KiB of LDS
+//        that the pipeline does not touch until the next barrier it issues
+//        itself -- the epilogue must end with all its LDS traffic complete
+//        (a __syncthreads() if it used scratch).
+template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
+  Stager3<P_KC> ps;
+  Stager3<Q_KC> qs;
+  FragReader<P_KC> pr;
+  FragReader<Q_KC> qr;
+  s16x8_t pf[2][kNB], qf[2][kNB];
+  char* lds;
+  Problem& prob;
+  int ktiles;
+  int load_tile;  // output tile the fetch stream is in
+
+  static constexpr int kPReads = P_KC ? 4 : 8;  // LDS read instructions per k-step
+  static constexpr int kQReads = Q_KC ? 4 : 8;
+  static constexpr int kReads = kPReads + kQReads;
+
+  LCE_DEV Pipe3(Problem& p) : prob(p) {}
+
+  LCE_DEV void stream_begin(int tile) {
+    load_tile = tile;
+    if (tile < prob.num_tiles()) {
+      const void *p, *q;
+      prob.origins(tile, p, q);
+      ps.base = reinterpret_cast<const char*>(p);
+      qs.base = reinterpret_cast<const char*>(q);
+      ps.range = qs.range = 0x7fffffffu;
+    } else {
+      ps.range = qs.range = 0;
+    }
+  }
+  LCE_DEV void stream_advance() {
+    ps.base += ps.k_stride;
+    qs.base += qs.k_stride;
+  }
+  // chunks 0..7 of a staged K tile belong to P, 8..15 to Q
+  LCE_DEV void store_chunks(const StageRegs& sp, const StageRegs& sq, char* stage, int c0, int c1) {
+    if (c0 < 8) ps.store(sp, stage, c0, c1 < 8 ? c1 : 8);
+    if (c1 > 8) qs.store(sq, stage + kTileBytes, c0 > 8 ? c0 - 8 : 0, c1 - 8);
+  }
+  LCE_DEV void load_chunks(StageRegs& sp, StageRegs& sq, int c0, int c1) {
+    if (c0 < 8) ps.load(sp, c0, c1 < 8 ? c1 : 8);
+    if (c1 > 8) qs.load(sq, c0 > 8 ? c0 - 8 : 0, c1 - 8);
+  }
+  LCE_DEV void read_frags(int buf, const char* stage, int ks) {
+#pragma unroll
+    for (int b = 0; b < kNB; ++b) pf[buf][b] = pr.read(stage, b, ks);
+#pragma unroll
+    for (int b = 0; b < kNB; ++b) qf[buf][b] = qr.read(stage + kTileBytes, b, ks);
+  }
+  template <bool ZERO> LCE_DEV void mfma_rows(f32x16_t (&acc)[kNB][kNB], int buf, int i0, int i1) {
+#pragma unroll
+    for (int i = i0; i < i1; ++i)
+#pragma unroll
+      for (int j = 0; j < kNB; ++j) {
+        f32x16_t c;
+        if (ZERO) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) c[r] = 0.f;
+        } else {
+          c = acc[i][j];
+        }
+        acc[i][j] = mfma32<T>(pf[buf][i], qf[buf][j], c);
+      }
+  }
+
+  // One K tile held in LDS stage STAGE.  `sp/sq` is the staging set holding K
+  // tile t+1: it is stored to the other LDS stage here and refilled with K tile
+  // t+3.  FIRST: first K tile of an output tile: the C operand is zero and K tile
+  // t+2 is fetched as well, into `op/oq` (the set of this tile's own parity),
+  // because the previous output tile's last step fetched nothing.  WRAP: K tile
+  // t+3 is the last of this output tile, so the stream moves on afterwards.
+  // LAST: last K tile of an output tile: no fetch, no fragment prefetch.
+  template <int STAGE, bool FIRST, bool WRAP, bool LAST>
+  LCE_DEV void step(f32x16_t (&acc)[kNB][kNB], StageRegs& sp, StageRegs& sq, StageRegs& op,
+                    StageRegs& oq) {
+    const char* cur = lds + STAGE * kStageBytes;
+    char* nxt = lds + (STAGE ^ 1) * kStageBytes;
+
+    // k-step 0: MFMAs on buffer 0; fragment reads for step 1; LDS stores 0..5
+    read_frags(1, cur, 1);
+    store_chunks(sp, sq, nxt, 0, 6);
+    if (FIRST) {
+      load_chunks(op, oq, 0, 16);
+      stream_advance();
+    }
+    mfma_rows<FIRST>(acc, 0, 0, kNB);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
+      if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
+      if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
+      if (FIRST) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // k-step 1: MFMAs on buffer 1; reads for step 2; stores 6..10; loads 0..5
+    read_frags(0, cur, 2);
+    store_chunks(sp, sq, nxt, 6, 11);
+    if (!LAST) load_chunks(sp, sq, 0, 6);
+    mfma_rows<false>(acc, 1, 0, kNB);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
+      if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
+      if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
+      if (!LAST && i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // k-step 2: MFMAs on buffer 0; reads for step 3; stores 11..15; loads 6..10
+    read_frags(1, cur, 3);
+    store_chunks(sp, sq, nxt, 11, 16);
+    if (!LAST) load_chunks(sp, sq, 6, 11);
+    mfma_rows<false>(acc, 0, 0, kNB);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
+      if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
+      if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
+      if (!LAST && i >= 6 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // k-step 3: first half with loads 11..15; barrier; reads for the next K tile's step 0; second half
+    if (!LAST) load_chunks(sp, sq, 11, 16);
+    mfma_rows<false>(acc, 1, 0, kNB / 2);
+    if (!LAST) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
+        if (i < 5) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (!LAST) {
+      if (WRAP) {
+        stream_begin(load_tile + (int)gridDim.x);
+      } else {
+        stream_advance();
+      }
+    }
+    __syncthreads();
+    if (!LAST) read_frags(0, nxt, 0);
+    mfma_rows<false>(acc, 1, kNB / 2, kNB);
+    if (!LAST) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
+        if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, (kReads + 3) / 4, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  LCE_DEV void run(int64_t ldp, int64_t ldq, int ktiles_, char* lds_) {
+    lds = lds_;
+    ktiles = ktiles_;
+    const int wave = threadIdx.x >> 6;
+    ps.init(ldp);
+    qs.init(ldq);
+    pr.init((wave & 1) * kWaveTile);
+    qr.init((wave >> 1) * kWaveTile);
+
+    StageRegs p0, q0, p1, q1;  // set 0 stages even K tiles, set 1 odd ones
+    stream_begin((int)blockIdx.x);
+    load_chunks(p0, q0, 0, 16);
+    stream_advance();
+    load_chunks(p1, q1, 0, 16);
+    stream_advance();
+    store_chunks(p0, q0, lds, 0, 16);
+    __syncthreads();
+
+    f32x16_t acc[kNB][kNB];
+    for (int tile = (int)blockIdx.x; tile < prob.num_tiles(); tile += (int)gridDim.x) {
+      read_frags(0, lds, 0);
+      if (ktiles == 4) {
+        step<0, true, true, false>(acc, p1, q1, p0, q0);
+      } else {
+        step<0, true, false, false>(acc, p1, q1, p0, q0);
+        step<1, false, false, false>(acc, p0, q0, p1, q1);
+        for (int t = 2; t < ktiles - 4; t += 2) {
+          step<0, false, false, false>(acc, p1, q1, p0, q0);
+          step<1, false, false, false>(acc, p0, q0, p1, q1);
+        }
+        step<0, false, true, false>(acc, p1, q1, p0, q0);
+      }
+      step<1, false, false, false>(acc, p0, q0, p1, q1);
+      step<0, false, false, false>(acc, p1, q1, p0, q0);
+      step<1, false, false, true>(acc, p0, q0, p1, q1);
+      prob.epilogue(tile, acc, lds + kStageBytes);
+    }
+  }
+};
+
+}  // namespace lce

@@ -23,6 +23,7 @@ struct FwdArgs {
   int64_t ignore_index;
   float scale, z_reg;
   int monitoring;
+  int num_cus;  // compute units of the device: grid size of the persistent kernels
   // outputs / scratch
   float* lse;        // [N]
   float* out5;       // [5]
@@ -53,6 +54,7 @@ struct BwdArgs {
   void* dz;         // [N][vs] staged dz in the compute type
   float* dx_acc;    // [N][H] fp32 running dx (null when there is a single slab)
   int first, last;  // slab position
+  int num_cus;      // compute units of the device: grid size of the persistent kernels
 };
 
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s);
