@@ -147,6 +147,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_bf16_N16384_H2048_V131072", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (a kernel of known traffic, to scale "
+                         "FETCH_SIZE / WRITE_SIZE counters collected with rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this operator is a single-GPU kernel path and this build measures one GPU only; "
@@ -173,6 +176,12 @@ def main():
         out[0].backward()
         return out[0]
 
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         loss = step()
     torch.cuda.synchronize()
