@@ -8,17 +8,17 @@
 //
 // Per K tile (64 deep) each wave issues 64 MFMAs and, between them,
 //   * the LDS reads of the next k-step's fragments (double buffered),
-//   * the LDS stores of K tile t+1 (from one of two register staging sets),
-//   * the buffer loads of K tile t+3 (into the set just stored),
+//   * the LDS stores of K tile t+1 (from the register staging set),
+//   * the buffer loads of K tile t+2 (each chunk into the register just stored),
 // spread over the k-steps so the four waves, which leave the single barrier
-// in lockstep, never oversubscribe the LDS port.  Staging set and LDS stage are
-// compile-time constants (the loop is unrolled by two); the accumulator of an
-// output tile is started by feeding a zero C operand to its first 16 MFMAs.
+// in lockstep, never oversubscribe the LDS port.  A load therefore has one K
+// tile (~2000 cycles) to arrive; a second staging set (two K tiles of slack)
+// measured less than 1 % faster and cost 64 registers, i.e. spills.  The LDS
+// stage is a compile-time constant (the loop is unrolled by two); the
+// accumulator of an output tile starts from a zero C operand.
 //
-// Across an epilogue only ONE staging set stays in flight (K tile 1 of the next
-// output tile) and no fragments: the last K tile of an output tile issues no
-// loads, and the first K tile of the next one issues two tiles' worth.  That
-// leaves the epilogue most of the register file, so nothing spills.
+// Across an epilogue the staging set (K tile 1 of the next output tile) stays in
+// flight but no fragments, which leaves the epilogue ~180 vector registers.
 //
 // K tiles per output tile (`ktiles`) must be a multiple of 2 and at least 4, so
 // that the first K tile of every output tile lands in LDS stage 0.
@@ -158,81 +158,69 @@ template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
       }
   }
 
-  // One K tile held in LDS stage STAGE.  `sp/sq` is the staging set holding K
-  // tile t+1: it is stored to the other LDS stage here and refilled with K tile
-  // t+3.  FIRST: first K tile of an output tile: the C operand is zero and K tile
-  // t+2 is fetched as well, into `op/oq` (the set of this tile's own parity),
-  // because the previous output tile's last step fetched nothing.  WRAP: K tile
-  // t+3 is the last of this output tile, so the stream moves on afterwards.
-  // LAST: last K tile of an output tile: no fetch, no fragment prefetch.
+  // One K tile t, held in LDS stage STAGE.  The staging set holds K tile t+1: it is
+  // stored to the other LDS stage and, chunk by chunk, refilled with K tile t+2.
+  // FIRST  first K tile of an output tile: zero C operand.
+  // WRAP   K tile t+2 is the last of this output tile: the stream moves on afterwards.
+  // LAST   last K tile of an output tile: no fragment prefetch (the epilogue follows).
   template <int STAGE, bool FIRST, bool WRAP, bool LAST>
-  LCE_DEV void step(f32x16_t (&acc)[kNB][kNB], StageRegs& sp, StageRegs& sq, StageRegs& op,
-                    StageRegs& oq) {
+  LCE_DEV void step(f32x16_t (&acc)[kNB][kNB], StageRegs& sp, StageRegs& sq) {
     const char* cur = lds + STAGE * kStageBytes;
     char* nxt = lds + (STAGE ^ 1) * kStageBytes;
 
     // k-step 0: MFMAs on buffer 0; fragment reads for step 1; LDS stores 0..5
     read_frags(1, cur, 1);
     store_chunks(sp, sq, nxt, 0, 6);
-    if (FIRST) {
-      load_chunks(op, oq, 0, 16);
-      stream_advance();
-    }
     mfma_rows<FIRST>(acc, 0, 0, kNB);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
       if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
-      if (FIRST) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
 
     // k-step 1: MFMAs on buffer 1; reads for step 2; stores 6..10; loads 0..5
     read_frags(0, cur, 2);
     store_chunks(sp, sq, nxt, 6, 11);
-    if (!LAST) load_chunks(sp, sq, 0, 6);
+    load_chunks(sp, sq, 0, 6);
     mfma_rows<false>(acc, 1, 0, kNB);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
       if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
-      if (!LAST && i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+      if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
 
     // k-step 2: MFMAs on buffer 0; reads for step 3; stores 11..15; loads 6..10
     read_frags(1, cur, 3);
     store_chunks(sp, sq, nxt, 11, 16);
-    if (!LAST) load_chunks(sp, sq, 6, 11);
+    load_chunks(sp, sq, 6, 11);
     mfma_rows<false>(acc, 0, 0, kNB);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
       if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
-      if (!LAST && i >= 6 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+      if (i >= 6 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
 
     // k-step 3: first half with loads 11..15; barrier; reads for the next K tile's step 0; second half
-    if (!LAST) load_chunks(sp, sq, 11, 16);
+    load_chunks(sp, sq, 11, 16);
     mfma_rows<false>(acc, 1, 0, kNB / 2);
-    if (!LAST) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
-        if (i < 5) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
-      }
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
+      if (i < 5) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (!LAST) {
-      if (WRAP) {
-        stream_begin(load_tile + (int)gridDim.x);
-      } else {
-        stream_advance();
-      }
+    if (WRAP) {
+      stream_begin(load_tile + (int)gridDim.x);
+    } else {
+      stream_advance();
     }
     __syncthreads();
     if (!LAST) read_frags(0, nxt, 0);
@@ -256,32 +244,30 @@ template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
     pr.init((wave & 1) * kWaveTile);
     qr.init((wave >> 1) * kWaveTile);
 
-    StageRegs p0, q0, p1, q1;  // set 0 stages even K tiles, set 1 odd ones
+    StageRegs sp, sq;
     stream_begin((int)blockIdx.x);
-    load_chunks(p0, q0, 0, 16);
+    load_chunks(sp, sq, 0, 16);
     stream_advance();
-    load_chunks(p1, q1, 0, 16);
+    store_chunks(sp, sq, lds, 0, 16);
+    load_chunks(sp, sq, 0, 16);
     stream_advance();
-    store_chunks(p0, q0, lds, 0, 16);
     __syncthreads();
 
     f32x16_t acc[kNB][kNB];
     for (int tile = (int)blockIdx.x; tile < prob.num_tiles(); tile += (int)gridDim.x) {
       read_frags(0, lds, 0);
-      if (ktiles == 4) {
-        step<0, true, true, false>(acc, p1, q1, p0, q0);
-      } else {
-        step<0, true, false, false>(acc, p1, q1, p0, q0);
-        step<1, false, false, false>(acc, p0, q0, p1, q1);
+      step<0, true, false, false>(acc, sp, sq);
+      if (ktiles > 4) {
+        step<1, false, false, false>(acc, sp, sq);
         for (int t = 2; t < ktiles - 4; t += 2) {
-          step<0, false, false, false>(acc, p1, q1, p0, q0);
-          step<1, false, false, false>(acc, p0, q0, p1, q1);
+          step<0, false, false, false>(acc, sp, sq);
+          step<1, false, false, false>(acc, sp, sq);
         }
-        step<0, false, true, false>(acc, p1, q1, p0, q0);
+        step<0, false, false, false>(acc, sp, sq);
       }
-      step<1, false, false, false>(acc, p0, q0, p1, q1);
-      step<0, false, false, false>(acc, p1, q1, p0, q0);
-      step<1, false, false, true>(acc, p0, q0, p1, q1);
+      step<1, false, true, false>(acc, sp, sq);
+      step<0, false, false, false>(acc, sp, sq);
+      step<1, false, false, true>(acc, sp, sq);
       prob.epilogue(tile, acc, lds + kStageBytes);
     }
   }
