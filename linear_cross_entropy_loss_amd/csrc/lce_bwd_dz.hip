@@ -106,21 +106,16 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
       const int row = idx >> 3, chunk = idx & 7;
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * kDzRowBytes + chunk * 16);
       *reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + ph * 64 + chunk * 8) = v;
+      if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most 4 rows in registers at a time
     }
   }
   __syncthreads();  // scratch is handed back to the main loop
 }
 
-template <class T>
-LCE_DEV void dz_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
-  if (a.z_reg != 0.f) {
-    dz_epilogue_impl<T, true>(a, acc, tp, tq, scratch);
-  } else {
-    dz_epilogue_impl<T, false>(a, acc, tp, tq, scratch);
-  }
-}
-
-template <class T> struct DzProblem {
+// ZREG (z_regularization != 0) is a compile-time switch of the kernels rather than a
+// branch inside them: with a branch the compiler hoists the accumulator reads of
+// both arms above it and needs every vector register at once.
+template <class T, bool ZREG> struct DzProblem {
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int tiles_p, tiles_q;
@@ -135,15 +130,15 @@ template <class T> struct DzProblem {
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
-    dz_epilogue<T>(a, acc, tp, tq, scratch);
+    dz_epilogue_impl<T, ZREG>(a, acc, tp, tq, scratch);
   }
 };
 
-template <class T>
+template <class T, bool ZREG>
 __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  DzProblem<T> prob(a);
-  Pipe3<T, false, true, DzProblem<T>> pipe(prob);
+  DzProblem<T, ZREG> prob(a);
+  Pipe3<T, false, true, DzProblem<T, ZREG>> pipe(prob);
   pipe.run(a.ldw, a.ldx, (int)(a.H / kBK), lds);
 }
 
@@ -157,7 +152,11 @@ __global__ __launch_bounds__(kThreads) void bwd_dz_kernel(const BwdArgs a) {
   gemm_mainloop<T, WSrc, false, XSrc, true>(
       acc, reinterpret_cast<const WSrc*>(a.w) + a.v0 + (int64_t)tp * kTile, a.ldw,
       reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx, a.ldx, (int)(a.H / kBK), lds);
-  dz_epilogue<T>(a, acc, tp, tq, lds);
+  if (a.z_reg != 0.f) {
+    dz_epilogue_impl<T, true>(a, acc, tp, tq, lds);
+  } else {
+    dz_epilogue_impl<T, false>(a, acc, tp, tq, lds);
+  }
 }
 
 template <class T, class XSrc, class WSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
@@ -170,8 +169,8 @@ template <class T, class XSrc, class WSrc> hipError_t launch(const BwdArgs& a, h
   return hipGetLastError();
 }
 
-template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dz_persistent_kernel<T>;
+template <class T, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dz_persistent_kernel<T, ZREG>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e != hipSuccess) return e;
@@ -179,6 +178,10 @@ template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s)
   const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kLdsBytes, s, a);
   return hipGetLastError();
+}
+
+template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  return a.z_reg != 0.f ? launch_persistent_z<T, true>(a, s) : launch_persistent_z<T, false>(a, s);
 }
 
 }  // namespace
