@@ -43,7 +43,7 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
   }
 }
 
-template <class T> struct DwProblem {
+template <class T, class XSrc> struct DwProblem {
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int tiles_p, tiles_q;
@@ -53,7 +53,7 @@ template <class T> struct DwProblem {
     int tp, tq;
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
     p = reinterpret_cast<const E*>(a.dz) + (int64_t)tp * kTile;
-    q = reinterpret_cast<const E*>(a.x) + (int64_t)tq * kTile;
+    q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile;
   }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
@@ -62,40 +62,17 @@ template <class T> struct DwProblem {
   }
 };
 
-template <class T>
+template <class T, class XSrc>
 __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  DwProblem<T> prob(a);
-  Pipe3<T, false, false, DwProblem<T>> pipe(prob);
+  typedef typename elem_of<T>::type E;
+  DwProblem<T, XSrc> prob(a);
+  Pipe3<T, E, false, XSrc, false, DwProblem<T, XSrc>> pipe(prob);
   pipe.run(a.vs, a.ldx, (int)(a.N / kBK), lds);
 }
 
-template <class T, class XSrc>
-__global__ __launch_bounds__(kThreads) void bwd_dw_kernel(const BwdArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  typedef typename elem_of<T>::type E;
-  const int tiles_p = (int)(a.vs / kTile), tiles_q = (int)(a.H / kTile);
-  int tp, tq;
-  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
-  f32x16_t acc[kNB][kNB];
-  gemm_mainloop<T, E, false, XSrc, false>(
-      acc, reinterpret_cast<const E*>(a.dz) + (int64_t)tp * kTile, a.vs,
-      reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile, a.ldx, (int)(a.N / kBK), lds);
-  dw_epilogue<T>(a, acc, tp, tq);
-}
-
-template <class T, class XSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dw_kernel<T, XSrc>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
-  if (e != hipSuccess) return e;
-  const int grid = (int)((a.vs / kTile) * (a.H / kTile));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
-  return hipGetLastError();
-}
-
-template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dw_persistent_kernel<T>;
+template <class T, class XSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dw_persistent_kernel<T, XSrc>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -110,9 +87,9 @@ template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s)
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
-  if (a.x_dtype == DT_F16) return launch_persistent<F16>(a, s);
-  if (a.x_dtype == DT_F32) return launch<BF16, float>(a, s);
+  if (a.x_dtype == DT_BF16) return launch_persistent<BF16, bf>(a, s);
+  if (a.x_dtype == DT_F16) return launch_persistent<F16, hf>(a, s);
+  if (a.x_dtype == DT_F32) return launch_persistent<BF16, float>(a, s);
   return hipErrorInvalidValue;
 }
 

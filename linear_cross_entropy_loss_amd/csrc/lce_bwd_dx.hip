@@ -44,7 +44,7 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
   }
 }
 
-template <class T> struct DxProblem {
+template <class T, class WSrc> struct DxProblem {
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int tiles_p, tiles_q;
@@ -53,7 +53,7 @@ template <class T> struct DxProblem {
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
-    p = reinterpret_cast<const E*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0;
+    p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0;
     q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs;
   }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
@@ -63,40 +63,17 @@ template <class T> struct DxProblem {
   }
 };
 
-template <class T>
+template <class T, class WSrc>
 __global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  DxProblem<T> prob(a);
-  Pipe3<T, true, true, DxProblem<T>> pipe(prob);
+  typedef typename elem_of<T>::type E;
+  DxProblem<T, WSrc> prob(a);
+  Pipe3<T, WSrc, true, E, true, DxProblem<T, WSrc>> pipe(prob);
   pipe.run(a.ldw, a.vs, (int)(a.vs / kBK), lds);
 }
 
-template <class T, class WSrc>
-__global__ __launch_bounds__(kThreads) void bwd_dx_kernel(const BwdArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  typedef typename elem_of<T>::type E;
-  const int tiles_p = (int)(a.H / kTile), tiles_q = (int)(a.N / kTile);
-  int tp, tq;
-  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
-  f32x16_t acc[kNB][kNB];
-  gemm_mainloop<T, WSrc, true, E, true>(
-      acc, reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0, a.ldw,
-      reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs, a.vs, (int)(a.vs / kBK), lds);
-  dx_epilogue<T>(a, acc, tp, tq);
-}
-
-template <class T, class WSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dx_kernel<T, WSrc>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
-  if (e != hipSuccess) return e;
-  const int grid = (int)((a.H / kTile) * (a.N / kTile));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
-  return hipGetLastError();
-}
-
-template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dx_persistent_kernel<T>;
+template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dx_persistent_kernel<T, WSrc>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -112,10 +89,10 @@ hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
   const bool bf_compute = a.x_dtype == DT_BF16 || a.x_dtype == DT_F32;
-  if (bf_compute && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
-  if (bf_compute && a.w_dtype == DT_F32) return launch<BF16, float>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch<F16, float>(a, s);
+  if (bf_compute && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf>(a, s);
+  if (bf_compute && a.w_dtype == DT_F32) return launch_persistent<BF16, float>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_persistent<F16, float>(a, s);
   return hipErrorInvalidValue;
 }
 

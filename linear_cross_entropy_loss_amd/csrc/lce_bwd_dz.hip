@@ -6,9 +6,8 @@
 // 16-bit compute type exactly where the reference casts dz before its dot
 // products (ops.py:314, 422).  The tile is transposed through LDS and written
 // to the row-major staging buffer dz[N][vs] of the current vocabulary slab
-// with 16-byte stores.  With 16-bit operands the kernel is persistent (one
-// workgroup per CU, operand stream pipelined across tiles); with an fp32
-// weight it runs one tile per workgroup and converts on the way into LDS.
+// with 16-byte stores.  The kernel is persistent (one workgroup per CU, operand
+// stream pipelined across tiles); fp32 operands are converted on the way into LDS.
 #include "lce_gemm3.h"
 #include "lce_internal.h"
 
@@ -18,7 +17,7 @@ namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kDzRowBytes = 64 * 2 + 16;             // padded LDS row of one 64-column pass
-constexpr int kLdsBytes = 160 * 1024;                // two main-loop stages + 32 KiB
+constexpr int kLdsBytes = 160 * 1024;                // two main-loop stages + 32 KiB of epilogue scratch
 static_assert(4 * kWaveTile * kDzRowBytes <= kLdsBytes - kStageBytes, "four wave slices must fit beside one stage");
 
 // Turns the finished logit tile (tp, tq) into dz and writes it out.
@@ -115,8 +114,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
 // ZREG (z_regularization != 0) is a compile-time switch of the kernels rather than a
 // branch inside them: with a branch the compiler hoists the accumulator reads of
 // both arms above it and needs every vector register at once.
-template <class T, bool ZREG> struct DzProblem {
-  typedef typename elem_of<T>::type E;
+template <class T, class XSrc, class WSrc, bool ZREG> struct DzProblem {
   const BwdArgs& a;
   int tiles_p, tiles_q;
   LCE_DEV DzProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.N / kTile)) {}
@@ -124,8 +122,8 @@ template <class T, bool ZREG> struct DzProblem {
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
-    p = reinterpret_cast<const E*>(a.w) + a.v0 + (int64_t)tp * kTile;
-    q = reinterpret_cast<const E*>(a.x) + (int64_t)tq * kTile * a.ldx;
+    p = reinterpret_cast<const WSrc*>(a.w) + a.v0 + (int64_t)tp * kTile;
+    q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
   }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
@@ -134,43 +132,16 @@ template <class T, bool ZREG> struct DzProblem {
   }
 };
 
-template <class T, bool ZREG>
+template <class T, class XSrc, class WSrc, bool ZREG>
 __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  DzProblem<T, ZREG> prob(a);
-  Pipe3<T, false, true, DzProblem<T, ZREG>> pipe(prob);
+  DzProblem<T, XSrc, WSrc, ZREG> prob(a);
+  Pipe3<T, WSrc, false, XSrc, true, DzProblem<T, XSrc, WSrc, ZREG>> pipe(prob);
   pipe.run(a.ldw, a.ldx, (int)(a.H / kBK), lds);
 }
 
-template <class T, class XSrc, class WSrc>
-__global__ __launch_bounds__(kThreads) void bwd_dz_kernel(const BwdArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int tiles_p = (int)(a.vs / kTile), tiles_q = (int)(a.N / kTile);
-  int tp, tq;
-  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
-  f32x16_t acc[kNB][kNB];
-  gemm_mainloop<T, WSrc, false, XSrc, true>(
-      acc, reinterpret_cast<const WSrc*>(a.w) + a.v0 + (int64_t)tp * kTile, a.ldw,
-      reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx, a.ldx, (int)(a.H / kBK), lds);
-  if (a.z_reg != 0.f) {
-    dz_epilogue_impl<T, true>(a, acc, tp, tq, lds);
-  } else {
-    dz_epilogue_impl<T, false>(a, acc, tp, tq, lds);
-  }
-}
-
-template <class T, class XSrc, class WSrc> hipError_t launch(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dz_kernel<T, XSrc, WSrc>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (e != hipSuccess) return e;
-  const int grid = (int)((a.vs / kTile) * (a.N / kTile));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kLdsBytes, s, a);
-  return hipGetLastError();
-}
-
-template <class T, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dz_persistent_kernel<T, ZREG>;
+template <class T, class XSrc, class WSrc, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dz_persistent_kernel<T, XSrc, WSrc, ZREG>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e != hipSuccess) return e;
@@ -180,8 +151,9 @@ template <class T, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, h
   return hipGetLastError();
 }
 
-template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  return a.z_reg != 0.f ? launch_persistent_z<T, true>(a, s) : launch_persistent_z<T, false>(a, s);
+template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  return a.z_reg != 0.f ? launch_persistent_z<T, XSrc, WSrc, true>(a, s)
+                        : launch_persistent_z<T, XSrc, WSrc, false>(a, s);
 }
 
 }  // namespace
@@ -189,11 +161,11 @@ template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s)
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch<BF16, bf, float>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch<F16, hf, float>(a, s);
-  if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch<BF16, float, float>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf, bf>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf, hf>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch_persistent<BF16, bf, float>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_persistent<F16, hf, float>(a, s);
+  if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch_persistent<BF16, float, float>(a, s);
   return hipErrorInvalidValue;
 }
 

@@ -104,9 +104,8 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, i
   }
 }
 
-// 16-bit x and W: persistent workgroups, pipelined across output tiles.
-template <class T> struct FwdProblem {
-  typedef typename elem_of<T>::type E;
+// Persistent workgroups, operand stream pipelined across output tiles.
+template <class T, class XSrc, class WSrc> struct FwdProblem {
   const FwdArgs& a;
   int tiles_p, tiles_q;
   LCE_DEV FwdProblem(const FwdArgs& a_) : a(a_), tiles_p((int)(a_.V / kTile)), tiles_q((int)(a_.N / kTile)) {}
@@ -114,8 +113,8 @@ template <class T> struct FwdProblem {
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
-    p = reinterpret_cast<const E*>(a.w) + (int64_t)tp * kTile;
-    q = reinterpret_cast<const E*>(a.x) + (int64_t)tq * kTile * a.ldx;
+    p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile;
+    q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
   }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
@@ -124,26 +123,12 @@ template <class T> struct FwdProblem {
   }
 };
 
-template <class T>
+template <class T, class XSrc, class WSrc>
 __global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  FwdProblem<T> prob(a);
-  Pipe3<T, false, true, FwdProblem<T>> pipe(prob);
+  FwdProblem<T, XSrc, WSrc> prob(a);
+  Pipe3<T, WSrc, false, XSrc, true, FwdProblem<T, XSrc, WSrc>> pipe(prob);
   pipe.run(a.ldw, a.ldx, (int)(a.H / kBK), lds);
-}
-
-// fp32 W (and possibly fp32 x), converted on the way into LDS: one tile per workgroup.
-template <class T, class XSrc, class WSrc>
-__global__ __launch_bounds__(kThreads) void fwd_tiles_kernel(const FwdArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int tiles_p = (int)(a.V / kTile), tiles_q = (int)(a.N / kTile);
-  int tp, tq;
-  tile_coords(blockIdx.x, gridDim.x, tiles_p, tiles_q, 4, tp, tq);
-  f32x16_t acc[kNB][kNB];
-  gemm_mainloop<T, WSrc, false, XSrc, true>(
-      acc, reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile, a.ldw,
-      reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx, a.ldx, (int)(a.H / kBK), lds);
-  fwd_epilogue<T>(a, acc, tp, tq);
 }
 
 // One workgroup = 64 tokens x 4 strided groups of slices.
@@ -259,18 +244,8 @@ __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
   for (; i < n; i += stride) p[i] = v;
 }
 
-template <class T, class XSrc, class WSrc> hipError_t launch_tiles(const FwdArgs& a, hipStream_t s) {
-  auto kern = fwd_tiles_kernel<T, XSrc, WSrc>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
-  if (e != hipSuccess) return e;
-  const int grid = (int)((a.V / kTile) * (a.N / kTile));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
-  return hipGetLastError();
-}
-
-template <class T> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
-  auto kern = fwd_tiles_persistent_kernel<T>;
+template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
+  auto kern = fwd_tiles_persistent_kernel<T, XSrc, WSrc>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -285,11 +260,11 @@ template <class T> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s)
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch_tiles<BF16, bf, float>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_tiles<F16, hf, float>(a, s);
-  if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch_tiles<BF16, float, float>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf, bf>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf, hf>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch_persistent<BF16, bf, float>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_persistent<F16, hf, float>(a, s);
+  if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch_persistent<BF16, float, float>(a, s);
   return hipErrorInvalidValue;
 }
 

@@ -106,73 +106,6 @@ LCE_DEV void tile_coords(int bid, int nblocks, int tiles_p, int tiles_q, int ban
 }
 
 // ---------------------------------------------------------------------------
-// Global -> register -> LDS staging of one operand tile.
-// SrcT is the element type in memory: 2 bytes (already the compute type) or
-// float (converted to the compute type on the way into LDS).
-// ---------------------------------------------------------------------------
-template <class T, class SrcT, bool KC> struct TileStager {
-  static constexpr bool kWide = sizeof(SrcT) == 4;
-  // 16-byte chunks of 8 compute elements; 2048 chunks per tile, 8 per thread.
-  static constexpr int kIter = kTile * kBK / 8 / kThreads;
-  u32x4_t raw[kIter * (kWide ? 2 : 1)];
-  const SrcT* gptr;     // this thread's first chunk of the current K tile
-  int64_t iter_stride;  // elements between this thread's consecutive chunks
-  int64_t k_stride;     // elements between consecutive K tiles
-  int lds_off;          // byte offset of the first chunk inside the operand tile
-
-  // origin: element (row0, k=0) for KC, (k=0, col0) for MC; ld = row stride.
-  LCE_DEV void init(const SrcT* origin, int64_t ld) {
-    const int t = threadIdx.x;
-    if (KC) {
-      const int c = t & 7, r = t >> 3;  // 8 chunks per 64-element row, 32 rows per pass
-      gptr = origin + (int64_t)r * ld + c * 8;
-      iter_stride = 32 * ld;
-      k_stride = kBK;
-      const int sw = (r & 7) ^ ((r >> 3) & 1);
-      lds_off = r * 128 + ((c ^ sw) << 4);
-    } else {
-      const int c = t & 31, k = t >> 5;  // 32 chunks per 256-element row, 8 k-rows per pass
-      gptr = origin + (int64_t)k * ld + c * 8;
-      iter_stride = 8 * ld;
-      k_stride = kBK * ld;
-      const int j = k & 3;
-      const int mask = ((j & 1) << 7) | ((j >> 1) << 6) | ((j & 1) << 5);
-      lds_off = k * 512 + ((c << 4) ^ mask);
-    }
-  }
-  LCE_DEV void load() {
-#pragma unroll
-    for (int i = 0; i < kIter; ++i) {
-      const u32x4_t* p = reinterpret_cast<const u32x4_t*>(gptr + i * iter_stride);
-      if (kWide) {
-        raw[2 * i] = p[0];
-        raw[2 * i + 1] = p[1];
-      } else {
-        raw[i] = p[0];
-      }
-    }
-    gptr += k_stride;
-  }
-  LCE_DEV void store(char* tile) const {
-    constexpr int step = KC ? 32 * 128 : 8 * 512;
-#pragma unroll
-    for (int i = 0; i < kIter; ++i) {
-      u32x4_t v;
-      if (kWide) {
-        const u32x4_t a = raw[2 * i], b = raw[2 * i + 1];
-        v[0] = pack2<T>(as_f32(a[0]), as_f32(a[1]));
-        v[1] = pack2<T>(as_f32(a[2]), as_f32(a[3]));
-        v[2] = pack2<T>(as_f32(b[0]), as_f32(b[1]));
-        v[3] = pack2<T>(as_f32(b[2]), as_f32(b[3]));
-      } else {
-        v = raw[i];
-      }
-      *reinterpret_cast<u32x4_t*>(tile + lds_off + i * step) = v;
-    }
-  }
-};
-
-// ---------------------------------------------------------------------------
 // Fragment readers: per-lane LDS offsets for the four 32-wide blocks of this
 // wave's 128-wide slice of an operand tile.
 // ---------------------------------------------------------------------------
@@ -217,67 +150,9 @@ template <> struct FragReader<false> {
   }
 };
 
-// ---------------------------------------------------------------------------
-// Main loop: acc[pb][qb] += P-block x Q-block over `ktiles` K tiles.
-// The wave at (wp, wq) of the 2 x 2 wave grid owns P rows [wp*128, +128) and
-// Q rows [wq*128, +128) of the tile.  Accumulator element r of block
-// (pb, qb) in lane l is
+// Accumulator layout shared by all kernels: the wave at (wp, wq) of the 2 x 2 wave
+// grid owns P rows [wp*128, +128) and Q rows [wq*128, +128) of the tile, and
+// element r of block (pb, qb) in lane l is
 //     p = wp*128 + pb*32 + 8*(r/4) + 4*(l/32) + r%4,   q = wq*128 + qb*32 + l%32.
-// ---------------------------------------------------------------------------
-template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC>
-LCE_DEV void gemm_mainloop(f32x16_t (&acc)[kNB][kNB], const PSrc* p_origin, int64_t ldp,
-                           const QSrc* q_origin, int64_t ldq, int ktiles, char* lds) {
-  const int wave = threadIdx.x >> 6;
-  const int wp = wave & 1, wq = wave >> 1;
-
-  TileStager<T, PSrc, P_KC> ps;
-  TileStager<T, QSrc, Q_KC> qs;
-  ps.init(p_origin, ldp);
-  qs.init(q_origin, ldq);
-  FragReader<P_KC> pr;
-  FragReader<Q_KC> qr;
-  pr.init(wp * kWaveTile);
-  qr.init(wq * kWaveTile);
-
-#pragma unroll
-  for (int i = 0; i < kNB; ++i)
-#pragma unroll
-    for (int j = 0; j < kNB; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  ps.load();
-  qs.load();
-  ps.store(lds);
-  qs.store(lds + kTileBytes);
-  __syncthreads();
-
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const char* cur = lds + (kt & 1) * kStageBytes;
-    char* nxt = lds + ((kt + 1) & 1) * kStageBytes;
-    const bool more = kt + 1 < ktiles;
-    if (more) {
-      ps.load();
-      qs.load();
-    }
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      s16x8_t pf[kNB], qf[kNB];
-#pragma unroll
-      for (int b = 0; b < kNB; ++b) pf[b] = pr.read(cur, b, ks);
-#pragma unroll
-      for (int b = 0; b < kNB; ++b) qf[b] = qr.read(cur + kTileBytes, b, ks);
-#pragma unroll
-      for (int i = 0; i < kNB; ++i)
-#pragma unroll
-        for (int j = 0; j < kNB; ++j) acc[i][j] = mfma32<T>(pf[i], qf[j], acc[i][j]);
-    }
-    if (more) {
-      ps.store(nxt);
-      qs.store(nxt + kTileBytes);
-    }
-    __syncthreads();
-  }
-}
 
 }  // namespace lce

@@ -1,4 +1,5 @@
-// Persistent, software-pipelined contraction for 16-bit operands.
+// Persistent, software-pipelined contraction.  Operands are 16-bit in LDS; in memory
+// they are either already 16-bit or fp32 (converted on the way into LDS).
 //
 // One workgroup per CU walks a list of 256 x 256 output tiles.  The operand
 // fetch is one continuous stream of K tiles that runs THROUGH output-tile
@@ -28,8 +29,10 @@
 
 namespace lce {
 
-struct StageRegs {
-  u32x4_t v[8];  // 8 x 16-byte chunks per thread per operand tile
+// Register staging of one operand tile: 8 chunks of 8 elements per thread; a chunk
+// is one 16-byte register quad for 16-bit sources and two for fp32 sources.
+template <bool WIDE> struct StageRegs {
+  u32x4_t v[WIDE ? 16 : 8];
 };
 
 #define LCE_SG_MFMA 0x008
@@ -41,7 +44,10 @@ struct StageRegs {
 // SGPRs) points at the current K tile, each thread contributes one 32-bit byte
 // offset, and the stride between a thread's 8 chunks is a scalar offset, so a
 // load costs one instruction and no vector address arithmetic.
-template <bool KC> struct Stager3 {
+template <class T, class SrcT, bool KC> struct Stager3 {
+  static constexpr bool kWide = sizeof(SrcT) == 4;
+  static constexpr int kEs = (int)sizeof(SrcT);
+  typedef StageRegs<kWide> Regs;
   const char* base;      // uniform: first byte of the K tile being loaded
   unsigned range;        // uniform: 0x7fffffff, or 0 when the stream has run off the last tile
   unsigned voff;         // per-thread byte offset of its first chunk
@@ -53,34 +59,52 @@ template <bool KC> struct Stager3 {
     const int t = threadIdx.x;
     if (KC) {
       const int c = t & 7, r = t >> 3;
-      voff = (unsigned)(((int64_t)r * ld + c * 8) * 2);
-      iter_stride = (unsigned)(32 * ld * 2);
-      k_stride = kBK * 2;
+      voff = (unsigned)(((int64_t)r * ld + c * 8) * kEs);
+      iter_stride = (unsigned)(32 * ld * kEs);
+      k_stride = kBK * kEs;
       const int sw = (r & 7) ^ ((r >> 3) & 1);
       lds_off = r * 128 + ((c ^ sw) << 4);
     } else {
       const int c = t & 31, k = t >> 5;
-      voff = (unsigned)(((int64_t)k * ld + c * 8) * 2);
-      iter_stride = (unsigned)(8 * ld * 2);
-      k_stride = (int64_t)kBK * ld * 2;
+      voff = (unsigned)(((int64_t)k * ld + c * 8) * kEs);
+      iter_stride = (unsigned)(8 * ld * kEs);
+      k_stride = (int64_t)kBK * ld * kEs;
       const int j = k & 3;
       const int mask = ((j & 1) << 7) | ((j >> 1) << 6) | ((j & 1) << 5);
       lds_off = k * 512 + ((c << 4) ^ mask);
     }
   }
-  LCE_DEV void load(StageRegs& r, int i0, int i1) const {
+  LCE_DEV void load(Regs& r, int i0, int i1) const {
     // 0x00020000: raw 32-bit data format.  range == 0 turns every load into a
     // zero-filling no-op (used once the stream is past the last output tile).
     const __amdgpu_buffer_rsrc_t rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, (int)range, 0x00020000);
 #pragma unroll
-    for (int i = i0; i < i1; ++i)
-      r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, (int)(i * iter_stride), 0);
+    for (int i = i0; i < i1; ++i) {
+      if (kWide) {
+        r.v[2 * i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, (int)(i * iter_stride), 0);
+        r.v[2 * i + 1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff + 16, (int)(i * iter_stride), 0);
+      } else {
+        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, (int)(i * iter_stride), 0);
+      }
+    }
   }
-  LCE_DEV void store(const StageRegs& r, char* tile, int i0, int i1) const {
+  LCE_DEV void store(const Regs& r, char* tile, int i0, int i1) const {
     constexpr int step = KC ? 32 * 128 : 8 * 512;
 #pragma unroll
-    for (int i = i0; i < i1; ++i) *reinterpret_cast<u32x4_t*>(tile + lds_off + i * step) = r.v[i];
+    for (int i = i0; i < i1; ++i) {
+      u32x4_t v;
+      if (kWide) {
+        const u32x4_t a = r.v[2 * i], b = r.v[2 * i + 1];
+        v[0] = pack2<T>(as_f32(a[0]), as_f32(a[1]));
+        v[1] = pack2<T>(as_f32(a[2]), as_f32(a[3]));
+        v[2] = pack2<T>(as_f32(b[0]), as_f32(b[1]));
+        v[3] = pack2<T>(as_f32(b[2]), as_f32(b[3]));
+      } else {
+        v = r.v[i];
+      }
+      *reinterpret_cast<u32x4_t*>(tile + lds_off + i * step) = v;
+    }
   }
 };
 
@@ -94,9 +118,15 @@ template <bool KC> struct Stager3 {
 //        that the pipeline does not touch until the next barrier it issues
 //        itself -- the epilogue must end with all its LDS traffic complete
 //        (a __syncthreads() if it used scratch).
-template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
-  Stager3<P_KC> ps;
-  Stager3<Q_KC> qs;
+template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> struct Pipe3 {
+  typedef Stager3<T, PSrc, P_KC> PStager;
+  typedef Stager3<T, QSrc, Q_KC> QStager;
+  typedef typename PStager::Regs PRegs;
+  typedef typename QStager::Regs QRegs;
+  static constexpr int kPW = PStager::kWide ? 2 : 1;  // load instructions per chunk
+  static constexpr int kQW = QStager::kWide ? 2 : 1;
+  PStager ps;
+  QStager qs;
   FragReader<P_KC> pr;
   FragReader<Q_KC> qr;
   s16x8_t pf[2][kNB], qf[2][kNB];
@@ -128,11 +158,11 @@ template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
     qs.base += qs.k_stride;
   }
   // chunks 0..7 of a staged K tile belong to P, 8..15 to Q
-  LCE_DEV void store_chunks(const StageRegs& sp, const StageRegs& sq, char* stage, int c0, int c1) {
+  LCE_DEV void store_chunks(const PRegs& sp, const QRegs& sq, char* stage, int c0, int c1) {
     if (c0 < 8) ps.store(sp, stage, c0, c1 < 8 ? c1 : 8);
     if (c1 > 8) qs.store(sq, stage + kTileBytes, c0 > 8 ? c0 - 8 : 0, c1 - 8);
   }
-  LCE_DEV void load_chunks(StageRegs& sp, StageRegs& sq, int c0, int c1) {
+  LCE_DEV void load_chunks(PRegs& sp, QRegs& sq, int c0, int c1) {
     if (c0 < 8) ps.load(sp, c0, c1 < 8 ? c1 : 8);
     if (c1 > 8) qs.load(sq, c0 > 8 ? c0 - 8 : 0, c1 - 8);
   }
@@ -164,7 +194,7 @@ template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
   // WRAP   K tile t+2 is the last of this output tile: the stream moves on afterwards.
   // LAST   last K tile of an output tile: no fragment prefetch (the epilogue follows).
   template <int STAGE, bool FIRST, bool WRAP, bool LAST>
-  LCE_DEV void step(f32x16_t (&acc)[kNB][kNB], StageRegs& sp, StageRegs& sq) {
+  LCE_DEV void step(f32x16_t (&acc)[kNB][kNB], PRegs& sp, QRegs& sq) {
     const char* cur = lds + STAGE * kStageBytes;
     char* nxt = lds + (STAGE ^ 1) * kStageBytes;
 
@@ -190,7 +220,7 @@ template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
       if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
-      if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+      if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 0..5: P
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -204,7 +234,8 @@ template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
       if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
-      if (i >= 6 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+      if (i >= 6 && i < 10 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 6, 7: P
+      if (i >= 10 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);           // chunks 8..10: Q
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -214,7 +245,7 @@ template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
-      if (i < 5) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
+      if (i < 5) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);  // chunks 11..15: Q
     }
     __builtin_amdgcn_sched_barrier(0);
     if (WRAP) {
@@ -244,7 +275,8 @@ template <class T, bool P_KC, bool Q_KC, class Problem> struct Pipe3 {
     pr.init((wave & 1) * kWaveTile);
     qr.init((wave >> 1) * kWaveTile);
 
-    StageRegs sp, sq;
+    PRegs sp;
+    QRegs sq;
     stream_begin((int)blockIdx.x);
     load_chunks(sp, sq, 0, 16);
     stream_advance();
