@@ -86,14 +86,7 @@ def time_phases(cfg, x, y, w, torch, reps=5):
     bwd(0)
     torch.cuda.synchronize()
     # launches per call: the backward runs once per vocabulary slab
-    slabs = 1
-    while True:
-        vs = V // slabs
-        if V % slabs == 0 and vs % 256 == 0:
-            need = N * vs * 2 + (N * H * 4 if slabs > 1 else 0)
-            if need <= cfg["n_chunk"] * V * 4:
-                break
-        slabs += 1
+    slabs, _ = _lib.backward_plan(prob(0))
     out = {}
     for name, fn, ph, launches, flops in (
         ("fwd_tiles", fwd, _lib.PHASE_FWD_TILES, 1, 2.0 * N * H * V),

@@ -109,6 +109,14 @@ int lce_check_problem(const lce_problem* p);
 int lce_workspace_bytes(const lce_problem* p, size_t* fwd_bytes, size_t* bwd_bytes);
 
 /*
+ * How lce_backward will split problem `p`: it stages dz for all tokens of one
+ * vocabulary slab at a time (`slab_width` columns, `slabs` = V / slab_width
+ * passes).  The counterpart of the reference's loop over N_chunk_size-row
+ * groups (ops.py:721), which exists for the same purpose: bounding scratch.
+ */
+int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width);
+
+/*
  * Forward.  Replaces the launch of linear_xent_fwd_prep_bwd_kernel_matmul_t
  * (ops.py:722-752) and the torch reductions around it (ops.py:705, 753-761,
  * 793-794, 802), without ever writing logits to memory.

@@ -20,6 +20,7 @@ EXPORTS = (
     "lce_last_hip_error",
     "lce_check_problem",
     "lce_workspace_bytes",
+    "lce_backward_plan",
     "lce_forward",
     "lce_backward",
 )
@@ -78,6 +79,8 @@ def load():
     lib.lce_check_problem.argtypes = [P]
     lib.lce_workspace_bytes.restype = ctypes.c_int
     lib.lce_workspace_bytes.argtypes = [P, ctypes.POINTER(sz), ctypes.POINTER(sz)]
+    lib.lce_backward_plan.restype = ctypes.c_int
+    lib.lce_backward_plan.argtypes = [P, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]
     lib.lce_forward.restype = ctypes.c_int
     lib.lce_forward.argtypes = [P, vp, vp, vp, vp, vp, vp, vp, sz, vp]
     lib.lce_backward.restype = ctypes.c_int
@@ -126,3 +129,11 @@ def workspace_bytes(prob: LceProblem) -> tuple[int, int]:
     raise_for_status(lib.lce_workspace_bytes(ctypes.byref(prob), ctypes.byref(f), ctypes.byref(b)),
                      "lce_workspace_bytes")
     return int(f.value), int(b.value)
+
+
+def backward_plan(prob: LceProblem) -> tuple[int, int]:
+    """(number of vocabulary slabs, slab width) lce_backward will use for `prob`."""
+    lib = load()
+    n, w = ctypes.c_int64(0), ctypes.c_int64(0)
+    raise_for_status(lib.lce_backward_plan(ctypes.byref(prob), ctypes.byref(n), ctypes.byref(w)), "lce_backward_plan")
+    return int(n.value), int(w.value)

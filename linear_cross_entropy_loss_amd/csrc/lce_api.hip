@@ -65,16 +65,19 @@ struct BwdPlan {
   size_t dz, dx_acc, total;
 };
 
-// Fewest vocabulary slabs whose staging fits in n_chunk * V * 4 bytes.
+// Fewest vocabulary slabs whose staging fits in n_chunk * V * 4 bytes.  The dz
+// stage itself is additionally capped at 1 GiB: wider slabs are not faster, so a
+// generous N_chunk_size does not translate into a larger footprint.
 int plan_bwd(const lce_problem* p, BwdPlan* b) {
   const size_t budget = (size_t)p->n_chunk * (size_t)p->V * 4;
+  const size_t dz_cap = (size_t)1 << 30;
   for (int64_t s = 1; s <= p->V / 256; ++s) {
     if (p->V % s) continue;
     const int64_t vs = p->V / s;
     if (vs % 256) continue;
     const size_t dz = align_up((size_t)p->N * (size_t)vs * 2);
     const size_t acc = s > 1 ? align_up((size_t)p->N * (size_t)p->H * 4) : 0;
-    if (dz + acc <= budget) {
+    if (dz + acc <= budget && (dz <= dz_cap || vs == 256)) {
       b->slabs = s;
       b->vs = vs;
       b->dz = 0;
@@ -132,6 +135,17 @@ int lce_workspace_bytes(const lce_problem* p, size_t* fwd_bytes, size_t* bwd_byt
     if (rc != LCE_OK) return rc;
     *bwd_bytes = b.total;
   }
+  return LCE_OK;
+}
+
+int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width) {
+  int rc = check(p, false);
+  if (rc != LCE_OK) return rc;
+  BwdPlan b;
+  rc = plan_bwd(p, &b);
+  if (rc != LCE_OK) return rc;
+  if (slabs) *slabs = b.slabs;
+  if (slab_width) *slab_width = b.vs;
   return LCE_OK;
 }
 

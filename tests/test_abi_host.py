@@ -93,6 +93,19 @@ def test_backward_scratch_within_n_chunk_bound(N, H, V, n_chunk):
     assert fwd >= (V // 128) * N * 4
 
 
+def test_backward_plan_is_consistent_with_workspace():
+    from linear_cross_entropy_loss_amd import _lib
+
+    for N, H, V, nc in ((16384, 2048, 131072, 4096), (16384, 2048, 131072, 8192), (65536, 8192, 262144, 8192),
+                        (512, 256, 4096, 512)):
+        p = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc)
+        slabs, width = _lib.backward_plan(p)
+        assert slabs * width == V and width % 256 == 0
+        _, bwd = _lib.workspace_bytes(p)
+        assert bwd == N * width * 2 + (N * H * 4 if slabs > 1 else 0)
+        assert N * width * 2 <= max(1 << 30, N * 256 * 2)   # dz stage capped at 1 GiB
+
+
 def test_null_and_small_workspace_are_rejected_without_touching_the_gpu(lib):
     from linear_cross_entropy_loss_amd import _lib
 

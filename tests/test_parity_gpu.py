@@ -72,3 +72,41 @@ def test_forward_backward_matches_oracle(N, H, V, dtype, w_dtype, ign, z_reg, sc
         assert torch.equal(dx.cpu()[ignored].view(torch.int16 if dx.element_size() == 2 else torch.int32),
                            torch.zeros_like(dx.cpu()[ignored]).view(
                                torch.int16 if dx.element_size() == 2 else torch.int32))
+
+
+MID_CASES = [
+    # N, H, V, dtype, w_dtype, zipf, ignore_frac, z_reg, scale, n_chunk, monitoring
+    (2048, 1024, 32768, torch.float16, None, True, 0.1, 1e-4, 0.5, 4096, True),        # config-3 style: all features
+    (2048, 1024, 32768, torch.float16, torch.float32, True, 0.1, 0.0, 1.0, 512, False),  # config-5 style: fp32 master W
+    (4096, 512, 65536, torch.bfloat16, None, False, 0.05, 0.0, 1.0, 512, False),        # several vocabulary slabs
+    (2048, 2048, 16384, torch.float32, None, False, 0.0, 0.0, 1.0, 4096, False),        # config 1 (fp32 tensors)
+]
+
+
+@pytest.mark.parametrize("N,H,V,dtype,w_dtype,zipf,ign,z_reg,scale,n_chunk,mon", MID_CASES)
+def test_mid_size_matches_fp64_oracle_evaluated_on_gpu(N, H, V, dtype, w_dtype, zipf, ign, z_reg, scale, n_chunk, mon):
+    """Same comparison as above at sizes where the oracle is evaluated in fp64 on the GPU (row chunks)."""
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+    from oracle import lce_forward_backward_fp64
+
+    print(f"mid case N={N} H={H} V={V} {dtype} w={w_dtype} zipf={zipf} ign={ign} zreg={z_reg} scale={scale} "
+          f"chunk={n_chunk}", flush=True)
+    x, y, w = make_inputs(N, H, V, dtype, seed=7 * N + V, ignore_frac=ign, zipf=zipf, w_dtype=w_dtype, device="cuda")
+    xd = x.clone().requires_grad_(True)
+    wd = w.clone().requires_grad_(True)
+    out = linear_cross_entropy(xd, y, wd, -1, z_reg, scale, n_chunk, mon)
+    out[0].backward()
+    torch.cuda.synchronize()
+    ref = lce_forward_backward_fp64(x, y, w, -1, z_reg, scale, chunk=512)
+    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item())
+    if mon:
+        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item()) + 1e-3
+        assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item())
+        assert abs(out[4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item())
+    for name, got, want in (("dx", xd.grad, ref.dx), ("dw", wd.grad, ref.dw)):
+        d = got.double() - want
+        emax = (d.abs().max() / want.abs().max()).item()
+        el2 = (d.norm() / want.norm()).item()
+        print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
+        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
+    assert (xd.grad[y == -1] == 0).all()
