@@ -20,26 +20,43 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
+  const int half = lane >> 5;
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
     const int64_t h = h0 + wq * kWaveTile + qb * kBlk + (lane & 31);
 #pragma unroll
-    for (int pb = 0; pb < kNB; ++pb)
+    for (int pb = 0; pb < kNB; ++pb) {
+      const int64_t vb = a.v0 + vl0 + wp * kWaveTile + pb * kBlk;
+      if (a.dw_dtype == DT_F32) {
 #pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int64_t v = a.v0 + vl0 + wp * kWaveTile + pb * kBlk + 8 * rq + 4 * (lane >> 5);
-        f32x4_t o;
+        for (int rq = 0; rq < 4; ++rq) {
+          f32x4_t o;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o[j] = acc[pb][qb][rq * 4 + j] * coef;
-        if (a.dw_dtype == DT_F32) {
-          *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + h * a.lddw + v) = o;
-        } else {
-          u32x2_t b;
-          b[0] = pack2<T>(o[0], o[1]);
-          b[1] = pack2<T>(o[2], o[3]);
-          *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + v) = b;
+          for (int j = 0; j < 4; ++j) o[j] = acc[pb][qb][rq * 4 + j] * coef;
+          *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + h * a.lddw + vb + 8 * rq + 4 * half) = o;
+        }
+      } else {
+        // Lanes l and l+32 hold the two halves of every run of 8 columns; one
+        // lane-half swap per pair of register quads gives each lane a whole run,
+        // so a store writes 32 contiguous bytes (a full sector) per row of dW.
+#pragma unroll
+        for (int g = 0; g < 4; g += 2) {
+          float d[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) d[i] = acc[pb][qb][g * 4 + i] * coef;
+          const unsigned x0 = pack2<T>(d[0], d[1]), x1 = pack2<T>(d[2], d[3]);
+          const unsigned y0 = pack2<T>(d[4], d[5]), y1 = pack2<T>(d[6], d[7]);
+          const auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+          u32x4_t o;
+          o[0] = s0[0];
+          o[1] = s1[0];
+          o[2] = s0[1];
+          o[3] = s1[1];
+          *reinterpret_cast<u32x4_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + vb + 8 * (g + half)) = o;
         }
       }
+    }
   }
 }
 

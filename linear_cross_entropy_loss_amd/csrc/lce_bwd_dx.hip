@@ -52,13 +52,13 @@ template <class T, class WSrc> struct DxProblem {
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
     p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0;
     q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs;
   }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
     dx_epilogue<T>(a, acc, tp, tq);
   }
 };

@@ -5,8 +5,8 @@
 // (linear_cross_entropy/ops.py:309-314 and 415-422), rounded once to the
 // 16-bit compute type exactly where the reference casts dz before its dot
 // products (ops.py:314, 422).  The tile is transposed through LDS and written
-// to the row-major staging buffer dz[N][vs] of the current vocabulary slab
-// with 16-byte stores.  The kernel is persistent (one workgroup per CU, operand
+// to the row-major staging buffer dz[N][vs] of the current vocabulary slab as
+// full 128-byte lines.  The kernel is persistent (one workgroup per CU, operand
 // stream pipelined across tiles); fp32 operands are converted on the way into LDS.
 #include "lce_gemm3.h"
 #include "lce_internal.h"
@@ -16,20 +16,28 @@ namespace lce {
 namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr int kDzRowBytes = 64 * 2 + 16;             // padded LDS row of one 64-column pass
-constexpr int kLdsBytes = 160 * 1024;                // two main-loop stages + 32 KiB of epilogue scratch
-static_assert(4 * kWaveTile * kDzRowBytes <= kLdsBytes - kStageBytes, "four wave slices must fit beside one stage");
+constexpr int kPassCols = 64;                        // columns staged per pass
+constexpr int kSliceBytes = kWaveTile * kPassCols * 2;  // one wave's staging slice: 128 rows of 128 bytes
+constexpr int kLdsBytes = kMainloopLds;  // the epilogue stages through main-loop stage 1, idle by then
+static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must fit beside one stage");
 
 // Turns the finished logit tile (tp, tq) into dz and writes it out.
 //
 // Each lane owns 4 tokens (columns of the accumulator) x 64 vocabulary entries
-// per token, four consecutive entries per register quad.  A wave stages its own
-// 128(token) x 128(v) sub-tile through a private slice of `scratch` in two
-// passes of 64 columns, so that it leaves the CU as full 128-byte lines; no
-// other wave is involved, hence no workgroup barrier until the very end.
+// per token, four consecutive entries per register quad; lanes l and l+32 hold
+// the two halves of every run of 8 entries.  One v_permlane32_swap per pair of
+// register quads hands each lane a full run of 8 (16 bytes in the 16-bit
+// staging type).  A wave stages its own 128(token) x 128(v) sub-tile through a
+// private slice of `scratch` in two passes of 64 columns and reads it back as
+// whole 128-byte rows, so dz leaves the CU as full lines; no other wave is
+// involved, hence no workgroup barrier until the very end.  Staging rows are
+// 128 bytes with the 16-byte chunk index XOR-ed by (row >> 1) & 7, which keeps
+// both the 16-byte writes (32 rows per instruction) and the row reads (8 rows
+// per instruction) free of bank conflicts.
 //   * ignored tokens use lse = +inf, which makes every exp2 an exact +0;
 //   * the "- onehot" is applied by the one lane that owns the target column,
-//     from the fp32 value, after the bulk store (one rounding, as in ops.py:313-314).
+//     from the fp32 value, onto the staged pass (one rounding, as in
+//     ops.py:313-314).
 template <class T, bool ZREG>
 LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
   typedef typename elem_of<T>::type E;
@@ -37,14 +45,15 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
   const int tid = opaque_tid();
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
+  const int half = lane >> 5;
   const int64_t slice_v0 = v0 + wp * kWaveTile;
   const float c1 = a.scale * kLog2e;
-  char* mine = scratch + wave * (kWaveTile * kDzRowBytes);
+  char* mine = scratch + wave * kSliceBytes;
   E* out = reinterpret_cast<E*>(a.dz) + (t0 + wq * kWaveTile) * a.vs + (int64_t)tp * kTile + wp * kWaveTile;
 
   // per-token scalars of this lane's four tokens
   float nlse[kNB], gain[kNB];
-  int ycol[kNB];
+  int ykey[kNB];
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
     const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
@@ -55,7 +64,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
     nlse[qb] = valid ? -l * kLog2e : -INFINITY;
     gain[qb] = 1.f + 2.f * a.z_reg * l;
     // target column inside this wave's slice, only in the lane half that holds it
-    ycol[qb] = (valid && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == (lane >> 5)) ? (int)rel : -1;
+    ykey[qb] = (valid && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == half) ? (int)rel : -1;
   }
 
 #pragma unroll
@@ -63,27 +72,38 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
 #pragma unroll
     for (int qb = 0; qb < kNB; ++qb) {
       const int row = qb * kBlk + (lane & 31);
+      char* lrow = mine + row * (kPassCols * 2);
+      const int sw = (row >> 1) & 7;
 #pragma unroll
       for (int pp = 0; pp < 2; ++pp) {
         const int pb = 2 * ph + pp;
 #pragma unroll
-        for (int rq = 0; rq < 4; ++rq) {
-          const int lcol = pp * kBlk + 8 * rq + 4 * (lane >> 5);  // column inside this pass
-          float d[4];
+        for (int g = 0; g < 4; g += 2) {
+          float d[8];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            d[j] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][rq * 4 + j], c1, nlse[qb]));
-            if (ZREG) d[j] *= gain[qb];
+          for (int i = 0; i < 8; ++i) {
+            d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
+            if (ZREG) d[i] *= gain[qb];
           }
-          u32x2_t v;
-          v[0] = pack2<T>(d[0], d[1]);
-          v[1] = pack2<T>(d[2], d[3]);
-          *reinterpret_cast<u32x2_t*>(mine + row * kDzRowBytes + lcol * 2) = v;
+          const unsigned x0 = pack2<T>(d[0], d[1]), x1 = pack2<T>(d[2], d[3]);
+          const unsigned y0 = pack2<T>(d[4], d[5]), y1 = pack2<T>(d[6], d[7]);
+          // lanes 0..31 keep their quad g and receive the partner's quad g; lanes
+          // 32..63 receive the partner's quad g+1 and keep their own
+          const auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+          u32x4_t o;
+          o[0] = s0[0];
+          o[1] = s1[0];
+          o[2] = s0[1];
+          o[3] = s1[1];
+          const int chunk = pp * 4 + g + half;  // 16-byte chunk of the 64-column pass
+          *reinterpret_cast<u32x4_t*>(lrow + ((chunk ^ sw) << 4)) = o;
         }
       }
-      // the target column, if it falls into this pass
-      const int yl = ycol[qb] - ph * 64;
-      if (yl >= 0 && yl < 64) {
+      // the target column, if it falls into this pass: overwrite the staged value
+      // with the rounding of the fp32 (p - 1), as ops.py:313-314 rounds once
+      const int yl = ykey[qb] - ph * kPassCols;
+      if (yl >= 0 && yl < kPassCols) {
         const int want = (yl >> 5) * 16 + ((yl >> 3) & 3) * 4 + (yl & 3);  // (pp, register) index
         float zt = 0.f;
 #pragma unroll
@@ -93,7 +113,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
             if (want == pp * 16 + r) zt = acc[2 * ph + pp][qb][r];
         float p = __builtin_amdgcn_exp2f(fmaf(zt, c1, nlse[qb]));
         if (ZREG) p *= gain[qb];
-        *reinterpret_cast<unsigned short*>(mine + row * kDzRowBytes + yl * 2) = to_bits<T>(p - 1.f);
+        *reinterpret_cast<unsigned short*>(lrow + (((yl >> 3) ^ sw) << 4) + (yl & 7) * 2) = to_bits<T>(p - 1.f);
       }
       // keep the register footprint small: an operand tile is in flight across this function
       __builtin_amdgcn_sched_barrier(0);
@@ -103,8 +123,8 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
     for (int i = 0; i < 16; ++i) {
       const int idx = i * 64 + lane;
       const int row = idx >> 3, chunk = idx & 7;
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * kDzRowBytes + chunk * 16);
-      *reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + ph * 64 + chunk * 8) = v;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * (kPassCols * 2) + ((chunk ^ ((row >> 1) & 7)) << 4));
+      *reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + ph * kPassCols + chunk * 8) = v;
       if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most 4 rows in registers at a time
     }
   }
@@ -121,13 +141,13 @@ template <class T, class XSrc, class WSrc, bool ZREG> struct DzProblem {
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
     p = reinterpret_cast<const WSrc*>(a.w) + a.v0 + (int64_t)tp * kTile;
     q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
   }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
     dz_epilogue_impl<T, ZREG>(a, acc, tp, tq, scratch);
   }
 };
