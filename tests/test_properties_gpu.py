@@ -235,3 +235,45 @@ def test_full_size_properties(big):
     s = dw.float().sum(1).abs().max().item()
     a = dw.float().abs().sum(1).max().item()
     assert s <= 2e-3 * a, (s, a)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# The reference's own accuracy protocol (bench_fusions.py:480-512, error measures bench_fusions.py:437-444):
+# A ~ randn(V, H) with std 1, x = 0.1*A[y] + randn ("simulate low loss"), no ignored labels, errors as
+# torch.dist (L2 norm of the difference) against the fp64 evaluation of the same rounded inputs.  Its published
+# figures for its fused operator at this shape are  bf16: |dloss| 4.2e-5, (|ddx|+|ddA|)/2 5.3e-4;
+# fp16: 6.9e-5, 1.4e-4  (bench-acc/*over N*.csv:8), on other hardware and another random draw, so this is a
+# soft cross-check: same order of magnitude, not equality.
+# ---------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,pub_loss,pub_grad", [(torch.bfloat16, 4.2e-5, 5.3e-4), (torch.float16, 6.9e-5, 1.4e-4)])
+def test_reference_accuracy_protocol_full_size(dtype, pub_loss, pub_grad):
+    from oracle import lce_forward_backward_fp64
+
+    print(f"reference accuracy protocol {dtype}", flush=True)
+    N, H, V = 16384, 2048, 131072
+    g = torch.Generator(device="cuda").manual_seed(11)
+    y = torch.randint(0, V, (N,), device="cuda", generator=g)
+    A = torch.randn(V, H, device="cuda", generator=g).to(dtype)
+    w = A.T.contiguous()
+    x = (0.1 * A[y].float() + torch.randn(N, H, device="cuda", generator=g)).to(dtype)
+    del A
+    out, dx, dw = _fb(x, y, w, n_chunk=4096)
+    ref = lce_forward_backward_fp64(x, y, w, -1, 0.0, 1.0, chunk=512)
+    loss_err = abs(out[0].float().item() - ref.loss.float().item())
+    dx_err = torch.dist(ref.dx.float(), dx.float()).item()
+    dw_err = torch.dist(ref.dw.float(), dw.float()).item()
+    grad_err = 0.5 * (dx_err + dw_err)
+    print(f"  loss {ref.loss.item():.5f} |dloss| {loss_err:.3e} (published {pub_loss:.1e});  "
+          f"(|ddx|+|ddW|)/2 {grad_err:.3e} (published {pub_grad:.1e}); dx {dx_err:.3e} dW {dw_err:.3e}", flush=True)
+    # hard gates of this build
+    assert loss_err <= 1e-3 * abs(ref.loss.item())
+    for got, want in ((dx, ref.dx), (dw, ref.dw)):
+        d = got.double() - want
+        assert (d.abs().max() / want.abs().max()).item() <= 2e-2
+        assert (d.norm() / want.norm()).item() <= 2e-2
+    # soft cross-check against the published figures: no worse than twice the reference's own error
+    # (observed on MI355X: bf16 0 / 5.3e-4, fp16 0 / 1.1e-4)
+    assert loss_err <= 2 * pub_loss
+    assert grad_err <= 2 * pub_grad
+    del ref
+    torch.cuda.empty_cache()
