@@ -107,6 +107,36 @@ def time_phases(cfg, x, y, w, torch, reps=5):
     return out
 
 
+def median_step_ms(step, torch, reps=20, flush=False):
+    """Median of per-step event timings; with `flush`, a 256 MiB buffer is zeroed before every step so that
+    no operand starts in L2 / Infinity Cache (the protocol of triton.testing.do_bench, which the reference's
+    bench_fusions.py:280-281 uses)."""
+    cache = torch.empty(256 << 20, dtype=torch.int8, device="cuda") if flush else None
+    ts = []
+    for _ in range(reps):
+        if flush:
+            cache.zero_()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        step()
+        e.record()
+        torch.cuda.synchronize()
+        ts.append(s.elapsed_time(e))
+    ts.sort()
+    return 0.5 * (ts[(reps - 1) // 2] + ts[reps // 2])
+
+
+def host_cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(cfg, torch):
     """Eager fp32 linear + F.cross_entropy fwd+bwd on host cores, on a bounded row sample of the same workload."""
     from oracle import eager_fp32_step
@@ -128,6 +158,7 @@ def cpu_baseline(cfg, torch):
         ts.append(time.perf_counter() - t0)
     t = sorted(ts)[0]
     return dict(value=8.0 * Ns * H * V / t / 1e12, unit="TFLOP/s (8*N*H*V convention)", cores=threads, kind="port",
+                host_cpu=host_cpu_model(), os_cpu_count=os.cpu_count(),
                 sample=f"first {Ns} of {cfg['N']} rows at full H={H}, V={V}; eager fp32 matmul + F.cross_entropy "
                        f"fwd+bwd; 1 warm-up + 2 timed, best; {t * 1e3:.0f} ms per sample step",
                 ms_per_sample_step=t * 1e3)
@@ -195,6 +226,11 @@ def main():
     tflops = flops / ms / 1e9
     peak = PEAK_TFLOPS[cfg["dtype"]]
 
+    ms_median = median_step_ms(step, torch, reps=20, flush=False)
+    ms_median_flushed = median_step_ms(step, torch, reps=20, flush=True)
+    x.grad = None
+    w.grad = None
+
     phases = time_phases(cfg, x.detach(), y, w.detach(), torch)
     dom = max(phases, key=lambda k: phases[k]["ms_per_launch"] * phases[k]["launches_per_step"])
     d = phases[dom]
@@ -216,6 +252,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms,
+        "ms_per_step_median_events": ms_median,
+        "ms_per_step_median_events_cache_flushed": ms_median_flushed,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": tflops / REFERENCE_PUBLISHED_TFLOPS_8NHV if args.workload.startswith("c2") else None,

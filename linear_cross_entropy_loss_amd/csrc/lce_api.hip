@@ -26,7 +26,7 @@ bool is16(int d) { return d == LCE_BF16 || d == LCE_F16; }
 int check(const lce_problem* p, bool backward) {
   if (!p) return LCE_EINVAL_ARG;
   if (p->N <= 0 || p->H <= 0 || p->V <= 0 || p->n_chunk <= 0) return LCE_EINVAL_SHAPE;
-  if (p->N % 512 || p->H % 256 || p->V % 4096 || p->n_chunk % 512) return LCE_EINVAL_SHAPE;
+  // Any N, H, V; only the row strides are constrained (below).
   if (p->N > (int64_t)1 << 30 || p->V > (int64_t)1 << 30 || p->H > (int64_t)1 << 20) return LCE_EINVAL_SHAPE;
   const int xd = p->x_dtype, wd = p->w_dtype;
   const bool ok = (is16(xd) && (wd == xd || wd == LCE_F32)) || (xd == LCE_F32 && wd == LCE_F32);
@@ -37,7 +37,8 @@ int check(const lce_problem* p, bool backward) {
   if (backward) {
     if (p->dx_dtype != xd && p->dx_dtype != LCE_F32) return LCE_EINVAL_DTYPE;
     if (p->dw_dtype != wd && p->dw_dtype != LCE_F32) return LCE_EINVAL_DTYPE;
-    if (p->lddx < p->H || p->lddx % 4 || p->lddw < p->V || p->lddw % 4) return LCE_EINVAL_ARG;
+    // dx is stored in 8-byte (16-bit types) or 16-byte pieces, dW in 16-byte pieces
+    if (p->lddx < p->H || p->lddx % 4 || p->lddw < p->V || p->lddw % (p->dw_dtype == LCE_F32 ? 4 : 8)) return LCE_EINVAL_ARG;
   }
   return LCE_OK;
 }
@@ -48,14 +49,15 @@ struct FwdPlan {
 
 FwdPlan plan_fwd(const lce_problem* p) {
   FwdPlan f;
-  const size_t part = align_up((size_t)(p->V / lce::kChunkV) * (size_t)p->N * 4);
+  const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V);
+  const size_t part = align_up(Vp / lce::kChunkV * Np * 4);
   size_t o = 0;
   f.part_lse = o; o += part;
   f.part_max = o; if (p->monitoring) o += part;
   f.part_pz = o; if (p->monitoring) o += part;
   f.part_sq = o; if (p->monitoring) o += part;
-  f.tgt = o; o += align_up((size_t)p->N * 4);
-  f.blk = o; o += align_up((size_t)(p->N / lce::kMergeRows) * 8 * sizeof(double));
+  f.tgt = o; o += align_up(Np * 4);
+  f.blk = o; o += align_up(Np / lce::kMergeRows * 8 * sizeof(double));
   f.total = o;
   return f;
 }
@@ -65,20 +67,27 @@ struct BwdPlan {
   size_t dz, dx_acc, total;
 };
 
-// Fewest vocabulary slabs whose staging fits in n_chunk * V * 4 bytes.  The dz
-// stage itself is additionally capped at 1 GiB: wider slabs are not faster, so a
-// generous N_chunk_size does not translate into a larger footprint.
+// Fewest vocabulary slabs (of a width that is a multiple of 256 columns; the last
+// one may be narrower) whose staging fits in n_chunk * V * 4 bytes.  The dz stage
+// itself is additionally capped at 1 GiB: wider slabs are not faster, so a
+// generous N_chunk_size does not translate into a larger footprint.  When even
+// the narrowest slab does not fit (small V with many tokens: the fp32 running
+// dx alone exceeds the budget) the narrowest plan is used all the same -- the
+// budget is a target, the operator never refuses a shape because of it.
 int plan_bwd(const lce_problem* p, BwdPlan* b) {
   const size_t budget = (size_t)p->n_chunk * (size_t)p->V * 4;
   const size_t dz_cap = (size_t)1 << 30;
-  for (int64_t s = 1; s <= p->V / 256; ++s) {
-    if (p->V % s) continue;
-    const int64_t vs = p->V / s;
-    if (vs % 256) continue;
-    const size_t dz = align_up((size_t)p->N * (size_t)vs * 2);
-    const size_t acc = s > 1 ? align_up((size_t)p->N * (size_t)p->H * 4) : 0;
-    if (dz + acc <= budget && (dz <= dz_cap || vs == 256)) {
-      b->slabs = s;
+  const size_t Np = (size_t)lce::padded_tokens(p->N), Hp = (size_t)lce::padded_hidden(p->H);
+  const int64_t Vp = lce::padded_vocab(p->V);
+  const int64_t cols = Vp / 256;
+  for (int64_t s = 1; s <= cols; ++s) {
+    const int64_t vs = (cols + s - 1) / s * 256;
+    if (s > 1 && (cols + s - 2) / (s - 1) * 256 == vs) continue;  // same width as with one slab fewer
+    const int64_t slabs = (Vp + vs - 1) / vs;
+    const size_t dz = align_up(Np * (size_t)vs * 2);
+    const size_t acc = slabs > 1 ? align_up(Np * Hp * 4) : 0;
+    if ((dz + acc <= budget && dz <= dz_cap) || vs == 256) {
+      b->slabs = slabs;
       b->vs = vs;
       b->dz = 0;
       b->dx_acc = dz;
@@ -111,10 +120,12 @@ const char* lce_strerror(int status) {
   switch (status) {
     case LCE_OK: return "ok";
     case LCE_EINVAL_SHAPE:
-      return "shape outside the supported set (need N % 512 == 0, H % 256 == 0, V % 4096 == 0, N_chunk_size % 512 == 0)";
+      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N, V <= 2^30, H <= 2^20)";
     case LCE_EINVAL_DTYPE:
       return "unsupported dtype combination (x: bf16/f16/f32; w: x dtype or f32; grads: same dtype or f32)";
-    case LCE_EINVAL_ARG: return "invalid argument (null or misaligned pointer, bad stride, logit_scale <= 0 or z_reg < 0)";
+    case LCE_EINVAL_ARG:
+      return "invalid argument (null or misaligned pointer; row strides must be >= the row length and multiples of 8 "
+             "elements for 16-bit data, 4 for fp32; logit_scale <= 0 or z_reg < 0)";
     case LCE_EWORKSPACE: return "workspace missing or too small for this problem and N_chunk_size";
     case LCE_EHIP: return "HIP error";
     default: return "unknown status";
@@ -164,6 +175,7 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
   memset(&a, 0, sizeof(a));
   a.x = x; a.w = w; a.y = y;
   a.N = p->N; a.H = p->H; a.V = p->V; a.ldx = p->ldx; a.ldw = p->ldw;
+  a.Np = lce::padded_tokens(p->N); a.Vp = lce::padded_vocab(p->V);
   a.x_dtype = p->x_dtype; a.w_dtype = p->w_dtype;
   a.ignore_index = p->ignore_index;
   a.scale = p->logit_scale; a.z_reg = p->z_reg; a.monitoring = p->monitoring ? 1 : 0;
@@ -181,7 +193,7 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
   hipError_t e;
   if (ph & LCE_PHASE_FWD_TILES) {
     if (ph & LCE_PHASE_FWD_REDUCE) {  // a tiles-only (profiling) call reuses the zeroed buffer
-      e = lce::launch_fill_f32(a.tgt, a.N, 0.f, s);
+      e = lce::launch_fill_f32(a.tgt, a.Np, 0.f, s);
       if (e != hipSuccess) return hip_fail(e, "fill");
     }
     e = lce::launch_fwd_tiles(a, s);
@@ -213,6 +225,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   memset(&a, 0, sizeof(a));
   a.x = x; a.w = w; a.y = y; a.lse = lse; a.n_valid = n_valid; a.grad_out = grad_out;
   a.N = p->N; a.H = p->H; a.V = p->V;
+  a.Np = lce::padded_tokens(p->N); a.Hp = lce::padded_hidden(p->H);
   a.ldx = p->ldx; a.ldw = p->ldw; a.lddx = p->lddx; a.lddw = p->lddw;
   a.x_dtype = p->x_dtype; a.w_dtype = p->w_dtype; a.dx_dtype = p->dx_dtype; a.dw_dtype = p->dw_dtype;
   a.ignore_index = p->ignore_index;
@@ -220,13 +233,14 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.dx = dx; a.dw = dw;
   a.dz = base + b.dz;
   a.dx_acc = b.slabs > 1 ? (float*)(base + b.dx_acc) : nullptr;
-  a.vs = b.vs;
   rc = current_num_cus(&a.num_cus);
   if (rc != LCE_OK) return rc;
   const int ph = p->phases ? p->phases : ~0;
 
   for (int64_t i = 0; i < b.slabs; ++i) {
     a.v0 = i * b.vs;
+    a.vw = p->V - a.v0 < b.vs ? p->V - a.v0 : b.vs;   // columns of this slab that exist
+    a.vs = lce::pad_to(a.vw, 256);                    // its padded width: dz row stride and K extent of dx
     a.first = i == 0;
     a.last = i == b.slabs - 1;
     hipError_t e;

@@ -24,12 +24,16 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
     const int64_t h = h0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+    const bool row_exists = h < a.H;
 #pragma unroll
     for (int pb = 0; pb < kNB; ++pb) {
       const int64_t vb = a.v0 + vl0 + wp * kWaveTile + pb * kBlk;
+      // Pieces (4 columns in fp32, 8 in the 16-bit types) that start at or past V are not
+      // stored; one that V cuts through is written whole, into the stride padding of its row.
       if (a.dw_dtype == DT_F32) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
+          if (vb + 8 * rq + 4 * half >= a.V || !row_exists) continue;
           f32x4_t o;
 #pragma unroll
           for (int j = 0; j < 4; ++j) o[j] = acc[pb][qb][rq * 4 + j] * coef;
@@ -53,7 +57,8 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
           o[1] = s1[0];
           o[2] = s0[1];
           o[3] = s1[1];
-          *reinterpret_cast<u32x4_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + vb + 8 * (g + half)) = o;
+          if (vb + 8 * (g + half) < a.V && row_exists)
+            *reinterpret_cast<u32x4_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + vb + 8 * (g + half)) = o;
         }
       }
     }
@@ -64,7 +69,7 @@ template <class T, class XSrc> struct DwProblem {
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int tiles_p, tiles_q;
-  LCE_DEV DwProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.H / kTile)) {}
+  LCE_DEV DwProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.Hp / kTile)) {}
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
@@ -72,6 +77,9 @@ template <class T, class XSrc> struct DwProblem {
     p = reinterpret_cast<const E*>(a.dz) + (int64_t)tp * kTile;
     q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile;
   }
+  LCE_DEV const void* p_end() const { return reinterpret_cast<const E*>(a.dz) + a.Np * a.vs; }
+  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
+  LCE_DEV int k_valid() const { return (int)a.Np; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);
@@ -85,7 +93,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdAr
   typedef typename elem_of<T>::type E;
   DwProblem<T, XSrc> prob(a);
   Pipe3<T, E, false, XSrc, false, DwProblem<T, XSrc>> pipe(prob);
-  pipe.run(a.vs, a.ldx, (int)(a.N / kBK), lds);
+  pipe.run(a.vs, a.ldx, (int)(a.Np / kBK), lds);
 }
 
 template <class T, class XSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
@@ -93,7 +101,7 @@ template <class T, class XSrc> hipError_t launch_persistent(const BwdArgs& a, hi
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
-  const int64_t tiles = (a.vs / kTile) * (a.H / kTile);
+  const int64_t tiles = (a.vs / kTile) * (a.Hp / kTile);
   const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
   return hipGetLastError();

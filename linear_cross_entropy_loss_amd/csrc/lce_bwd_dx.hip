@@ -10,6 +10,13 @@ namespace lce {
 
 namespace {
 
+// The running sum lives in a padded [Np][Hp] fp32 buffer and needs no bounds.
+// The final result goes out through range-checked buffer stores: the descriptor
+// ends at the last element of dx, so rows past N are dropped by the hardware,
+// and quads of hidden indices that start at or past H are given an
+// out-of-range offset (a quad that H cuts through is written whole: the row
+// stride is a multiple of 4, so it stays inside its row).  No branches: a branch
+// around accumulator reads makes the compiler read all of them up front.
 template <class T>
 LCE_DEV void dx_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   typedef typename elem_of<T>::type E;
@@ -18,27 +25,45 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
+  const int es = a.dx_dtype == DT_F32 ? 4 : 2;
+  // descriptor over the rows of this tile: base = first row, range = bytes to the end of dx
+  const char* tile_base = reinterpret_cast<const char*>(a.dx) + t0 * a.lddx * es;
+  // whole dwords: with 16-bit data and an odd H the last row ends one element into its stride padding
+  const int64_t hcols = es == 2 ? (a.H + 1) & ~(int64_t)1 : a.H;
+  const int64_t left = (reinterpret_cast<const char*>(a.dx) + ((a.N - 1) * a.lddx + hcols) * es) - tile_base;
+  const unsigned range = left <= 0 ? 0u : (left > 0x7fffffff ? 0x7fffffffu : (unsigned)left);
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(tile_base), 0, (int)range, 0x00020000);
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+    const int row = wq * kWaveTile + qb * kBlk + (lane & 31);  // row inside the tile
+    const int64_t tok = t0 + row;
+    const unsigned row_off = (unsigned)(row * a.lddx * es);
 #pragma unroll
     for (int pb = 0; pb < kNB; ++pb)
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        const int64_t h = h0 + wp * kWaveTile + pb * kBlk + 8 * rq + 4 * (lane >> 5);
+        const int64_t hrun = h0 + wp * kWaveTile + pb * kBlk + 8 * rq;
+        const int64_t h = hrun + 4 * (lane >> 5);
         f32x4_t v;
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = acc[pb][qb][rq * 4 + j];
-        if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + tok * a.H + h);
+        if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + tok * a.Hp + h);
         if (!a.last) {
-          *reinterpret_cast<f32x4_t*>(a.dx_acc + tok * a.H + h) = v;
-        } else if (a.dx_dtype == DT_F32) {
-          *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dx) + tok * a.lddx + h) = v * coef;
+          *reinterpret_cast<f32x4_t*>(a.dx_acc + tok * a.Hp + h) = v;
         } else {
-          u32x2_t o;
-          o[0] = pack2<T>(v[0] * coef, v[1] * coef);
-          o[1] = pack2<T>(v[2] * coef, v[3] * coef);
-          *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dx) + tok * a.lddx + h) = o;
+          const unsigned off = h < a.H ? row_off + (unsigned)(h * es) : 0x80000000u;
+          if (a.dx_dtype == DT_F32) {
+            const f32x4_t o = v * coef;
+            u32x4_t bits;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bits[j] = __builtin_bit_cast(unsigned, (float)o[j]);
+            __builtin_amdgcn_raw_buffer_store_b128(bits, rsrc, (int)off, 0, 0);
+          } else {
+            u32x2_t o;
+            o[0] = pack2<T>(v[0] * coef, v[1] * coef);
+            o[1] = pack2<T>(v[2] * coef, v[3] * coef);
+            __builtin_amdgcn_raw_buffer_store_b64(o, rsrc, (int)off, 0, 0);
+          }
         }
       }
   }
@@ -48,7 +73,7 @@ template <class T, class WSrc> struct DxProblem {
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int tiles_p, tiles_q;
-  LCE_DEV DxProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.H / kTile)), tiles_q((int)(a_.N / kTile)) {}
+  LCE_DEV DxProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.Hp / kTile)), tiles_q((int)(a_.Np / kTile)) {}
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
@@ -56,6 +81,9 @@ template <class T, class WSrc> struct DxProblem {
     p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0;
     q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs;
   }
+  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.V); }
+  LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + a.Np * a.vs; }
+  LCE_DEV int k_valid() const { return (int)a.vw; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
@@ -77,7 +105,7 @@ template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hi
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
-  const int64_t tiles = (a.H / kTile) * (a.N / kTile);
+  const int64_t tiles = (a.Hp / kTile) * (a.Np / kTile);
   const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
   return hipGetLastError();

@@ -38,7 +38,13 @@ static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must
 //   * the "- onehot" is applied by the one lane that owns the target column,
 //     from the fp32 value, onto the staged pass (one rounding, as in
 //     ops.py:313-314).
-template <class T, bool ZREG>
+//
+// VTAIL is the variant for the one tile column that straddles the end of the
+// vocabulary: every run of 8 columns (a pair of register quads in lanes l, l+32)
+// but at most one is inside or outside as a whole, uniformly over the wave; the
+// one run that V cuts through is handled element by element.  Columns outside
+// are written as exact zeros.
+template <class T, bool ZREG, bool VTAIL>
 LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
   typedef typename elem_of<T>::type E;
   const int64_t v0 = a.v0 + (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
@@ -48,6 +54,11 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
   const int half = lane >> 5;
   const int64_t slice_v0 = v0 + wp * kWaveTile;
   const float c1 = a.scale * kLog2e;
+  // columns of this wave's slice that exist: nq whole runs of 8, then `cut` more columns
+  const int64_t left = a.v0 + a.vw - slice_v0;
+  const int vrem = VTAIL ? (int)(left < 0 ? 0 : (left > kWaveTile ? kWaveTile : left)) : kWaveTile;
+  const int nq = vrem >> 3, cut = vrem & 7;
+  const int cut_mine = cut - 4 * half;  // elements of this lane's quad of the cut run that exist (<= 0: none)
   char* mine = scratch + wave * kSliceBytes;
   E* out = reinterpret_cast<E*>(a.dz) + (t0 + wq * kWaveTile) * a.vs + (int64_t)tp * kTile + wp * kWaveTile;
 
@@ -57,10 +68,11 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
     const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-    const int64_t yy = a.y[tok];
+    const bool exists = tok < a.N;  // rows past N are staged as zeros, like ignored tokens
+    const int64_t yy = exists ? a.y[tok] : a.ignore_index;
     const int64_t rel = yy - slice_v0;
     const bool valid = yy != a.ignore_index;
-    const float l = a.lse[tok];
+    const float l = exists ? a.lse[tok] : 0.f;
     nlse[qb] = valid ? -l * kLog2e : -INFINITY;
     gain[qb] = 1.f + 2.f * a.z_reg * l;
     // target column inside this wave's slice, only in the lane half that holds it
@@ -81,9 +93,24 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
         for (int g = 0; g < 4; g += 2) {
           float d[8];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
-            if (ZREG) d[i] *= gain[qb];
+          for (int h2 = 0; h2 < 2; ++h2) {
+            if (!VTAIL || pb * 4 + g + h2 < nq) {
+#pragma unroll
+              for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
+                d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
+                if (ZREG) d[i] *= gain[qb];
+              }
+            } else if (pb * 4 + g + h2 == nq && cut != 0) {
+#pragma unroll
+              for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
+                d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
+                if (ZREG) d[i] *= gain[qb];
+                d[i] = (i - 4 * h2) < cut_mine ? d[i] : 0.f;
+              }
+            } else {
+#pragma unroll
+              for (int i = 4 * h2; i < 4 * h2 + 4; ++i) d[i] = 0.f;
+            }
           }
           const unsigned x0 = pack2<T>(d[0], d[1]), x1 = pack2<T>(d[2], d[3]);
           const unsigned y0 = pack2<T>(d[4], d[5]), y1 = pack2<T>(d[6], d[7]);
@@ -134,41 +161,64 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
 // ZREG (z_regularization != 0) is a compile-time switch of the kernels rather than a
 // branch inside them: with a branch the compiler hoists the accumulator reads of
 // both arms above it and needs every vector register at once.
-template <class T, class XSrc, class WSrc, bool ZREG> struct DzProblem {
+// The launch covers `tiles_p` tile columns of the slab starting at column tile
+// `tp0`: all the full ones, or (VTAIL) those from the one straddling the end
+// of the vocabulary to the end of the padded slab.
+template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL> struct DzProblem {
   const BwdArgs& a;
-  int tiles_p, tiles_q;
-  LCE_DEV DzProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.N / kTile)) {}
+  int tp0, tiles_p, tiles_q;
+  LCE_DEV DzProblem(const BwdArgs& a_)
+      : a(a_), tp0(VTAIL ? (int)(a_.vw / kTile) : 0),
+        tiles_p(VTAIL ? (int)(a_.vs / kTile - a_.vw / kTile) : (int)(a_.vw / kTile)), tiles_q((int)(a_.Np / kTile)) {}
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
+  LCE_DEV void coords(int tile, int& tp, int& tq) const {
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
+    tp += tp0;
+  }
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
+    coords(tile, tp, tq);
     p = reinterpret_cast<const WSrc*>(a.w) + a.v0 + (int64_t)tp * kTile;
     q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
   }
+  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.V); }
+  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
+  LCE_DEV int k_valid() const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
-    dz_epilogue_impl<T, ZREG>(a, acc, tp, tq, scratch);
+    coords(tile, tp, tq);
+    dz_epilogue_impl<T, ZREG, VTAIL>(a, acc, tp, tq, scratch);
   }
 };
 
-template <class T, class XSrc, class WSrc, bool ZREG>
+template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL>
 __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  DzProblem<T, XSrc, WSrc, ZREG> prob(a);
-  Pipe3<T, WSrc, false, XSrc, true, DzProblem<T, XSrc, WSrc, ZREG>> pipe(prob);
-  pipe.run(a.ldw, a.ldx, (int)(a.H / kBK), lds);
+  DzProblem<T, XSrc, WSrc, ZREG, VTAIL> prob(a);
+  Pipe3<T, WSrc, false, XSrc, true, DzProblem<T, XSrc, WSrc, ZREG, VTAIL>> pipe(prob);
+  pipe.run(a.ldw, a.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
-template <class T, class XSrc, class WSrc, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dz_persistent_kernel<T, XSrc, WSrc, ZREG>;
+template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL>
+hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
+  auto kern = bwd_dz_persistent_kernel<T, XSrc, WSrc, ZREG, VTAIL>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e != hipSuccess) return e;
-  const int64_t tiles = (a.vs / kTile) * (a.N / kTile);
   const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kLdsBytes, s, a);
   return hipGetLastError();
+}
+
+// All full tile columns of the slab, then the column that straddles the end of the vocabulary.
+template <class T, class XSrc, class WSrc, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
+  const int64_t tq = a.Np / kTile, full = a.vw / kTile, tail = a.vs / kTile - full;
+  if (full > 0) {
+    hipError_t e = launch_one<T, XSrc, WSrc, ZREG, false>(a, full * tq, s);
+    if (e != hipSuccess) return e;
+  }
+  if (tail > 0) return launch_one<T, XSrc, WSrc, ZREG, true>(a, tail * tq, s);
+  return hipSuccess;
 }
 
 template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {

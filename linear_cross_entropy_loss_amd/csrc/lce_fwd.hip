@@ -29,34 +29,59 @@ LCE_DEV float fast_log(float v) { return __builtin_amdgcn_logf(v) * kLn2; }
 // per-slice partials.  Accumulator rows (v) lie along registers and columns
 // (tokens) along lanes, so each lane reduces its own tokens in registers and
 // meets the other half of the vocabulary slice in lane ^ 32.
-template <class T>
+//
+// VTAIL is the variant for the one tile column that straddles V (V % 256 != 0).
+// A register quad covers 4 columns of a run of 8 (lanes l and l+32 hold the two
+// halves), so every run but at most one is inside or outside the vocabulary as a
+// whole, uniformly over the wave, and is taken or skipped with a scalar branch;
+// the one run that V cuts through is handled element by element.
+template <class T, bool VTAIL>
 LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   const int64_t v0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
   const int tid = opaque_tid();
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
   const int64_t slice_v0 = v0 + wp * kWaveTile;
-
-  // Column of the target inside this wave's 128-wide slice, or -1.
-  int ycol[kNB];
-#pragma unroll
-  for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-    const int64_t yy = a.y[tok];
-    const int64_t rel = yy - slice_v0;
-    ycol[qb] = (yy != a.ignore_index && rel >= 0 && rel < kWaveTile) ? (int)rel : -1;
-  }
+  // columns of this wave's slice inside the vocabulary: nq whole runs of 8, then `cut` more columns
+  const int64_t left = a.V - slice_v0;
+  const int vrem = VTAIL ? (int)(left < 0 ? 0 : (left > kWaveTile ? kWaveTile : left)) : kWaveTile;
+  const int nq = vrem >> 3, cut = vrem & 7;
+  const int mine = cut - 4 * (lane >> 5);  // elements of this lane's quad of the cut run that exist (<= 0: none)
 
   const float c1 = a.scale * kLog2e;
   const int64_t slice = slice_v0 / kChunkV;
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
     const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+    const int64_t o = slice * a.Np + tok;
+    if (VTAIL && vrem == 0) {  // nothing of this slice exists
+      if (lane < 32) {
+        a.part_lse[o] = -INFINITY;
+        if (a.monitoring) {
+          a.part_max[o] = -INFINITY;
+          a.part_pz[o] = 0.f;
+          a.part_sq[o] = 0.f;
+        }
+      }
+      continue;
+    }
+    // Column of the target inside this wave's 128-wide slice, or -1.
+    const int64_t yy = tok < a.N ? a.y[tok] : a.ignore_index;
+    const int64_t rel = yy - slice_v0;
+    const int yl = (yy != a.ignore_index && rel >= 0 && rel < kWaveTile) ? (int)rel : -1;
+
     float m = -INFINITY;
 #pragma unroll
     for (int pb = 0; pb < kNB; ++pb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) m = fmaxf(m, acc[pb][qb][r]);
+      for (int rq = 0; rq < 4; ++rq)
+        if (!VTAIL || pb * 4 + rq < nq) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) m = fmaxf(m, acc[pb][qb][rq * 4 + j]);
+        } else if (pb * 4 + rq == nq && cut != 0) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) m = j < mine ? fmaxf(m, acc[pb][qb][rq * 4 + j]) : m;
+        }
     m = fmaxf(m, __shfl_xor(m, 32));
     m *= a.scale;  // logit_scale > 0, so max commutes with the scaling
     const float mo = m * kLog2e;
@@ -65,24 +90,46 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, i
 #pragma unroll
       for (int pb = 0; pb < kNB; ++pb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = fast_exp2(fmaf(acc[pb][qb][r], c1, -mo));
-          const float z = acc[pb][qb][r] * a.scale;
-          s += e;
-          pz = fmaf(e, z, pz);
-          sq = fmaf(z, z, sq);
-        }
+        for (int rq = 0; rq < 4; ++rq)
+          if (!VTAIL || pb * 4 + rq < nq) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float e = fast_exp2(fmaf(acc[pb][qb][rq * 4 + j], c1, -mo));
+              const float z = acc[pb][qb][rq * 4 + j] * a.scale;
+              s += e;
+              pz = fmaf(e, z, pz);
+              sq = fmaf(z, z, sq);
+            }
+          } else if (pb * 4 + rq == nq && cut != 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float e = fast_exp2(fmaf(acc[pb][qb][rq * 4 + j], c1, -mo));
+              const float z = acc[pb][qb][rq * 4 + j] * a.scale;
+              s += j < mine ? e : 0.f;
+              pz = j < mine ? fmaf(e, z, pz) : pz;
+              sq = j < mine ? fmaf(z, z, sq) : sq;
+            }
+          }
       pz += __shfl_xor(pz, 32);
       sq += __shfl_xor(sq, 32);
     } else {
 #pragma unroll
       for (int pb = 0; pb < kNB; ++pb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s += fast_exp2(fmaf(acc[pb][qb][r], c1, -mo));
+        for (int rq = 0; rq < 4; ++rq)
+          if (!VTAIL || pb * 4 + rq < nq) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s += fast_exp2(fmaf(acc[pb][qb][rq * 4 + j], c1, -mo));
+          } else if (pb * 4 + rq == nq && cut != 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float e = fast_exp2(fmaf(acc[pb][qb][rq * 4 + j], c1, -mo));
+              s += j < mine ? e : 0.f;
+            }
+          }
     }
     s += __shfl_xor(s, 32);
     if (lane < 32) {
-      const int64_t o = slice * a.N + tok;
       a.part_lse[o] = m + fast_log(s);
       if (a.monitoring) {
         a.part_max[o] = m;
@@ -90,7 +137,6 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, i
         a.part_sq[o] = sq;
       }
     }
-    const int yl = ycol[qb];
     if (yl >= 0 && ((yl >> 2) & 1) == (lane >> 5)) {
       const int want_pb = yl >> 5, want_r = ((yl >> 3) & 3) * 4 + (yl & 3);
       float zt = 0.f;
@@ -104,31 +150,42 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, i
   }
 }
 
-// Persistent workgroups, operand stream pipelined across output tiles.
-template <class T, class XSrc, class WSrc> struct FwdProblem {
+// Persistent workgroups, operand stream pipelined across output tiles.  The
+// launch covers `tiles_p` tile columns of the vocabulary starting at column
+// tile `tp0` (all full columns, or the one straddling V for the VTAIL variant).
+template <class T, class XSrc, class WSrc, bool VTAIL> struct FwdProblem {
   const FwdArgs& a;
-  int tiles_p, tiles_q;
-  LCE_DEV FwdProblem(const FwdArgs& a_) : a(a_), tiles_p((int)(a_.V / kTile)), tiles_q((int)(a_.N / kTile)) {}
+  int tp0, tiles_p, tiles_q;
+  LCE_DEV FwdProblem(const FwdArgs& a_)
+      : a(a_), tp0(VTAIL ? (int)(a_.V / kTile) : 0), tiles_p(VTAIL ? 1 : (int)(a_.V / kTile)),
+        tiles_q((int)(a_.Np / kTile)) {}
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
+  LCE_DEV void coords(int tile, int& tp, int& tq) const {
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
+    tp += tp0;
+  }
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
+    coords(tile, tp, tq);
     p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile;
     q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
   }
+  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.V); }
+  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
+  LCE_DEV int k_valid() const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
-    fwd_epilogue<T>(a, acc, tp, tq);
+    coords(tile, tp, tq);
+    fwd_epilogue<T, VTAIL>(a, acc, tp, tq);
   }
 };
 
-template <class T, class XSrc, class WSrc>
+template <class T, class XSrc, class WSrc, bool VTAIL>
 __global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  FwdProblem<T, XSrc, WSrc> prob(a);
-  Pipe3<T, WSrc, false, XSrc, true, FwdProblem<T, XSrc, WSrc>> pipe(prob);
-  pipe.run(a.ldw, a.ldx, (int)(a.H / kBK), lds);
+  FwdProblem<T, XSrc, WSrc, VTAIL> prob(a);
+  Pipe3<T, WSrc, false, XSrc, true, FwdProblem<T, XSrc, WSrc, VTAIL>> pipe(prob);
+  pipe.run(a.ldw, a.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
 // One workgroup = 64 tokens x 4 strided groups of slices.
@@ -137,12 +194,14 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
   __shared__ float sh_pz[4][kMergeRows], sh_sq[4][kMergeRows], sh_mx[4][kMergeRows];
   __shared__ double sh_red[6][kMergeRows];
   const int r = threadIdx.x & 63, g = threadIdx.x >> 6;
-  const int64_t tok = (int64_t)blockIdx.x * kMergeRows + r;
-  const int nslices = (int)(a.V / kChunkV);
+  const int64_t tok = (int64_t)blockIdx.x * kMergeRows + r;  // < Np; rows >= N only keep the block sums aligned
+  const bool exists = tok < a.N;
+  const int nslices = (int)(a.Vp / kChunkV);
 
   float M = -INFINITY, S = 0.f;
   for (int c = g; c < nslices; c += 4) {
-    const float l = a.part_lse[(int64_t)c * a.N + tok];
+    const float l = a.part_lse[(int64_t)c * a.Np + tok];
+    if (l == -INFINITY) continue;  // a slice without a single valid column
     const float Mn = fmaxf(M, l);
     S = S * fast_exp2((M - Mn) * kLog2e) + fast_exp2((l - Mn) * kLog2e);
     M = Mn;
@@ -154,17 +213,18 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
     float Mt = fmaxf(fmaxf(sh_m[0][r], sh_m[1][r]), fmaxf(sh_m[2][r], sh_m[3][r]));
     float St = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) St += sh_s[i][r] * fast_exp2((sh_m[i][r] - Mt) * kLog2e);
+    for (int i = 0; i < 4; ++i)
+      if (sh_s[i][r] != 0.f) St += sh_s[i][r] * fast_exp2((sh_m[i][r] - Mt) * kLog2e);
     const float lse = Mt + fast_log(St);
     sh_lse[r] = lse;
-    a.lse[tok] = lse;
+    if (exists) a.lse[tok] = lse;
   }
   __syncthreads();
   const float lse = sh_lse[r];
   if (a.monitoring) {
     float pz = 0.f, sq = 0.f, mx = -INFINITY;
     for (int c = g; c < nslices; c += 4) {
-      const int64_t o = (int64_t)c * a.N + tok;
+      const int64_t o = (int64_t)c * a.Np + tok;
       pz = fmaf(a.part_pz[o], fast_exp2((a.part_lse[o] - lse) * kLog2e), pz);
       sq += a.part_sq[o];
       mx = fmaxf(mx, a.part_max[o]);
@@ -175,10 +235,10 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
   }
   __syncthreads();
   if (g == 0) {
-    const bool valid = a.y[tok] != a.ignore_index;
+    const bool valid = exists && a.y[tok] != a.ignore_index;
     const double l = (double)lse;
     double ent = 0.0, nrm = 0.0, mx = -INFINITY;
-    if (a.monitoring) {
+    if (a.monitoring && exists) {
       const float pz = (sh_pz[0][r] + sh_pz[1][r]) + (sh_pz[2][r] + sh_pz[3][r]);
       const float sq = (sh_sq[0][r] + sh_sq[1][r]) + (sh_sq[2][r] + sh_sq[3][r]);
       mx = (double)fmaxf(fmaxf(sh_mx[0][r], sh_mx[1][r]), fmaxf(sh_mx[2][r], sh_mx[3][r]));
@@ -203,7 +263,7 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
 
 __global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
   __shared__ double sh[6][256];
-  const int nblk = (int)(a.N / kMergeRows);
+  const int nblk = (int)(a.Np / kMergeRows);
   const double* blk = reinterpret_cast<const double*>(a.blk);
   double v[6] = {0, 0, 0, 0, -INFINITY, 0};
   for (int b = threadIdx.x; b < nblk; b += 256) {
@@ -244,15 +304,25 @@ __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
   for (; i < n; i += stride) p[i] = v;
 }
 
-template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
-  auto kern = fwd_tiles_persistent_kernel<T, XSrc, WSrc>;
+template <class T, class XSrc, class WSrc, bool VTAIL> hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
+  auto kern = fwd_tiles_persistent_kernel<T, XSrc, WSrc, VTAIL>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
-  const int64_t tiles = (a.V / kTile) * (a.N / kTile);
   const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
   return hipGetLastError();
+}
+
+// All full tile columns of the vocabulary, then the column that straddles V.
+template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
+  const int64_t tq = a.Np / kTile, full = a.V / kTile;
+  if (full > 0) {
+    hipError_t e = launch_one<T, XSrc, WSrc, false>(a, full * tq, s);
+    if (e != hipSuccess) return e;
+  }
+  if (a.V % kTile) return launch_one<T, XSrc, WSrc, true>(a, tq, s);
+  return hipSuccess;
 }
 
 }  // namespace
@@ -269,7 +339,7 @@ hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
 }
 
 hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s) {
-  hipLaunchKernelGGL(fwd_rows_kernel, dim3((unsigned)(a.N / kMergeRows)), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(fwd_rows_kernel, dim3((unsigned)(a.Np / kMergeRows)), dim3(256), 0, s, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(fwd_final_kernel, dim3(1), dim3(256), 0, s, a);

@@ -49,8 +49,11 @@ template <class T, class SrcT, bool KC> struct Stager3 {
   static constexpr int kEs = (int)sizeof(SrcT);
   typedef StageRegs<kWide> Regs;
   const char* base;      // uniform: first byte of the K tile being loaded
-  unsigned range;        // uniform: 0x7fffffff, or 0 when the stream has run off the last tile
+  const char* end;       // uniform: one past the last valid byte of the operand (loads beyond return 0)
+  unsigned range;        // uniform: bytes from `base` to `end`, clamped to [0, 2^31)
   unsigned voff;         // per-thread byte offset of its first chunk
+  unsigned voff_cur;     // voff, or an always-out-of-range offset when this thread's k lies past the K extent
+  int kpos;              // KC only: first k (element index inside a K tile) this thread loads
   unsigned iter_stride;  // uniform: bytes between this thread's consecutive chunks
   int64_t k_stride;      // bytes between consecutive K tiles
   int lds_off;           // per-thread byte offset of chunk 0 inside the operand tile
@@ -64,6 +67,7 @@ template <class T, class SrcT, bool KC> struct Stager3 {
       k_stride = kBK * kEs;
       const int sw = (r & 7) ^ ((r >> 3) & 1);
       lds_off = r * 128 + ((c ^ sw) << 4);
+      kpos = c * 8;
     } else {
       const int c = t & 31, k = t >> 5;
       voff = (unsigned)(((int64_t)k * ld + c * 8) * kEs);
@@ -72,20 +76,41 @@ template <class T, class SrcT, bool KC> struct Stager3 {
       const int j = k & 3;
       const int mask = ((j & 1) << 7) | ((j >> 1) << 6) | ((j & 1) << 5);
       lds_off = k * 512 + ((c << 4) ^ mask);
+      kpos = 0;
     }
+    voff_cur = voff;
+    base = end = nullptr;
+    range = 0;
+  }
+  // Called whenever `base` moves.  `k_rem` = valid k elements from the start of
+  // this K tile on.  Along K a K-contiguous operand runs on into the next row, so
+  // its threads past the K extent are switched to an out-of-range offset; a
+  // row-contiguous operand has K as its slow index and simply runs off `end`.
+  LCE_DEV void retarget(int k_rem) {
+    // clamp(end - base, 0, 2^31 - 1), on 32-bit halves so that it stays on the scalar unit
+    const int64_t left = end - base;
+    int hi = (int)(left >> 32);
+    unsigned lo = (unsigned)left;
+    asm("" : "+s"(hi), "+s"(lo));  // keeps the compiler from fusing the halves back into 64-bit vector compares
+    const unsigned low = lo < 0x7fffffffu ? lo : 0x7fffffffu;
+    const unsigned capped = hi != 0 ? 0x7fffffffu : low;
+    range = hi < 0 ? 0u : capped;
+    if (KC) voff_cur = kpos < k_rem ? voff : 0x80000000u;
   }
   LCE_DEV void load(Regs& r, int i0, int i1) const {
-    // 0x00020000: raw 32-bit data format.  range == 0 turns every load into a
-    // zero-filling no-op (used once the stream is past the last output tile).
+    // 0x00020000: raw 32-bit data format.  The hardware returns 0 for every
+    // dword at or beyond `range` bytes (voffset + soffset are both checked), which
+    // zero-fills rows past the end of the operand and, with range == 0, turns
+    // every load into a no-op once the stream is past the last output tile.
     const __amdgpu_buffer_rsrc_t rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, (int)range, 0x00020000);
 #pragma unroll
     for (int i = i0; i < i1; ++i) {
       if (kWide) {
-        r.v[2 * i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, (int)(i * iter_stride), 0);
-        r.v[2 * i + 1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff + 16, (int)(i * iter_stride), 0);
+        r.v[2 * i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff_cur, (int)(i * iter_stride), 0);
+        r.v[2 * i + 1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff_cur + 16, (int)(i * iter_stride), 0);
       } else {
-        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, (int)(i * iter_stride), 0);
+        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff_cur, (int)(i * iter_stride), 0);
       }
     }
   }
@@ -108,11 +133,24 @@ template <class T, class SrcT, bool KC> struct Stager3 {
   }
 };
 
+// One past the last byte the loads of a row-major matrix may touch.  The range
+// check of a buffer load works on whole dwords, so for 16-bit elements the last
+// row is taken to end on a dword boundary: with an odd row length the element
+// after the last one is read (it lies in the stride padding, must be finite and
+// never reaches a valid output).
+template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows, int64_t ld, int64_t cols) {
+  const int64_t c = sizeof(S) == 2 ? (cols + 1) & ~(int64_t)1 : cols;
+  return reinterpret_cast<const S*>(base) + (rows - 1) * ld + c;
+}
+
 // What a kernel plugs into the persistent loop.
 //   int  num_tiles()                              output tiles in this launch
 //   void origins(int tile, const void*& p, const void*& q)
 //        first element of the P / Q operand of that output tile:
 //        (row0, k=0) for a KC operand, (k=0, col0) for an MC operand
+//   const void* p_end(), q_end()                  one past the last valid byte of each operand
+//   int  k_valid()                                K extent; the K tiles of the loop may run past
+//        it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
 //   void epilogue(int tile, acc, char* scratch)
 //        consumes the finished accumulator; may use `scratch`, 96 KiB of LDS
 //        that the pipeline does not touch until the next barrier it issues
@@ -134,6 +172,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
   Problem& prob;
   int ktiles;
   int load_tile;  // output tile the fetch stream is in
+  int k_rem;      // valid k elements left from the K tile the stream points at
 
   static constexpr int kPReads = P_KC ? 4 : 8;  // LDS read instructions per k-step
   static constexpr int kQReads = Q_KC ? 4 : 8;
@@ -148,14 +187,22 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
       prob.origins(tile, p, q);
       ps.base = reinterpret_cast<const char*>(p);
       qs.base = reinterpret_cast<const char*>(q);
-      ps.range = qs.range = 0x7fffffffu;
+      ps.end = reinterpret_cast<const char*>(prob.p_end());
+      qs.end = reinterpret_cast<const char*>(prob.q_end());
     } else {
-      ps.range = qs.range = 0;
+      ps.end = ps.base;  // nothing left to fetch: every load returns 0
+      qs.end = qs.base;
     }
+    k_rem = prob.k_valid();
+    ps.retarget(k_rem);
+    qs.retarget(k_rem);
   }
   LCE_DEV void stream_advance() {
     ps.base += ps.k_stride;
     qs.base += qs.k_stride;
+    k_rem -= kBK;
+    ps.retarget(k_rem);
+    qs.retarget(k_rem);
   }
   // chunks 0..7 of a staged K tile belong to P, 8..15 to Q
   LCE_DEV void store_chunks(const PRegs& sp, const QRegs& sq, char* stage, int c0, int c1) {
@@ -248,13 +295,15 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
       if (i < 5) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);  // chunks 11..15: Q
     }
     __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    if (!LAST) read_frags(0, nxt, 0);
+    // The fetch stream moves on to K tile t+3 (first needed by the next step's loads).  Its scalar
+    // address / range arithmetic sits in this region so that it issues between the MFMAs below.
     if (WRAP) {
       stream_begin(load_tile + (int)gridDim.x);
     } else {
       stream_advance();
     }
-    __syncthreads();
-    if (!LAST) read_frags(0, nxt, 0);
     mfma_rows<false>(acc, 1, kNB / 2, kNB);
     if (!LAST) {
 #pragma unroll

@@ -14,11 +14,23 @@ constexpr int kChunkV = 128;
 // Rows handled by one workgroup of the row-merge kernel.
 constexpr int kMergeRows = 64;
 
+// Shapes need not be multiples of the tile sizes: the kernels work on the padded
+// extents below, operand loads past the real extents return zero (buffer range
+// checks and a K mask), and the epilogues neither use logits of columns >= V nor
+// store anything for rows >= N, columns >= V or hidden indices >= H.
+constexpr int64_t pad_to(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+constexpr int64_t padded_tokens(int64_t N) { return pad_to(N, 256); }   // token tiles; K tiles of the dW contraction
+constexpr int64_t padded_vocab(int64_t V) { return pad_to(V, 256); }    // vocabulary tiles
+constexpr int64_t padded_hidden(int64_t H) { return pad_to(H, 256); }   // hidden tiles of dx and dW
+// K extent of the logit contraction: an even number of 64-wide K tiles, at least four
+constexpr int64_t padded_k(int64_t H) { return pad_to(H, 128) < 256 ? 256 : pad_to(H, 128); }
+
 struct FwdArgs {
   const void* x;
   const void* w;
   const int64_t* y;
   int64_t N, H, V, ldx, ldw;
+  int64_t Np, Vp;  // padded_tokens(N), padded_vocab(V)
   int x_dtype, w_dtype;  // compute type = x_dtype (bf16 / f16)
   int64_t ignore_index;
   float scale, z_reg;
@@ -28,12 +40,12 @@ struct FwdArgs {
   float* lse;        // [N]
   float* out5;       // [5]
   int64_t* n_valid;  // [1]
-  float* part_lse;   // [V/128][N]  per-slice logsumexp
-  float* part_max;   // [V/128][N]  per-slice max            (monitoring)
-  float* part_pz;    // [V/128][N]  per-slice sum softmax*z  (monitoring)
-  float* part_sq;    // [V/128][N]  per-slice sum z^2        (monitoring)
-  float* tgt;        // [N]         target logit, pre-zeroed
-  float* blk;        // [N/64][8]   per-merge-block partial sums
+  float* part_lse;   // [Vp/128][Np]  per-slice logsumexp (-inf for a slice with no valid column)
+  float* part_max;   // [Vp/128][Np]  per-slice max            (monitoring)
+  float* part_pz;    // [Vp/128][Np]  per-slice sum softmax*z  (monitoring)
+  float* part_sq;    // [Vp/128][Np]  per-slice sum z^2        (monitoring)
+  float* tgt;        // [Np]          target logit, pre-zeroed
+  float* blk;        // [Np/64][8]    per-merge-block partial sums
 };
 
 struct BwdArgs {
@@ -44,15 +56,17 @@ struct BwdArgs {
   const int64_t* n_valid;
   const float* grad_out;
   int64_t N, H, V, ldx, ldw, lddx, lddw;
+  int64_t Np, Hp;  // padded_tokens(N), padded_hidden(H)
   int x_dtype, w_dtype, dx_dtype, dw_dtype;
   int64_t ignore_index;
   float scale, z_reg;
   void* dx;
   void* dw;
   // slab being processed
-  int64_t v0, vs;   // first column and width of the vocabulary slab
-  void* dz;         // [N][vs] staged dz in the compute type
-  float* dx_acc;    // [N][H] fp32 running dx (null when there is a single slab)
+  int64_t v0, vs;   // first column and padded width (multiple of 256) of the vocabulary slab
+  int64_t vw;       // columns of the slab that exist: min(vs, V - v0)
+  void* dz;         // [Np][vs] staged dz in the compute type (exact zeros outside N x vw)
+  float* dx_acc;    // [Np][Hp] fp32 running dx (null when there is a single slab)
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
 };

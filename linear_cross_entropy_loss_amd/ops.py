@@ -34,6 +34,33 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
 
+def _row_multiple(dtype):
+    """Row strides must keep rows 16-byte aligned: 8 elements for 16-bit data, 4 for float32."""
+    return 4 if dtype == torch.float32 else 8
+
+
+def _aligned_rows(t):
+    """`t` itself when the kernels can read it in place, else a copy whose row stride is padded with zeros.
+
+    The kernels take any number of rows and columns, but rows must start on 16-byte boundaries.  Only a
+    matrix whose row length is not a multiple of 8 (16-bit) / 4 (fp32) elements AND is stored densely needs
+    the copy; padding the vocabulary or hidden size of the model to a multiple of 8 avoids it.
+    """
+    m = _row_multiple(t.dtype)
+    if t.stride(-1) == 1 and t.stride(0) % m == 0 and t.stride(0) >= t.shape[1] and t.data_ptr() % 16 == 0:
+        return t
+    rows, cols = t.shape
+    padded = torch.zeros((rows, -(-cols // m) * m), dtype=t.dtype, device=t.device)
+    padded[:, :cols] = t
+    return padded[:, :cols]
+
+
+def _empty_rows(rows, cols, dtype, device):
+    """Uninitialised (rows, cols) matrix whose row stride satisfies the kernels' alignment rule."""
+    m = 8  # gradients are stored in pieces of up to 8 elements
+    return torch.empty((rows, -(-cols // m) * m), dtype=dtype, device=device)[:, :cols]
+
+
 def _check_inputs(x, y, At):
     if not (x.is_cuda and y.is_cuda and At.is_cuda):
         raise RuntimeError(
@@ -66,11 +93,9 @@ class LinearXentImplementation(torch.autograd.Function):
         if torch.is_autocast_enabled("cuda") and x_in.dtype == torch.float32:
             x_in = x_in.to(torch.get_autocast_dtype("cuda"))
         with torch.cuda.device(x_in.device):
-            x = x_in.reshape(-1, x_in.shape[-1])
-            if x.stride(-1) != 1:
-                x = x.contiguous()
+            x = _aligned_rows(x_in.reshape(-1, x_in.shape[-1]))
             y1 = y.reshape(-1).contiguous()
-            w = At if At.stride(-1) == 1 else At.contiguous()
+            w = _aligned_rows(At)
             N, H = x.shape
             H_A, V = w.shape
             if H_A != H:
@@ -78,7 +103,7 @@ class LinearXentImplementation(torch.autograd.Function):
             if y1.shape != (N,):
                 raise ValueError("labels must have one entry per input row")
             prob = _lib.make_problem(
-                N, H, V, x.stride(0), w.stride(0), H, V, x.dtype, w.dtype, x.dtype, w.dtype,
+                N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
                 ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring,
             )
             lib = _lib.load()
@@ -111,11 +136,12 @@ class LinearXentImplementation(torch.autograd.Function):
         V = w.shape[1]
         with torch.cuda.device(x.device):
             dev = x.device
-            dx = torch.empty((N, H), dtype=x.dtype, device=dev) if need_dx else None
-            dw = torch.empty((H, V), dtype=w.dtype, device=dev) if need_dw else None
+            dx = _empty_rows(N, H, x.dtype, dev) if need_dx else None
+            dw = _empty_rows(H, V, w.dtype, dev) if need_dw else None
             if need_dx or need_dw:
                 prob = _lib.make_problem(
-                    N, H, V, x.stride(0), w.stride(0), H, V, x.dtype, w.dtype, x.dtype, w.dtype,
+                    N, H, V, x.stride(0), w.stride(0), dx.stride(0) if need_dx else H + (-H) % 8,
+                    dw.stride(0) if need_dw else V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
                     ignore_index, logit_scale, z_regularization, N_chunk_size, False,
                 )
                 lib = _lib.load()
@@ -128,7 +154,9 @@ class LinearXentImplementation(torch.autograd.Function):
                 _lib.raise_for_status(rc, "lce_backward")
                 del ws
         if dx is not None:
-            dx = dx.view(ctx.x_shape)
+            dx = dx.reshape(ctx.x_shape)  # a copy only when H is not a multiple of 8
+        if dw is not None and not dw.is_contiguous():
+            dw = dw.contiguous()  # V not a multiple of 8
         return dx, None, dw, None, None, None, None, None
 
 
@@ -155,13 +183,15 @@ class LinearCrossEntropyLoss(torch.nn.Linear):
     weight is stored transposed, ``(in_features, out_features)``, and there is no bias.
 
     Args:
-        in_features: hidden size (multiple of 256).
-        out_features: vocabulary size / number of classes (multiple of 4096).
+        in_features: hidden size (any; multiples of 8 avoid a padded copy of the input).
+        out_features: vocabulary size / number of classes (any; multiples of 8 avoid a padded copy of
+            the weight and of its gradient).  The reference requires multiples of 256 / 4096
+            (``ops.py:905-906``); those restrictions are lifted here.
         ignore_index: label value that is skipped. Default -100.
         logit_scale: positive factor applied to the logits before the loss. Default 1.0.
         z_regularization: weight of the ``mean(logsumexp(z)^2)`` penalty. Default 0.0.
         N_chunk_size: bounds the scratch memory of a call to ``N_chunk_size * out_features * 4`` bytes
-            (multiple of 512; the number of rows of ``x`` must be a multiple of 512). Default 4096.
+            (the number of rows of ``x`` is free). Default 4096.
         init_method: optional callable applied to the weight instead of the default truncated normal.
 
     Set ``module.monitoring = True`` to also collect ``logit_norm``, ``logit_max``, ``logit_entropy`` and
@@ -183,9 +213,7 @@ class LinearCrossEntropyLoss(torch.nn.Linear):
         factory_kwargs = {"device": device, "dtype": dtype}
         torch.nn.Module.__init__(self)
 
-        assert in_features % 256 == 0
-        assert out_features % 4096 == 0
-        assert N_chunk_size % 512 == 0
+        assert in_features > 0 and out_features > 0 and N_chunk_size > 0
         assert logit_scale > 0
         assert z_regularization >= 0
 

@@ -1,0 +1,245 @@
+"""Sweep harness writing CSV files with the reference's schema.
+
+The reference publishes its results as CSV files written by `bench_fusions.py`
+(one per precision mode and swept variable, under `bench/`, `bench-mem/` and
+`bench-acc/`): first column the swept variable, one column per provider.  This
+module runs the same three protocols on one MI355X and writes files with the
+same names, the same first column, the same units and the same FLOP convention
+for the speed files (`3 * (2*N*H*V + 3*N*V)` for fwd+bwd, bench_fusions.py:287-291),
+so that a curve from here can be laid over the reference's curve.
+
+  speed   fwd+bwd TFLOP/s, median of event timings      bench_fusions.py:210-297
+  mem     peak GiB beyond the inputs                    bench_fusions.py:304-394
+  acc     torch.dist to an fp64 evaluation              bench_fusions.py:399-519
+
+Providers: `torch-baseline` (eager `F.linear` + `F.cross_entropy` on the GPU, the
+reference's first column, bench_fusions.py:31-33) and `hip-gfx950` (this
+package).  A point a provider cannot run is left empty, as in the reference's
+files.  Sweep ranges are the reference's: H 2^8..2^13, V 2^8..2^17, N 2^8..2^16
+(bench_fusions.py:113; accuracy N up to 2^15, bench_fusions.py:446).
+
+Usage:  python -m linear_cross_entropy_loss_amd.sweep --out DIR
+            [--kind speed mem acc] [--acc bf16 fp16 fp16-mixed] [--vars N V H] [--quick]
+"""
+from __future__ import annotations
+
+import argparse
+import math
+import os
+import sys
+
+DEFAULTS = dict(N=16384, H=2048, V=131072)
+RANGES = {"H": range(8, 14), "V": range(8, 18), "N": range(8, 17)}
+ACC_RANGES = {"H": range(8, 14), "V": range(8, 18), "N": range(8, 16)}
+PROVIDERS = ["torch-baseline", "hip-gfx950"]
+TITLE_DEFAULTS = "Defaults: N=B*S=16384, H=2048, V=131072"
+# The eager baseline materialises N x V fp32 logits and their gradient; skip it beyond this many elements.
+BASELINE_MAX_LOGITS = 65536 * 131072
+
+
+def _dtype(torch, acc):
+    return {"fp16": torch.float16, "bf16": torch.bfloat16}.get(acc, torch.float32)
+
+
+def _inputs(torch, N, H, V, acc, low_loss=False, seed=0):
+    """Inputs of the reference's sweeps: A ~ randn(V, H), y uniform, x ~ randn (or 0.1*A[y] + randn for accuracy)."""
+    dt = _dtype(torch, acc)
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    y = torch.randint(0, V, (N,), device="cuda", generator=g)
+    A = torch.randn(V, H, device="cuda", generator=g).to(dt)
+    if low_loss:
+        x = (0.1 * A[y].float() + torch.randn(N, H, device="cuda", generator=g)).to(dt)
+    else:
+        x = torch.randn(N, H, device="cuda", generator=g).to(dt)
+    At = A.T.contiguous()
+    return x.requires_grad_(), y, A.requires_grad_(), At.requires_grad_()
+
+
+def _make_fn(torch, provider, x, y, A, At, acc):
+    import torch.nn.functional as F
+
+    mixed = "mixed" in acc
+    amp_dtype = torch.bfloat16 if "bf16" in acc else torch.float16
+    if provider == "torch-baseline":
+        def loss_fn():
+            return F.cross_entropy(F.linear(x, A).float(), y)
+        grads = (x, A)
+    else:
+        from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+        def loss_fn():
+            return linear_cross_entropy(x, y, At)[0]
+        grads = (x, At)
+
+    def step():
+        for t in grads:
+            t.grad = None
+        with torch.autocast("cuda", dtype=amp_dtype, enabled=mixed):
+            loss = loss_fn()
+        loss.backward()
+        return loss
+
+    return step, grads
+
+
+def _median_ms(torch, step, warmup, reps):
+    cache = torch.empty(256 << 20, dtype=torch.int8, device="cuda")  # flushed before every repetition
+    for _ in range(warmup):
+        step()
+    ts = []
+    for _ in range(reps):
+        cache.zero_()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        step()
+        e.record()
+        torch.cuda.synchronize()
+        ts.append(s.elapsed_time(e))
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def _skip_baseline(provider, N, V):
+    return provider == "torch-baseline" and N * V > BASELINE_MAX_LOGITS
+
+
+def point_speed(torch, provider, N, H, V, acc, quick):
+    if _skip_baseline(provider, N, V):
+        return float("nan")
+    x, y, A, At = _inputs(torch, N, H, V, acc)
+    step, _ = _make_fn(torch, provider, x, y, A, At, acc)
+    ms = _median_ms(torch, step, 2 if quick else 5, 5 if quick else 20)
+    flop = 3 * (2 * N * H * V + 3 * N * V)
+    return flop * 1e-12 / (ms * 1e-3)
+
+
+def point_mem(torch, provider, N, H, V, acc, quick):
+    if _skip_baseline(provider, N, V):
+        return float("nan")
+    x, y, A, At = _inputs(torch, N, H, V, acc)
+    if provider == "torch-baseline":
+        del At
+        At = None
+    else:
+        A = A.detach()
+    step, grads = _make_fn(torch, provider, x, y, A, At, acc)
+    step()  # warm-up (allocator pools, lazy initialisation)
+    for t in grads:
+        t.grad = None
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    initial = torch.cuda.memory_allocated()
+    step()
+    torch.cuda.synchronize()
+    return (torch.cuda.max_memory_allocated() - initial) / 1024**3
+
+
+def _fp64_reference(torch, x, y, A, chunk=512):
+    """Loss and gradients in fp64, row-chunked (the reference's torch_checkpoint in double, bench_fusions.py:408)."""
+    import torch.nn.functional as F
+
+    N = x.shape[0]
+    Ad = A.detach().double().requires_grad_()
+    dx = torch.empty(x.shape, dtype=torch.float64, device=x.device)
+    loss = torch.zeros((), dtype=torch.float64, device=x.device)
+    for i in range(0, N, chunk):
+        xb = x[i:i + chunk].detach().double().requires_grad_()
+        part = F.cross_entropy(F.linear(xb, Ad), y[i:i + chunk], reduction="sum") / N
+        part.backward()
+        dx[i:i + chunk] = xb.grad
+        loss += part.detach()
+    return loss.float(), Ad.grad.float(), dx.float()
+
+
+def point_acc(torch, provider, N, H, V, acc, mode):
+    if _skip_baseline(provider, N, V):
+        return float("nan")
+    x, y, A, At = _inputs(torch, N, H, V, acc, low_loss=True, seed=1)
+    ref_loss, ref_dA, ref_dx = _fp64_reference(torch, x, y, A)
+    step, grads = _make_fn(torch, provider, x, y, A, At, acc)
+    loss = step()
+    if mode == "fwd":
+        return torch.dist(loss.float(), ref_loss).item()
+    if provider == "torch-baseline":
+        a_err = torch.dist(ref_dA, A.grad.float()).item()
+    else:
+        a_err = torch.dist(ref_dA.T, At.grad.float()).item()
+    x_err = torch.dist(ref_dx, x.grad.float()).item()
+    return 0.5 * (x_err + a_err)
+
+
+def _write_csv(path, var, rows):
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    with open(path, "w") as f:
+        f.write(",".join([var] + PROVIDERS) + "\n")
+        for xval, vals in rows:
+            cells = ["%f" % xval] + ["" if (v is None or math.isnan(v)) else "%f" % v for v in vals]
+            f.write(",".join(cells) + "\n")
+
+
+def run(out, kinds, accs, variables, quick=False, log=print):
+    import torch
+
+    if not torch.cuda.is_available():
+        raise RuntimeError("the sweep needs an AMD GPU")
+    written = []
+    for kind in kinds:
+        modes = ["fwd", "bwd"] if kind == "acc" else ["fwd-bwd"]
+        for mode in modes:
+            for acc in accs:
+                if kind == "acc" and "mixed" in acc:
+                    continue  # the reference's accuracy sweep covers fp16 and bf16 only (bench_fusions.py:448)
+                for var in variables:
+                    rng = (ACC_RANGES if kind == "acc" else RANGES)[var]
+                    xs = [2**i for i in rng]
+                    if quick:
+                        xs = xs[::3]
+                    rows = []
+                    for xv in xs:
+                        shape = dict(DEFAULTS)
+                        shape[var] = xv
+                        vals = []
+                        for prov in PROVIDERS:
+                            try:
+                                torch.cuda.empty_cache()
+                                if kind == "speed":
+                                    v = point_speed(torch, prov, shape["N"], shape["H"], shape["V"], acc, quick)
+                                elif kind == "mem":
+                                    v = point_mem(torch, prov, shape["N"], shape["H"], shape["V"], acc, quick)
+                                else:
+                                    v = point_acc(torch, prov, shape["N"], shape["H"], shape["V"], acc, mode)
+                            except (ValueError, RuntimeError, torch.OutOfMemoryError) as exc:
+                                log(f"  {prov} N={shape['N']} H={shape['H']} V={shape['V']} {acc}: {type(exc).__name__}: "
+                                    f"{str(exc).splitlines()[0][:120]}")
+                                v = float("nan")
+                            vals.append(v)
+                        log(f"{kind} {mode} {acc} {var}={xv}: " + ", ".join(f"{p}={v:.4g}" for p, v in zip(PROVIDERS, vals)))
+                        rows.append((float(xv), vals))
+                    if kind == "speed":
+                        name = f"bench/{acc} {mode}-Linear+Loss Performance over {var}. {TITLE_DEFAULTS}.csv"
+                    elif kind == "mem":
+                        name = f"bench-mem/{acc} {mode}-Linear+Loss Memory Peak over {var}. {TITLE_DEFAULTS}.csv"
+                    else:
+                        name = f"bench-acc/ {mode} {acc} Linear+Loss Accuracy over {var}. {TITLE_DEFAULTS}.csv"
+                    path = os.path.join(out, name)
+                    _write_csv(path, var, rows)
+                    written.append(path)
+    return written
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--out", required=True)
+    ap.add_argument("--kind", nargs="+", default=["speed", "mem", "acc"], choices=["speed", "mem", "acc"])
+    ap.add_argument("--acc", nargs="+", default=["fp16", "bf16", "fp16-mixed"], choices=["fp16", "bf16", "fp16-mixed"])
+    ap.add_argument("--vars", nargs="+", default=["H", "N", "V"], choices=["H", "N", "V"])
+    ap.add_argument("--quick", action="store_true", help="every third point, fewer repetitions")
+    args = ap.parse_args(argv)
+    for p in run(args.out, args.kind, args.acc, args.vars, args.quick, log=lambda m: print(m, flush=True)):
+        print("wrote", p, flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

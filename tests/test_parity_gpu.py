@@ -110,3 +110,96 @@ def test_mid_size_matches_fp64_oracle_evaluated_on_gpu(N, H, V, dtype, w_dtype, 
         print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
         assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
     assert (xd.grad[y == -1] == 0).all()
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Shapes that are not multiples of the tile sizes (the reference refuses them, ops.py:689-691, and names
+# them as an open caveat, README.md:30).  Covers: token / vocabulary / hidden tails, a hidden size below
+# one K loop, sizes that are not multiples of 8 (padded row strides), a single row, several uneven
+# vocabulary slabs, strided inputs, a target in the last valid column, fp32 tensors, fp32 master weight.
+# ---------------------------------------------------------------------------------------------------------
+ODD_CASES = [
+    # N, H, V, dtype, w_dtype, ignore_frac, z_reg, scale, n_chunk, monitoring
+    (1000, 520, 5000, torch.bfloat16, None, 0.05, 0.0, 1.0, 4096, False),
+    (777, 264, 10008, torch.float16, None, 0.1, 1e-4, 0.5, 512, True),
+    (300, 100, 1001, torch.bfloat16, None, 0.1, 1e-3, 1.0, 4096, True),
+    (1, 8, 8, torch.bfloat16, None, 0.0, 0.0, 1.0, 4096, True),
+    (33, 72, 263, torch.float16, None, 0.0, 0.0, 2.0, 16, False),
+    (513, 1024, 4104, torch.float32, None, 0.05, 1e-4, 1.0, 512, True),
+    (640, 328, 3003, torch.float16, torch.float32, 0.1, 0.0, 1.0, 64, False),
+    (2049, 136, 2500, torch.bfloat16, None, 0.3, 0.0, 0.7, 32, True),
+    (257, 101, 515, torch.bfloat16, None, 0.0, 0.0, 1.0, 4096, True),
+    (130, 77, 333, torch.float32, None, 0.1, 1e-3, 1.0, 4096, False),
+]
+
+
+@pytest.mark.parametrize("N,H,V,dtype,w_dtype,ign,z_reg,scale,n_chunk,mon", ODD_CASES)
+def test_arbitrary_shapes_match_oracle(N, H, V, dtype, w_dtype, ign, z_reg, scale, n_chunk, mon):
+    print(f"odd case N={N} H={H} V={V} {dtype} w={w_dtype} ign={ign} zreg={z_reg} scale={scale} chunk={n_chunk}",
+          flush=True)
+    x, y, w = make_inputs(N, H, V, dtype, seed=N + H + V, ignore_frac=ign, w_dtype=w_dtype)
+    y[0] = V - 1  # a target in the last valid column
+    out, dx, dw = _run(x, y, w, -1, z_reg, scale, n_chunk, mon, grad_output=0.9)
+    ref = _oracle(x, y, w, -1, z_reg, scale, grad_output=0.9)
+    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item()), (out[0].item(), ref.loss.item())
+    assert abs(out[1].item() - ref.z_reg.item()) <= LOSS_RTOL * abs(ref.z_reg.item())
+    if mon:
+        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item()) + 1e-3
+        assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item()) + 1e-4
+        assert abs(out[4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item())
+    assert dx.shape == x.shape and dw.shape == w.shape and dx.dtype == x.dtype and dw.dtype == w.dtype
+    for name, got, want in (("dx", dx, ref.dx), ("dw", dw, ref.dw)):
+        emax, el2 = rel_errors(got, want)
+        print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
+        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
+    ignored = (y == -1)
+    if ignored.any():
+        assert (dx.cpu()[ignored] == 0).all()
+
+
+def test_strided_inputs_and_garbage_in_the_stride_padding():
+    """x and W handed over as views with padded row strides whose padding holds large finite garbage: the
+    result must be bit-identical to the dense call (the kernels never let the padding reach a valid output)."""
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    print("strided inputs", flush=True)
+    N, H, V = 700, 200, 3000
+    x, y, w = make_inputs(N, H, V, torch.bfloat16, seed=5, ignore_frac=0.1, device="cuda")
+    xs = torch.full((N, H + 24), 1e30, dtype=x.dtype, device="cuda")
+    ws = torch.full((H, V + 40), -1e30, dtype=w.dtype, device="cuda")
+    xs[:, :H] = x
+    ws[:, :V] = w
+    res = []
+    for xi, wi in ((x, w), (xs[:, :H], ws[:, :V])):
+        xi = xi.detach().requires_grad_(True)
+        wi = wi.detach().requires_grad_(True)
+        out = linear_cross_entropy(xi, y, wi, -1, 1e-4, 1.0, 256, True)
+        out[0].backward()
+        res.append((torch.stack(out).detach(), xi.grad[:, :H].clone(), wi.grad[:, :V].clone()))
+    for a, b in zip(res[0], res[1]):
+        assert torch.equal(a, b)
+
+
+def test_gpt2_vocabulary_matches_fp64_oracle_evaluated_on_gpu():
+    """V = 50257 (not a multiple of 8), H = 768, N = 3000: oracle in fp64 on the GPU."""
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+    from oracle import lce_forward_backward_fp64
+
+    print("gpt2 vocabulary", flush=True)
+    N, H, V = 3000, 768, 50257
+    x, y, w = make_inputs(N, H, V, torch.bfloat16, seed=50257, ignore_frac=0.05, zipf=True, device="cuda")
+    y[1] = V - 1
+    xd = x.clone().requires_grad_(True)
+    wd = w.clone().requires_grad_(True)
+    out = linear_cross_entropy(xd, y, wd, -1, 0.0, 1.0, 1024, True)
+    out[0].backward()
+    ref = lce_forward_backward_fp64(x, y, w, -1, 0.0, 1.0, chunk=512)
+    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item())
+    assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item())
+    for name, got, want in (("dx", xd.grad, ref.dx), ("dw", wd.grad, ref.dw)):
+        d = got.double() - want
+        emax = (d.abs().max() / want.abs().max()).item()
+        el2 = (d.norm() / want.norm()).item()
+        print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
+        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
+    assert (xd.grad[y == -1] == 0).all()

@@ -155,10 +155,15 @@ def test_shape_errors_raise_value_error():
     x = torch.randn(500, 256, device="cuda", dtype=torch.bfloat16)
     w = torch.randn(256, 4096, device="cuda", dtype=torch.bfloat16)
     y = torch.randint(0, 4096, (500,), device="cuda")
+    # the reference's error for an unsupported shape (ops.py:43-44); here only degenerate sizes are unsupported
     with pytest.raises(ValueError, match="Provided shape outside the range of valid configs"):
-        linear_cross_entropy(x, y, w)
+        linear_cross_entropy(x[:0], y[:0], w)
     with pytest.raises(ValueError):
         linear_cross_entropy(torch.randn(512, 256, device="cuda", dtype=torch.bfloat16), y[:12], w)
+    with pytest.raises(ValueError):
+        linear_cross_entropy(x, y, w[:128])            # in_features mismatch
+    with pytest.raises(ValueError):
+        linear_cross_entropy(x, y.to(torch.int32), w)  # labels must be int64
 
 
 def test_autocast_keeps_fp32_master_weight_and_returns_fp32_dw():
