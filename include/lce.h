@@ -14,9 +14,17 @@
  *   - x is (N, H) row-major with row stride ldx; w is the TRANSPOSED weight
  *     (H, V) row-major with row stride ldw (linear_cross_entropy/ops.py:913);
  *     y is N contiguous int64 labels (ops.py:210).
- *   - Supported shapes: N % 512 == 0, H % 256 == 0, V % 4096 == 0,
- *     n_chunk % 512 == 0 -- the reference's own contract (ops.py:689-691,
- *     ops.py:905-907).
+ *   - Shapes: any N, H, V, n_chunk >= 1 (N, V <= 2^30, H <= 2^20).  The
+ *     reference's divisibility rules (N % 512, H % 256, V % 4096,
+ *     ops.py:689-691, 905-907) are lifted; shapes that obey them run at full
+ *     speed, others pay for partly empty tiles.
+ *   - Row strides keep every row 16-byte aligned: ldx, ldw (and lddw for a
+ *     16-bit dW) are multiples of 8 elements for 16-bit data, 4 for fp32; lddx
+ *     is a multiple of 4.  A stride larger than the row length is fine.  When
+ *     the row length is not such a multiple, the elements between the end of a
+ *     row and the next multiple ("stride padding") are read, must be finite,
+ *     and never influence a result; the same positions of dx / dW rows may be
+ *     written.
  *   - Every function returns LCE_OK (0) or a negative lce_status; nothing
  *     throws or aborts.
  */
@@ -38,7 +46,7 @@ typedef enum lce_dtype {
 
 typedef enum lce_status {
   LCE_OK = 0,
-  LCE_EINVAL_SHAPE = -1, /* shape outside the supported set (ops.py:43-44, 689-691) */
+  LCE_EINVAL_SHAPE = -1, /* non-positive or oversized N, H, V, n_chunk (ops.py:43-44)  */
   LCE_EINVAL_DTYPE = -2, /* unsupported dtype combination                            */
   LCE_EINVAL_ARG = -3,   /* null pointer, bad stride, bad scalar                     */
   LCE_EWORKSPACE = -4,   /* workspace missing or smaller than lce_workspace_bytes    */
@@ -101,17 +109,19 @@ int lce_check_problem(const lce_problem* p);
 
 /*
  * Scratch sizes in bytes for lce_forward and lce_backward on problem `p`.
- * The backward size never exceeds n_chunk * V * 4 bytes -- the memory bound
- * the reference documents for N_chunk_size (ops.py:677, 700, 860) -- unless
- * even the smallest staging unit does not fit, in which case
- * LCE_EWORKSPACE is returned.
+ * The backward size stays within n_chunk * V * 4 bytes -- the memory bound the
+ * reference documents for N_chunk_size (ops.py:677, 700, 860) -- whenever the
+ * narrowest split (256-column slabs plus an fp32 running dx) fits in it; for
+ * the remaining shapes (a small vocabulary with many tokens) that narrowest
+ * split is used and its size reported: the bound is a target, not a reason
+ * to refuse a shape the reference runs.
  */
 int lce_workspace_bytes(const lce_problem* p, size_t* fwd_bytes, size_t* bwd_bytes);
 
 /*
  * How lce_backward will split problem `p`: it stages dz for all tokens of one
- * vocabulary slab at a time (`slab_width` columns, `slabs` = V / slab_width
- * passes).  The counterpart of the reference's loop over N_chunk_size-row
+ * vocabulary slab at a time (`slab_width` columns, a multiple of 256; `slabs`
+ * passes, the last one over whatever columns remain).  The counterpart of the reference's loop over N_chunk_size-row
  * groups (ops.py:721), which exists for the same purpose: bounding scratch.
  */
 int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width);

@@ -64,35 +64,52 @@ FwdPlan plan_fwd(const lce_problem* p) {
 
 struct BwdPlan {
   int64_t slabs, vs;
-  size_t dz, dx_acc, total;
+  size_t dz, dx_acc, dx_part, total;
 };
 
+// Bytes of the split-K partial sums of dx for slabs of `vs` columns (0 when dx is not split).
+size_t dx_part_bytes(size_t Np, size_t Hp, int64_t vs) {
+  int split, kseg;
+  lce::dx_split_plan((int64_t)Np, (int64_t)Hp, vs, &split, &kseg);
+  return split > 1 ? align_up((size_t)split * Np * Hp * 4) : 0;
+}
+
 // Fewest vocabulary slabs (of a width that is a multiple of 256 columns; the last
-// one may be narrower) whose staging fits in n_chunk * V * 4 bytes.  The dz stage
-// itself is additionally capped at 1 GiB: wider slabs are not faster, so a
-// generous N_chunk_size does not translate into a larger footprint.  When even
-// the narrowest slab does not fit (small V with many tokens: the fp32 running
-// dx alone exceeds the budget) the narrowest plan is used all the same -- the
-// budget is a target, the operator never refuses a shape because of it.
+// one may be narrower) whose staging fits the scratch bound.  The dz stage itself
+// is additionally capped at 1 GiB: wider slabs are not faster, so a generous
+// N_chunk_size does not translate into a larger footprint.
+//
+// The bound is n_chunk * V * 4 bytes, what the reference spends on its logits
+// chunk (ops.py:700).  Shapes with a small vocabulary and many tokens cannot
+// meet it (the fp32 running dx alone is larger, and a split into very narrow
+// slabs leaves the GPU idle); for those the bound is widened by N * H * 4 bytes,
+// the fp32 x_grad buffer the reference allocates next to its logits chunk
+// (ops.py:693) and this library does not.  If even that fails, the narrowest
+// split is used: the bound is a target, the operator never refuses a shape.
 int plan_bwd(const lce_problem* p, BwdPlan* b) {
-  const size_t budget = (size_t)p->n_chunk * (size_t)p->V * 4;
+  const size_t strict = (size_t)p->n_chunk * (size_t)p->V * 4;
   const size_t dz_cap = (size_t)1 << 30;
   const size_t Np = (size_t)lce::padded_tokens(p->N), Hp = (size_t)lce::padded_hidden(p->H);
   const int64_t Vp = lce::padded_vocab(p->V);
   const int64_t cols = Vp / 256;
-  for (int64_t s = 1; s <= cols; ++s) {
-    const int64_t vs = (cols + s - 1) / s * 256;
-    if (s > 1 && (cols + s - 2) / (s - 1) * 256 == vs) continue;  // same width as with one slab fewer
-    const int64_t slabs = (Vp + vs - 1) / vs;
-    const size_t dz = align_up(Np * (size_t)vs * 2);
-    const size_t acc = slabs > 1 ? align_up(Np * Hp * 4) : 0;
-    if ((dz + acc <= budget && dz <= dz_cap) || vs == 256) {
-      b->slabs = slabs;
-      b->vs = vs;
-      b->dz = 0;
-      b->dx_acc = dz;
-      b->total = dz + acc;
-      return LCE_OK;
+  for (int pass = 0; pass < 2; ++pass) {
+    const size_t budget = strict + (pass ? (size_t)p->N * (size_t)p->H * 4 : 0);
+    for (int64_t s = 1; s <= cols; ++s) {
+      const int64_t vs = (cols + s - 1) / s * 256;
+      if (s > 1 && (cols + s - 2) / (s - 1) * 256 == vs) continue;  // same width as with one slab fewer
+      const int64_t slabs = (Vp + vs - 1) / vs;
+      const size_t dz = align_up(Np * (size_t)vs * 2);
+      const size_t acc = slabs > 1 ? align_up(Np * Hp * 4) : 0;
+      const size_t part = dx_part_bytes(Np, Hp, vs);  // at most 64 MiB
+      if ((dz + acc + part <= budget && (dz <= dz_cap || vs == 256)) || (pass == 1 && vs == 256)) {
+        b->slabs = slabs;
+        b->vs = vs;
+        b->dz = 0;
+        b->dx_acc = dz;
+        b->dx_part = dz + acc;
+        b->total = dz + acc + part;
+        return LCE_OK;
+      }
     }
   }
   return LCE_EWORKSPACE;
@@ -233,6 +250,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.dx = dx; a.dw = dw;
   a.dz = base + b.dz;
   a.dx_acc = b.slabs > 1 ? (float*)(base + b.dx_acc) : nullptr;
+  a.dx_part = (float*)(base + b.dx_part);
   rc = current_num_cus(&a.num_cus);
   if (rc != LCE_OK) return rc;
   const int ph = p->phases ? p->phases : ~0;
@@ -241,6 +259,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     a.v0 = i * b.vs;
     a.vw = p->V - a.v0 < b.vs ? p->V - a.v0 : b.vs;   // columns of this slab that exist
     a.vs = lce::pad_to(a.vw, 256);                    // its padded width: dz row stride and K extent of dx
+    lce::dx_split_plan(a.Np, a.Hp, a.vs, &a.dx_split, &a.dx_kseg);
     a.first = i == 0;
     a.last = i == b.slabs - 1;
     hipError_t e;

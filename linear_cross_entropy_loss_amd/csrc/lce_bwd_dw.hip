@@ -79,7 +79,7 @@ template <class T, class XSrc> struct DwProblem {
   }
   LCE_DEV const void* p_end() const { return reinterpret_cast<const E*>(a.dz) + a.Np * a.vs; }
   LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
-  LCE_DEV int k_valid() const { return (int)a.Np; }
+  LCE_DEV int k_valid(int) const { return (int)a.Np; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 4, tp, tq);

@@ -69,45 +69,125 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
   }
 }
 
-template <class T, class WSrc> struct DxProblem {
+// Split mode: the raw fp32 partial sum of K segment `seg` goes to dx_part[seg][Np][Hp].
+LCE_DEV void dx_partial_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, int seg) {
+  const int64_t h0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wp = wave & 1, wq = wave >> 1;
+  float* part = a.dx_part + (int64_t)seg * a.Np * a.Hp;
+#pragma unroll
+  for (int qb = 0; qb < kNB; ++qb) {
+    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+#pragma unroll
+    for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int64_t h = h0 + wp * kWaveTile + pb * kBlk + 8 * rq + 4 * (lane >> 5);
+        f32x4_t v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = acc[pb][qb][rq * 4 + j];
+        *reinterpret_cast<f32x4_t*>(part + tok * a.Hp + h) = v;
+      }
+  }
+}
+
+// Work item = (output tile, K segment); segment fastest, so that with a
+// power-of-two split the workgroups of one XCD work on the same segment and
+// share its W rows and dz columns in their L2.
+template <class T, class WSrc, bool SPLIT> struct DxProblem {
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
-  int tiles_p, tiles_q;
-  LCE_DEV DxProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.Hp / kTile)), tiles_q((int)(a_.Np / kTile)) {}
-  LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
-  LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
-    int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
-    p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0;
-    q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs;
+  int tiles_p, tiles_q, split, kseg;
+  LCE_DEV DxProblem(const BwdArgs& a_)
+      : a(a_), tiles_p((int)(a_.Hp / kTile)), tiles_q((int)(a_.Np / kTile)), split(SPLIT ? a_.dx_split : 1),
+        kseg(a_.dx_kseg) {}
+  LCE_DEV int num_tiles() const { return tiles_p * tiles_q * split; }
+  LCE_DEV void decode(int item, int& tp, int& tq, int& seg) const {
+    seg = SPLIT ? item % split : 0;
+    tile_coords(SPLIT ? item / split : item, tiles_p * tiles_q, tiles_p, tiles_q, 8, tp, tq);
+  }
+  LCE_DEV void origins(int item, const void*& p, const void*& q) const {
+    int tp, tq, seg;
+    decode(item, tp, tq, seg);
+    const int64_t k0 = (int64_t)seg * kseg * kBK;
+    p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0 + k0;
+    q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs + k0;
   }
   LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.V); }
   LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + a.Np * a.vs; }
-  LCE_DEV int k_valid() const { return (int)a.vw; }
-  LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
-    int tp, tq;
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
-    dx_epilogue<T>(a, acc, tp, tq);
+  LCE_DEV int k_valid(int item) const {
+    const int seg = SPLIT ? item % split : 0;
+    const int64_t left = a.vw - (int64_t)seg * kseg * kBK;
+    return (int)(left < 0 ? 0 : left);
+  }
+  LCE_DEV void epilogue(int item, f32x16_t (&acc)[kNB][kNB], char*) const {
+    int tp, tq, seg;
+    decode(item, tp, tq, seg);
+    if (SPLIT) {
+      dx_partial_epilogue(a, acc, tp, tq, seg);
+    } else {
+      dx_epilogue<T>(a, acc, tp, tq);
+    }
   }
 };
 
-template <class T, class WSrc>
+template <class T, class WSrc, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DxProblem<T, WSrc> prob(a);
-  Pipe3<T, WSrc, true, E, true, DxProblem<T, WSrc>> pipe(prob);
-  pipe.run(a.ldw, a.vs, (int)(a.vs / kBK), lds);
+  DxProblem<T, WSrc, SPLIT> prob(a);
+  Pipe3<T, WSrc, true, E, true, DxProblem<T, WSrc, SPLIT>> pipe(prob);
+  pipe.run(a.ldw, a.vs, SPLIT ? a.dx_kseg : (int)(a.vs / kBK), lds);
 }
 
-template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dx_persistent_kernel<T, WSrc>;
+// Split mode, second step: dx (+)= sum over segments, in segment order; same
+// running-sum / final-store rules as the tile kernel's own epilogue.
+template <class T>
+__global__ __launch_bounds__(256) void dx_reduce_kernel(const BwdArgs a) {
+  typedef typename elem_of<T>::type E;
+  const int64_t quads_per_row = a.Hp / 4;
+  const int64_t total = a.N * quads_per_row;
+  const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t tok = i / quads_per_row, h = (i - tok * quads_per_row) * 4;
+    if (h >= a.H) continue;
+    const int64_t o = tok * a.Hp + h;
+    f32x4_t v = *reinterpret_cast<const f32x4_t*>(a.dx_part + o);
+    for (int s = 1; s < a.dx_split; ++s) v += *reinterpret_cast<const f32x4_t*>(a.dx_part + (int64_t)s * a.Np * a.Hp + o);
+    if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + o);
+    if (!a.last) {
+      *reinterpret_cast<f32x4_t*>(a.dx_acc + o) = v;
+    } else if (a.dx_dtype == DT_F32) {
+      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dx) + tok * a.lddx + h) = v * coef;
+    } else {
+      u32x2_t b;
+      b[0] = pack2<T>(v[0] * coef, v[1] * coef);
+      b[1] = pack2<T>(v[2] * coef, v[3] * coef);
+      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dx) + tok * a.lddx + h) = b;
+    }
+  }
+}
+
+template <class T, class WSrc, bool SPLIT> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dx_persistent_kernel<T, WSrc, SPLIT>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
-  const int64_t tiles = (a.Hp / kTile) * (a.Np / kTile);
-  const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
+  const int64_t items = (a.Hp / kTile) * (a.Np / kTile) * (SPLIT ? a.dx_split : 1);
+  const int grid = (int)(items < a.num_cus ? items : a.num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
+  return hipGetLastError();
+}
+
+template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  if (a.dx_split <= 1) return launch_tiles<T, WSrc, false>(a, s);
+  hipError_t e = launch_tiles<T, WSrc, true>(a, s);
+  if (e != hipSuccess) return e;
+  const int64_t quads = a.N * (a.Hp / 4);
+  int64_t blocks = (quads + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(dx_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 

@@ -172,7 +172,7 @@ template <class T, class XSrc, class WSrc, bool VTAIL> struct FwdProblem {
   }
   LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.V); }
   LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
-  LCE_DEV int k_valid() const { return (int)a.H; }
+  LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     coords(tile, tp, tq);

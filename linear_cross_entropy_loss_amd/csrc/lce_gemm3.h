@@ -149,8 +149,8 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //        first element of the P / Q operand of that output tile:
 //        (row0, k=0) for a KC operand, (k=0, col0) for an MC operand
 //   const void* p_end(), q_end()                  one past the last valid byte of each operand
-//   int  k_valid()                                K extent; the K tiles of the loop may run past
-//        it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
+//   int  k_valid(int tile)                        K extent of that tile's contraction; the K tiles of the
+//        loop may run past it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
 //   void epilogue(int tile, acc, char* scratch)
 //        consumes the finished accumulator; may use `scratch`, 96 KiB of LDS
 //        that the pipeline does not touch until the next barrier it issues
@@ -193,7 +193,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
       ps.end = ps.base;  // nothing left to fetch: every load returns 0
       qs.end = qs.base;
     }
-    k_rem = prob.k_valid();
+    k_rem = prob.k_valid(tile);
     ps.retarget(k_rem);
     qs.retarget(k_rem);
   }

@@ -67,6 +67,11 @@ struct BwdArgs {
   int64_t vw;       // columns of the slab that exist: min(vs, V - v0)
   void* dz;         // [Np][vs] staged dz in the compute type (exact zeros outside N x vw)
   float* dx_acc;    // [Np][Hp] fp32 running dx (null when there is a single slab)
+  // dx with few output tiles: the K extent of a slab is cut into `dx_split` segments of `dx_kseg`
+  // K tiles, one work item each; the partial sums meet in dx_part [dx_split][Np][Hp] (fp32) and a
+  // small kernel adds them in a fixed order.  dx_split == 1: no partials, the tile kernel finishes dx.
+  int dx_split, dx_kseg;
+  float* dx_part;
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
 };
@@ -76,6 +81,20 @@ hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s);
 hipError_t launch_fill_f32(float* p, int64_t n, float v, hipStream_t s);
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s);
+
+// Split of the dx contraction of a slab of `vs` columns (host side, shared by planning and launch):
+// with T output tiles on a device assumed to run 256 workgroups, up to 256/T segments of at least
+// 16 K tiles each (a power of two, so that segments map onto XCDs evenly).
+inline void dx_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* kseg) {
+  const int64_t tiles = (Np / 256) * (Hp / 256), ktiles = vs / 64;
+  int s = 1;
+  while (tiles * s * 2 <= 256 && ktiles / (s * 2) >= 16) s *= 2;
+  int64_t seg = (ktiles + s - 1) / s;
+  seg = (seg + 1) & ~(int64_t)1;  // an even number of K tiles, as the pipelined loop requires
+  if (seg < 4) seg = 4;
+  *kseg = (int)seg;
+  *split = (int)((ktiles + seg - 1) / seg);
+}
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
 
 }  // namespace lce
