@@ -73,7 +73,73 @@ def _check_inputs(x, y, At):
         raise ValueError("weight must be 2-D with shape (in_features, out_features)")
 
 
+def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring):
+    """Runs lce_forward.  Returns (out5, lse, n_valid) and the (x, y, w) views the kernels read."""
+    _check_inputs(x_in, y, At)
+    with torch.cuda.device(x_in.device):
+        x = _aligned_rows(x_in.reshape(-1, x_in.shape[-1]))
+        y1 = y.reshape(-1).contiguous()
+        w = _aligned_rows(At)
+        N, H = x.shape
+        H_A, V = w.shape
+        if H_A != H:
+            raise ValueError(f"weight has in_features={H_A}, input has {H}")
+        if y1.shape != (N,):
+            raise ValueError("labels must have one entry per input row")
+        prob = _lib.make_problem(
+            N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
+            ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring,
+        )
+        lib = _lib.load()
+        _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")
+        fwd_bytes, _ = _lib.workspace_bytes(prob)
+        dev = x.device
+        ws = torch.empty(fwd_bytes, dtype=torch.uint8, device=dev)
+        lse = torch.empty(N, dtype=torch.float32, device=dev)
+        out5 = torch.empty(5, dtype=torch.float32, device=dev)
+        n_valid = torch.empty(1, dtype=torch.int64, device=dev)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = lib.lce_forward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(lse), _ptr(out5),
+                             _ptr(n_valid), _ptr(ws), fwd_bytes, ctypes.c_void_p(stream))
+        _lib.raise_for_status(rc, "lce_forward")
+        del ws
+    return out5, lse, n_valid, x, y1, w
+
+
+def _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,
+                   N_chunk_size, need_dx, need_dw):
+    """Runs lce_backward on what _forward_impl returned.  dx is (N, H), dw is (H, V); None when not needed."""
+    N, H = x.shape
+    V = w.shape[1]
+    with torch.cuda.device(x.device):
+        dev = x.device
+        dx = _empty_rows(N, H, x.dtype, dev) if need_dx else None
+        dw = _empty_rows(H, V, w.dtype, dev) if need_dw else None
+        if need_dx or need_dw:
+            prob = _lib.make_problem(
+                N, H, V, x.stride(0), w.stride(0), dx.stride(0) if need_dx else H + (-H) % 8,
+                dw.stride(0) if need_dw else V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
+                ignore_index, logit_scale, z_regularization, N_chunk_size, False,
+            )
+            lib = _lib.load()
+            _, bwd_bytes = _lib.workspace_bytes(prob)
+            ws = torch.empty(bwd_bytes, dtype=torch.uint8, device=dev)
+            g = grad_output.detach().to(device=dev, dtype=torch.float32).reshape(1).contiguous()
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            rc = lib.lce_backward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(lse), _ptr(n_valid),
+                                  _ptr(g), _ptr(dx), _ptr(dw), _ptr(ws), bwd_bytes, ctypes.c_void_p(stream))
+            _lib.raise_for_status(rc, "lce_backward")
+            del ws
+    if dx is not None and not dx.is_contiguous():
+        dx = dx.contiguous()  # H not a multiple of 8
+    if dw is not None and not dw.is_contiguous():
+        dw = dw.contiguous()  # V not a multiple of 8
+    return dx, dw
+
+
 class LinearXentImplementation(torch.autograd.Function):
+    """The reference's autograd Function (``ops.py:661-810``): same arguments, same 5-tuple."""
+
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(
@@ -87,38 +153,12 @@ class LinearXentImplementation(torch.autograd.Function):
         N_chunk_size: int = 4096,
         monitoring: bool = True,
     ):
-        _check_inputs(x_in, y, At)
         # Under autocast the activations take the autocast dtype; a float32 weight is NOT copied:
         # the kernels read the fp32 master weight and round it on the way into LDS.
         if torch.is_autocast_enabled("cuda") and x_in.dtype == torch.float32:
             x_in = x_in.to(torch.get_autocast_dtype("cuda"))
-        with torch.cuda.device(x_in.device):
-            x = _aligned_rows(x_in.reshape(-1, x_in.shape[-1]))
-            y1 = y.reshape(-1).contiguous()
-            w = _aligned_rows(At)
-            N, H = x.shape
-            H_A, V = w.shape
-            if H_A != H:
-                raise ValueError(f"weight has in_features={H_A}, input has {H}")
-            if y1.shape != (N,):
-                raise ValueError("labels must have one entry per input row")
-            prob = _lib.make_problem(
-                N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-                ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring,
-            )
-            lib = _lib.load()
-            _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")
-            fwd_bytes, _ = _lib.workspace_bytes(prob)
-            dev = x.device
-            ws = torch.empty(fwd_bytes, dtype=torch.uint8, device=dev)
-            lse = torch.empty(N, dtype=torch.float32, device=dev)
-            out5 = torch.empty(5, dtype=torch.float32, device=dev)
-            n_valid = torch.empty(1, dtype=torch.int64, device=dev)
-            stream = torch.cuda.current_stream(dev).cuda_stream
-            rc = lib.lce_forward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(lse), _ptr(out5),
-                                 _ptr(n_valid), _ptr(ws), fwd_bytes, ctypes.c_void_p(stream))
-            _lib.raise_for_status(rc, "lce_forward")
-            del ws
+        out5, lse, n_valid, x, y1, w = _forward_impl(
+            x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring)
         ctx.save_for_backward(x, y1, w, lse, n_valid)
         ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size)
         ctx.x_shape = x_in.shape
@@ -131,33 +171,76 @@ class LinearXentImplementation(torch.autograd.Function):
     def backward(ctx, grad_output, void0=None, void1=None, void2=None, void3=None):
         x, y1, w, lse, n_valid = ctx.saved_tensors
         ignore_index, z_regularization, logit_scale, N_chunk_size = ctx.lce_cfg
-        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[2]
-        N, H = x.shape
-        V = w.shape[1]
-        with torch.cuda.device(x.device):
-            dev = x.device
-            dx = _empty_rows(N, H, x.dtype, dev) if need_dx else None
-            dw = _empty_rows(H, V, w.dtype, dev) if need_dw else None
-            if need_dx or need_dw:
-                prob = _lib.make_problem(
-                    N, H, V, x.stride(0), w.stride(0), dx.stride(0) if need_dx else H + (-H) % 8,
-                    dw.stride(0) if need_dw else V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-                    ignore_index, logit_scale, z_regularization, N_chunk_size, False,
-                )
-                lib = _lib.load()
-                _, bwd_bytes = _lib.workspace_bytes(prob)
-                ws = torch.empty(bwd_bytes, dtype=torch.uint8, device=dev)
-                g = grad_output.detach().to(device=dev, dtype=torch.float32).reshape(1).contiguous()
-                stream = torch.cuda.current_stream(dev).cuda_stream
-                rc = lib.lce_backward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(lse), _ptr(n_valid),
-                                      _ptr(g), _ptr(dx), _ptr(dw), _ptr(ws), bwd_bytes, ctypes.c_void_p(stream))
-                _lib.raise_for_status(rc, "lce_backward")
-                del ws
+        dx, dw = _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,
+                                N_chunk_size, ctx.needs_input_grad[0], ctx.needs_input_grad[2])
         if dx is not None:
-            dx = dx.reshape(ctx.x_shape)  # a copy only when H is not a multiple of 8
-        if dw is not None and not dw.is_contiguous():
-            dw = dw.contiguous()  # V not a multiple of 8
+            dx = dx.view(ctx.x_shape)
         return dx, None, dw, None, None, None, None, None
+
+
+# ---------------------------------------------------------------------------------------------------------
+# torch.library registration: the same two device calls as opaque operators with fake (shape-only)
+# implementations and an autograd formula, so that torch.compile / torch.export can trace through a
+# model that ends in this loss without touching the ctypes calls.  (The reference leaves
+# `torch._dynamo.disable` commented out on its Function, ops.py:664, and hard-codes fp16 autocast,
+# ops.py:665-667; here autocast follows the active autocast dtype.)
+# ---------------------------------------------------------------------------------------------------------
+@torch.library.custom_op("lce_amd::forward", mutates_args=(), device_types="cuda")
+def _op_forward(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, ignore_index: int, z_regularization: float,
+                logit_scale: float, N_chunk_size: int, monitoring: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    out5, lse, n_valid, _, _, _ = _forward_impl(x, y, At, ignore_index, z_regularization, logit_scale,
+                                                N_chunk_size, monitoring)
+    return out5, lse, n_valid
+
+
+@_op_forward.register_fake
+def _(x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring):
+    n = x.numel() // x.shape[-1]
+    return (x.new_empty((5,), dtype=torch.float32), x.new_empty((n,), dtype=torch.float32),
+            x.new_empty((1,), dtype=torch.int64))
+
+
+@torch.library.custom_op("lce_amd::backward", mutates_args=(), device_types="cuda")
+def _op_backward(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, lse: torch.Tensor, n_valid: torch.Tensor,
+                 grad_loss: torch.Tensor, ignore_index: int, z_regularization: float, logit_scale: float,
+                 N_chunk_size: int, need_dx: bool, need_dw: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    x2 = _aligned_rows(x.reshape(-1, x.shape[-1]))
+    dx, dw = _backward_impl(x2, y.reshape(-1).contiguous(), _aligned_rows(At), lse, n_valid, grad_loss,
+                            ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw)
+    dx = dx.view(x.shape) if dx is not None else x.new_empty((0,))
+    dw = dw if dw is not None else At.new_empty((0,))
+    return dx, dw
+
+
+@_op_backward.register_fake
+def _(x, y, At, lse, n_valid, grad_loss, ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw):
+    return (torch.empty_like(x, memory_format=torch.contiguous_format) if need_dx else x.new_empty((0,)),
+            torch.empty_like(At, memory_format=torch.contiguous_format) if need_dw else At.new_empty((0,)))
+
+
+def _op_setup_context(ctx, inputs, output):
+    x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, _ = inputs
+    _, lse, n_valid = output
+    ctx.save_for_backward(x, y, At, lse, n_valid)
+    ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size)
+
+
+def _op_autograd(ctx, grad_out5, grad_lse, grad_n_valid):
+    # Only the loss (entry 0 of the 5 scalars) is differentiable; the monitoring values are treated as
+    # constants, as the reference marks them non-differentiable (ops.py:798-800).
+    x, y, At, lse, n_valid = ctx.saved_tensors
+    ignore_index, z_regularization, logit_scale, N_chunk_size = ctx.lce_cfg
+    need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[2]
+    dx = dw = None
+    if need_dx or need_dw:
+        gx, gw = _op_backward(x, y, At, lse, n_valid, grad_out5[0:1].to(torch.float32), ignore_index,
+                              z_regularization, logit_scale, N_chunk_size, need_dx, need_dw)
+        dx = gx if need_dx else None
+        dw = gw if need_dw else None
+    return dx, None, dw, None, None, None, None, None
+
+
+_op_forward.register_autograd(_op_autograd, setup_context=_op_setup_context)
 
 
 def linear_cross_entropy(
@@ -170,10 +253,19 @@ def linear_cross_entropy(
     N_chunk_size: int = 4096,
     monitoring: bool = False,
 ):
-    """Functional form; returns ``(loss, z_reg, logit_max, logit_entropy, logit_norm)``."""
-    return LinearXentImplementation.apply(
-        x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring
-    )
+    """Functional form (``ops.py:814-826``); returns ``(loss, z_reg, logit_max, logit_entropy, logit_norm)``.
+
+    Goes through the registered operator ``torch.ops.lce_amd.forward``, so it can sit inside a
+    ``torch.compile``d region.  Under autocast an fp32 ``x`` takes the autocast dtype; an fp32 weight is
+    read as is (no 16-bit copy) and gets an fp32 gradient.
+    """
+    _check_inputs(x, y, At)
+    if torch.is_autocast_enabled("cuda") and x.dtype == torch.float32:
+        x = x.to(torch.get_autocast_dtype("cuda"))
+    out5, _, _ = _op_forward(x, y, At, int(ignore_index), float(z_regularization), float(logit_scale),
+                             int(N_chunk_size), bool(monitoring))
+    loss, z_reg, logit_max, logit_ent, logit_norm = out5.unbind(0)
+    return loss, z_reg.detach(), logit_max.detach(), logit_ent.detach(), logit_norm.detach()
 
 
 class LinearCrossEntropyLoss(torch.nn.Linear):
@@ -240,7 +332,7 @@ class LinearCrossEntropyLoss(torch.nn.Linear):
             torch.nn.init.trunc_normal_(self.weight, mean=0.0, std=std, a=-3 * std, b=3 * std)
 
     def forward(self, x, y):
-        loss, z_reg, logit_max, logit_ent, logit_norm = LinearXentImplementation.apply(
+        loss, z_reg, logit_max, logit_ent, logit_norm = linear_cross_entropy(
             x, y, self.weight, self.ignore_index, self.z_regularization, self.logit_scale,
             self.N_chunk_size, self.monitoring,
         )

@@ -282,3 +282,64 @@ def test_reference_accuracy_protocol_full_size(dtype, pub_loss, pub_grad):
     assert grad_err <= 2 * pub_grad
     del ref
     torch.cuda.empty_cache()
+
+
+# ---------------------------------------------------------------------------------------------------------
+# torch.library registration: operator checks and torch.compile (the reference leaves compile support open:
+# `_dynamo.disable` commented out at ops.py:664).  Backend "aot_eager" traces forward and backward through
+# fake tensors and the registered autograd formula without generating any device code of its own.
+# ---------------------------------------------------------------------------------------------------------
+def test_registered_operator_passes_opcheck():
+    import linear_cross_entropy_loss_amd  # noqa: F401  (registers torch.ops.lce_amd)
+
+    print("opcheck", flush=True)
+    x, y, w = make_inputs(512, 256, 4096, torch.bfloat16, seed=9, ignore_frac=0.1, device="cuda")
+    args = (x.requires_grad_(True), y, w.requires_grad_(True), -1, 1e-4, 1.0, 512, True)
+    torch.library.opcheck(torch.ops.lce_amd.forward.default, args,
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+
+
+def test_torch_compile_matches_eager():
+    from linear_cross_entropy_loss_amd import LinearCrossEntropyLoss
+
+    print("torch.compile aot_eager", flush=True)
+    torch.manual_seed(3)
+    head = LinearCrossEntropyLoss(256, 5000, device="cuda", dtype=torch.bfloat16, ignore_index=-1, z_regularization=1e-4)
+    body = torch.nn.Linear(256, 256, device="cuda", dtype=torch.bfloat16)
+    x = torch.randn(4, 150, 256, device="cuda", dtype=torch.bfloat16)
+    y = torch.randint(0, 5000, (4, 150), device="cuda")
+    y[0, :7] = -1
+
+    def model(x, y):
+        return head(torch.nn.functional.gelu(body(x)), y)
+
+    loss = model(x, y)
+    loss.backward()
+    ref = (loss.detach().clone(), head.weight.grad.clone(), body.weight.grad.clone())
+    head.weight.grad = None
+    body.weight.grad = None
+    compiled = torch.compile(model, backend="aot_eager", fullgraph=True)
+    for _ in range(2):
+        head.weight.grad = None
+        body.weight.grad = None
+        loss_c = compiled(x, y)
+        loss_c.backward()
+        assert torch.equal(loss_c.detach(), ref[0])
+        assert torch.equal(head.weight.grad, ref[1])
+        assert torch.equal(body.weight.grad, ref[2])
+
+
+def test_function_and_registered_operator_agree_bitwise():
+    from linear_cross_entropy_loss_amd import LinearXentImplementation, linear_cross_entropy
+
+    print("Function vs operator", flush=True)
+    x, y, w = make_inputs(777, 264, 10008, torch.float16, seed=10, ignore_frac=0.1, device="cuda")
+    res = []
+    for fn in (LinearXentImplementation.apply, linear_cross_entropy):
+        xi = x.clone().requires_grad_(True)
+        wi = w.clone().requires_grad_(True)
+        out = fn(xi, y, wi, -1, 1e-4, 0.5, 512, True)
+        out[0].backward()
+        res.append((torch.stack([o.detach() for o in out]), xi.grad, wi.grad))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
