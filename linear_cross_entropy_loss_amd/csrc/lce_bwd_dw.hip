@@ -66,6 +66,7 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
 }
 
 template <class T, class XSrc> struct DwProblem {
+  static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int tiles_p, tiles_q;

@@ -95,7 +95,8 @@ LCE_DEV void dx_partial_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], in
 // Work item = (output tile, K segment); segment fastest, so that with a
 // power-of-two split the workgroups of one XCD work on the same segment and
 // share its W rows and dz columns in their L2.
-template <class T, class WSrc, bool SPLIT> struct DxProblem {
+template <class T, class WSrc, bool SPLIT, bool KMASK> struct DxProblem {
+  static constexpr bool kKMask = KMASK;
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int tiles_p, tiles_q, split, kseg;
@@ -132,12 +133,12 @@ template <class T, class WSrc, bool SPLIT> struct DxProblem {
   }
 };
 
-template <class T, class WSrc, bool SPLIT>
+template <class T, class WSrc, bool SPLIT, bool KMASK>
 __global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DxProblem<T, WSrc, SPLIT> prob(a);
-  Pipe3<T, WSrc, true, E, true, DxProblem<T, WSrc, SPLIT>> pipe(prob);
+  DxProblem<T, WSrc, SPLIT, KMASK> prob(a);
+  Pipe3<T, WSrc, true, E, true, DxProblem<T, WSrc, SPLIT, KMASK>> pipe(prob);
   pipe.run(a.ldw, a.vs, SPLIT ? a.dx_kseg : (int)(a.vs / kBK), lds);
 }
 
@@ -169,8 +170,8 @@ __global__ __launch_bounds__(256) void dx_reduce_kernel(const BwdArgs a) {
   }
 }
 
-template <class T, class WSrc, bool SPLIT> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dx_persistent_kernel<T, WSrc, SPLIT>;
+template <class T, class WSrc, bool SPLIT, bool KMASK> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dx_persistent_kernel<T, WSrc, SPLIT, KMASK>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -181,8 +182,10 @@ template <class T, class WSrc, bool SPLIT> hipError_t launch_tiles(const BwdArgs
 }
 
 template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  if (a.dx_split <= 1) return launch_tiles<T, WSrc, false>(a, s);
-  hipError_t e = launch_tiles<T, WSrc, true>(a, s);
+  // the K mask is only needed when the K tiles of a work item run past the columns that exist
+  if (a.dx_split <= 1) return a.vw == a.vs ? launch_tiles<T, WSrc, false, false>(a, s) : launch_tiles<T, WSrc, false, true>(a, s);
+  const bool exact_k = a.vw == a.vs && (int64_t)a.dx_split * a.dx_kseg * kBK == a.vs;
+  hipError_t e = exact_k ? launch_tiles<T, WSrc, true, false>(a, s) : launch_tiles<T, WSrc, true, true>(a, s);
   if (e != hipSuccess) return e;
   const int64_t quads = a.N * (a.Hp / 4);
   int64_t blocks = (quads + 255) / 256;

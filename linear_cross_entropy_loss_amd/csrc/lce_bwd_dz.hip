@@ -164,7 +164,8 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
 // The launch covers `tiles_p` tile columns of the slab starting at column tile
 // `tp0`: all the full ones, or (VTAIL) those from the one straddling the end
 // of the vocabulary to the end of the padded slab.
-template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL> struct DzProblem {
+template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK> struct DzProblem {
+  static constexpr bool kKMask = KMASK;
   const BwdArgs& a;
   int tp0, tiles_p, tiles_q;
   LCE_DEV DzProblem(const BwdArgs& a_)
@@ -191,17 +192,17 @@ template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL> struct DzProbl
   }
 };
 
-template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL>
+template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK>
 __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  DzProblem<T, XSrc, WSrc, ZREG, VTAIL> prob(a);
-  Pipe3<T, WSrc, false, XSrc, true, DzProblem<T, XSrc, WSrc, ZREG, VTAIL>> pipe(prob);
+  DzProblem<T, XSrc, WSrc, ZREG, VTAIL, KMASK> prob(a);
+  Pipe3<T, WSrc, false, XSrc, true, DzProblem<T, XSrc, WSrc, ZREG, VTAIL, KMASK>> pipe(prob);
   pipe.run(a.ldw, a.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
-template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL>
+template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK>
 hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = bwd_dz_persistent_kernel<T, XSrc, WSrc, ZREG, VTAIL>;
+  auto kern = bwd_dz_persistent_kernel<T, XSrc, WSrc, ZREG, VTAIL, KMASK>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e != hipSuccess) return e;
@@ -213,11 +214,13 @@ hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
 // All full tile columns of the slab, then the column that straddles the end of the vocabulary.
 template <class T, class XSrc, class WSrc, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
   const int64_t tq = a.Np / kTile, full = a.vw / kTile, tail = a.vs / kTile - full;
+  const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = launch_one<T, XSrc, WSrc, ZREG, false>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, XSrc, WSrc, ZREG, false, false>(a, full * tq, s)
+                           : launch_one<T, XSrc, WSrc, ZREG, false, true>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (tail > 0) return launch_one<T, XSrc, WSrc, ZREG, true>(a, tail * tq, s);
+  if (tail > 0) return launch_one<T, XSrc, WSrc, ZREG, true, true>(a, tail * tq, s);
   return hipSuccess;
 }
 

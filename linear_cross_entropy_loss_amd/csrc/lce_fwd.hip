@@ -153,7 +153,8 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, i
 // Persistent workgroups, operand stream pipelined across output tiles.  The
 // launch covers `tiles_p` tile columns of the vocabulary starting at column
 // tile `tp0` (all full columns, or the one straddling V for the VTAIL variant).
-template <class T, class XSrc, class WSrc, bool VTAIL> struct FwdProblem {
+template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdProblem {
+  static constexpr bool kKMask = KMASK;
   const FwdArgs& a;
   int tp0, tiles_p, tiles_q;
   LCE_DEV FwdProblem(const FwdArgs& a_)
@@ -180,11 +181,11 @@ template <class T, class XSrc, class WSrc, bool VTAIL> struct FwdProblem {
   }
 };
 
-template <class T, class XSrc, class WSrc, bool VTAIL>
+template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK>
 __global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  FwdProblem<T, XSrc, WSrc, VTAIL> prob(a);
-  Pipe3<T, WSrc, false, XSrc, true, FwdProblem<T, XSrc, WSrc, VTAIL>> pipe(prob);
+  FwdProblem<T, XSrc, WSrc, VTAIL, KMASK> prob(a);
+  Pipe3<T, WSrc, false, XSrc, true, FwdProblem<T, XSrc, WSrc, VTAIL, KMASK>> pipe(prob);
   pipe.run(a.ldw, a.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
@@ -304,8 +305,9 @@ __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
   for (; i < n; i += stride) p[i] = v;
 }
 
-template <class T, class XSrc, class WSrc, bool VTAIL> hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = fwd_tiles_persistent_kernel<T, XSrc, WSrc, VTAIL>;
+template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK>
+hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
+  auto kern = fwd_tiles_persistent_kernel<T, XSrc, WSrc, VTAIL, KMASK>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -317,11 +319,13 @@ template <class T, class XSrc, class WSrc, bool VTAIL> hipError_t launch_one(con
 // All full tile columns of the vocabulary, then the column that straddles V.
 template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
   const int64_t tq = a.Np / kTile, full = a.V / kTile;
+  const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = launch_one<T, XSrc, WSrc, false>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, XSrc, WSrc, false, false>(a, full * tq, s)
+                           : launch_one<T, XSrc, WSrc, false, true>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (a.V % kTile) return launch_one<T, XSrc, WSrc, true>(a, tq, s);
+  if (a.V % kTile) return launch_one<T, XSrc, WSrc, true, true>(a, tq, s);
   return hipSuccess;
 }
 

@@ -44,7 +44,8 @@ template <bool WIDE> struct StageRegs {
 // SGPRs) points at the current K tile, each thread contributes one 32-bit byte
 // offset, and the stride between a thread's 8 chunks is a scalar offset, so a
 // load costs one instruction and no vector address arithmetic.
-template <class T, class SrcT, bool KC> struct Stager3 {
+// KMASK = false compiles the K mask out, for launches whose K tiles cover the K extent exactly.
+template <class T, class SrcT, bool KC, bool KMASK> struct Stager3 {
   static constexpr bool kWide = sizeof(SrcT) == 4;
   static constexpr int kEs = (int)sizeof(SrcT);
   typedef StageRegs<kWide> Regs;
@@ -95,7 +96,7 @@ template <class T, class SrcT, bool KC> struct Stager3 {
     const unsigned low = lo < 0x7fffffffu ? lo : 0x7fffffffu;
     const unsigned capped = hi != 0 ? 0x7fffffffu : low;
     range = hi < 0 ? 0u : capped;
-    if (KC) voff_cur = kpos < k_rem ? voff : 0x80000000u;
+    if (KC && KMASK) voff_cur = kpos < k_rem ? voff : 0x80000000u;
   }
   LCE_DEV void load(Regs& r, int i0, int i1) const {
     // 0x00020000: raw 32-bit data format.  The hardware returns 0 for every
@@ -149,6 +150,7 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //        first element of the P / Q operand of that output tile:
 //        (row0, k=0) for a KC operand, (k=0, col0) for an MC operand
 //   const void* p_end(), q_end()                  one past the last valid byte of each operand
+//   static constexpr bool kKMask                  false if `ktiles * 64 == k_valid` for every tile of the launch
 //   int  k_valid(int tile)                        K extent of that tile's contraction; the K tiles of the
 //        loop may run past it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
 //   void epilogue(int tile, acc, char* scratch)
@@ -157,8 +159,8 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //        itself -- the epilogue must end with all its LDS traffic complete
 //        (a __syncthreads() if it used scratch).
 template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> struct Pipe3 {
-  typedef Stager3<T, PSrc, P_KC> PStager;
-  typedef Stager3<T, QSrc, Q_KC> QStager;
+  typedef Stager3<T, PSrc, P_KC, Problem::kKMask> PStager;
+  typedef Stager3<T, QSrc, Q_KC, Problem::kKMask> QStager;
   typedef typename PStager::Regs PRegs;
   typedef typename QStager::Regs QRegs;
   static constexpr int kPW = PStager::kWide ? 2 : 1;  // load instructions per chunk
