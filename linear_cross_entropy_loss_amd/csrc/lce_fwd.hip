@@ -199,12 +199,26 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
   const bool exists = tok < a.N;
   const int nslices = (int)(a.Vp / kChunkV);
 
+  // Online (max, sum) merge of this group's slices, 8 at a time so that the loads of a
+  // batch are in flight together (a slice without a single valid column holds -inf and
+  // contributes exp2(-inf) = 0).
   float M = -INFINITY, S = 0.f;
-  for (int c = g; c < nslices; c += 4) {
-    const float l = a.part_lse[(int64_t)c * a.Np + tok];
-    if (l == -INFINITY) continue;  // a slice without a single valid column
-    const float Mn = fmaxf(M, l);
-    S = S * fast_exp2((M - Mn) * kLog2e) + fast_exp2((l - Mn) * kLog2e);
+  for (int c0 = g; c0 < nslices; c0 += 32) {
+    float l[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int c = c0 + 4 * u;
+      l[u] = c < nslices ? a.part_lse[(int64_t)c * a.Np + tok] : -INFINITY;
+    }
+    float mb = l[0];
+#pragma unroll
+    for (int u = 1; u < 8; ++u) mb = fmaxf(mb, l[u]);
+    if (mb == -INFINITY) continue;
+    float sb = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sb += fast_exp2((l[u] - mb) * kLog2e);
+    const float Mn = fmaxf(M, mb);
+    S = S * fast_exp2((M - Mn) * kLog2e) + sb * fast_exp2((mb - Mn) * kLog2e);
     M = Mn;
   }
   sh_m[g][r] = M;
@@ -224,11 +238,24 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
   const float lse = sh_lse[r];
   if (a.monitoring) {
     float pz = 0.f, sq = 0.f, mx = -INFINITY;
-    for (int c = g; c < nslices; c += 4) {
-      const int64_t o = (int64_t)c * a.Np + tok;
-      pz = fmaf(a.part_pz[o], fast_exp2((a.part_lse[o] - lse) * kLog2e), pz);
-      sq += a.part_sq[o];
-      mx = fmaxf(mx, a.part_max[o]);
+    for (int c0 = g; c0 < nslices; c0 += 32) {
+      float pl[8], pp[8], ps[8], pm[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int c = c0 + 4 * u;
+        const bool in = c < nslices;
+        const int64_t o = (int64_t)(in ? c : 0) * a.Np + tok;
+        pl[u] = in ? a.part_lse[o] : -INFINITY;
+        pp[u] = in ? a.part_pz[o] : 0.f;
+        ps[u] = in ? a.part_sq[o] : 0.f;
+        pm[u] = in ? a.part_max[o] : -INFINITY;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        pz = fmaf(pp[u], fast_exp2((pl[u] - lse) * kLog2e), pz);
+        sq += ps[u];
+        mx = fmaxf(mx, pm[u]);
+      }
     }
     sh_pz[g][r] = pz;
     sh_sq[g][r] = sq;
