@@ -31,9 +31,9 @@ static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must
 // private slice of `scratch` in two passes of 64 columns and reads it back as
 // whole 128-byte rows, so dz leaves the CU as full lines; no other wave is
 // involved, hence no workgroup barrier until the very end.  Staging rows are
-// 128 bytes with the 16-byte chunk index XOR-ed by (row >> 1) & 7, which keeps
-// both the 16-byte writes (32 rows per instruction) and the row reads (8 rows
-// per instruction) free of bank conflicts.
+// 128 bytes with the 16-byte chunk index XOR-ed by (row & 7) ^ ((row >> 3) & 1),
+// the swizzle of the K-contiguous operand tiles, for the 16-byte writes (32
+// rows per instruction) and the row reads (8 rows per instruction).
 //   * ignored tokens use lse = +inf, which makes every exp2 an exact +0;
 //   * the "- onehot" is applied by the one lane that owns the target column,
 //     from the fp32 value, onto the staged pass (one rounding, as in
@@ -85,7 +85,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
     for (int qb = 0; qb < kNB; ++qb) {
       const int row = qb * kBlk + (lane & 31);
       char* lrow = mine + row * (kPassCols * 2);
-      const int sw = (row >> 1) & 7;
+      const int sw = (row & 7) ^ ((row >> 3) & 1);
 #pragma unroll
       for (int pp = 0; pp < 2; ++pp) {
         const int pb = 2 * ph + pp;
@@ -148,9 +148,10 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
     // read the pass back as 128-byte rows and send it out
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int idx = i * 64 + lane;
-      const int row = idx >> 3, chunk = idx & 7;
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * (kPassCols * 2) + ((chunk ^ ((row >> 1) & 7)) << 4));
+      // 8 rows per instruction, 8 lanes each; the upper 32 lanes take their four rows in the order
+      // 5, 4, 7, 6 so that lanes l and l+32 always sit in rows of opposite parity (opposite bank halves)
+      const int row = i * 8 + (lane >> 3) + ((lane >> 5) ? 1 - 2 * ((lane >> 3) & 1) : 0), chunk = lane & 7;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * (kPassCols * 2) + ((chunk ^ (row & 7) ^ ((row >> 3) & 1)) << 4));
       *reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + ph * kPassCols + chunk * 8) = v;
       if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most 4 rows in registers at a time
     }
