@@ -44,8 +44,12 @@ int check(const lce_problem* p, bool backward) {
 }
 
 struct FwdPlan {
-  size_t part_lse, part_max, part_pz, part_sq, tgt, blk, total;
+  size_t part_lse, part_max, part_pz, part_sq, tgt, blk, w16, total;
+  int64_t vs;  // columns per forward launch: all of V, or the width of the 16-bit slab copy of an fp32 weight
 };
+
+// 16-bit type the kernels compute in: that of the activations (bf16 for fp32 activations).
+int compute_dtype(const lce_problem* p) { return p->x_dtype == LCE_F16 ? LCE_F16 : LCE_BF16; }
 
 FwdPlan plan_fwd(const lce_problem* p) {
   FwdPlan f;
@@ -58,13 +62,22 @@ FwdPlan plan_fwd(const lce_problem* p) {
   f.part_sq = o; if (p->monitoring) o += part;
   f.tgt = o; o += align_up(Np * 4);
   f.blk = o; o += align_up(Np / lce::kMergeRows * 8 * sizeof(double));
+  f.w16 = o;
+  f.vs = (int64_t)Vp;
+  if (p->w_dtype == LCE_F32) {
+    // slab copies of at most 256 MiB (at least one tile column)
+    int64_t cols = ((int64_t)256 << 20) / (p->H * 2) / 256 * 256;
+    if (cols < 256) cols = 256;
+    if (cols < f.vs) f.vs = cols;
+    o += align_up((size_t)p->H * (size_t)f.vs * 2);
+  }
   f.total = o;
   return f;
 }
 
 struct BwdPlan {
   int64_t slabs, vs;
-  size_t dz, dx_acc, dx_part, total;
+  size_t dz, dx_acc, dx_part, w16, total;
 };
 
 // Bytes of the split-K partial sums of dx for slabs of `vs` columns (0 when dx is not split).
@@ -101,13 +114,15 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
       const size_t dz = align_up(Np * (size_t)vs * 2);
       const size_t acc = slabs > 1 ? align_up(Np * Hp * 4) : 0;
       const size_t part = dx_part_bytes(Np, Hp, vs);  // at most 64 MiB
-      if ((dz + acc + part <= budget && (dz <= dz_cap || vs == 256)) || (pass == 1 && vs == 256)) {
+      const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2) : 0;  // 16-bit copy of the slab of W
+      if ((dz + acc + part + w16 <= budget && (dz <= dz_cap || vs == 256)) || (pass == 1 && vs == 256)) {
         b->slabs = slabs;
         b->vs = vs;
         b->dz = 0;
         b->dx_acc = dz;
         b->dx_part = dz + acc;
-        b->total = dz + acc + part;
+        b->w16 = dz + acc + part;
+        b->total = dz + acc + part + w16;
         return LCE_OK;
       }
     }
@@ -213,8 +228,22 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
       e = lce::launch_fill_f32(a.tgt, a.Np, 0.f, s);
       if (e != hipSuccess) return hip_fail(e, "fill");
     }
-    e = lce::launch_fwd_tiles(a, s);
-    if (e != hipSuccess) return hip_fail(e, "fwd_tiles");
+    // One launch over the whole vocabulary, or -- fp32 weight -- one per slab, each on a
+    // 16-bit copy of its columns made just before it (same stream, one buffer).
+    for (int64_t v0 = 0; v0 < p->V; v0 += f.vs) {
+      a.v0 = v0;
+      a.vw = p->V - v0 < f.vs ? p->V - v0 : f.vs;
+      if (p->w_dtype == LCE_F32) {
+        const int64_t ld16 = lce::pad_to(a.vw, 256);
+        e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, v0, a.vw, base + f.w16, ld16, compute_dtype(p), s);
+        if (e != hipSuccess) return hip_fail(e, "convert_w");
+        a.w = base + f.w16; a.ldw = ld16; a.w_dtype = compute_dtype(p); a.wv0 = v0; a.Vw = a.vw;
+      } else {
+        a.wv0 = 0; a.Vw = p->V;
+      }
+      e = lce::launch_fwd_tiles(a, s);
+      if (e != hipSuccess) return hip_fail(e, "fwd_tiles");
+    }
   }
   if (ph & LCE_PHASE_FWD_REDUCE) {
     e = lce::launch_fwd_reduce(a, s);
@@ -260,9 +289,19 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     a.vw = p->V - a.v0 < b.vs ? p->V - a.v0 : b.vs;   // columns of this slab that exist
     a.vs = lce::pad_to(a.vw, 256);                    // its padded width: dz row stride and K extent of dx
     lce::dx_split_plan(a.Np, a.Hp, a.vs, &a.dx_split, &a.dx_kseg);
+    hipError_t e;
+    if (p->w_dtype == LCE_F32) {
+      // dz and dx of this slab read a 16-bit copy of its columns of the fp32 weight
+      if ((ph & LCE_PHASE_BWD_DZ) || (dx && (ph & LCE_PHASE_BWD_DX))) {
+        e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, a.v0, a.vw, base + b.w16, a.vs, compute_dtype(p), s);
+        if (e != hipSuccess) return hip_fail(e, "convert_w");
+      }
+      a.w = base + b.w16; a.ldw = a.vs; a.w_dtype = compute_dtype(p); a.wv0 = a.v0; a.Vw = a.vw;
+    } else {
+      a.wv0 = 0; a.Vw = p->V;
+    }
     a.first = i == 0;
     a.last = i == b.slabs - 1;
-    hipError_t e;
     if (ph & LCE_PHASE_BWD_DZ) {
       e = lce::launch_bwd_dz(a, s);
       if (e != hipSuccess) return hip_fail(e, "bwd_dz");

@@ -112,10 +112,10 @@ template <class T, class WSrc, bool SPLIT, bool KMASK> struct DxProblem {
     int tp, tq, seg;
     decode(item, tp, tq, seg);
     const int64_t k0 = (int64_t)seg * kseg * kBK;
-    p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + a.v0 + k0;
+    p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + (a.v0 - a.wv0) + k0;
     q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs + k0;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.V); }
+  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
   LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + a.Np * a.vs; }
   LCE_DEV int k_valid(int item) const {
     const int seg = SPLIT ? item % split : 0;
@@ -200,10 +200,9 @@ hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<BF16>::type bf;
   typedef elem_of<F16>::type hf;
   const bool bf_compute = a.x_dtype == DT_BF16 || a.x_dtype == DT_F32;
+  // an fp32 weight arrives here as a 16-bit slab copy
   if (bf_compute && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf>(a, s);
-  if (bf_compute && a.w_dtype == DT_F32) return launch_persistent<BF16, float>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_persistent<F16, float>(a, s);
   return hipErrorInvalidValue;
 }
 

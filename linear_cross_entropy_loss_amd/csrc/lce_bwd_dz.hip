@@ -180,10 +180,10 @@ template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK> st
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     coords(tile, tp, tq);
-    p = reinterpret_cast<const WSrc*>(a.w) + a.v0 + (int64_t)tp * kTile;
+    p = reinterpret_cast<const WSrc*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
     q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.V); }
+  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
   LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
@@ -237,9 +237,8 @@ hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<F16>::type hf;
   if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf, bf>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf, hf>(a, s);
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch_persistent<BF16, bf, float>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_persistent<F16, hf, float>(a, s);
-  if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch_persistent<BF16, float, float>(a, s);
+  // an fp32 weight arrives here as a 16-bit slab copy; fp32 activations are converted on the way into LDS
+  if (a.x_dtype == DT_F32 && a.w_dtype == DT_BF16) return launch_persistent<BF16, float, bf>(a, s);
   return hipErrorInvalidValue;
 }
 

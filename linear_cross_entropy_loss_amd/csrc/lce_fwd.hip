@@ -151,14 +151,15 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, i
 }
 
 // Persistent workgroups, operand stream pipelined across output tiles.  The
-// launch covers `tiles_p` tile columns of the vocabulary starting at column
-// tile `tp0` (all full columns, or the one straddling V for the VTAIL variant).
+// launch covers `tiles_p` tile columns of the vocabulary window [v0, v0 + vw)
+// starting at its column tile `tp0` (all full columns, or the one straddling V
+// for the VTAIL variant).
 template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdProblem {
   static constexpr bool kKMask = KMASK;
   const FwdArgs& a;
   int tp0, tiles_p, tiles_q;
   LCE_DEV FwdProblem(const FwdArgs& a_)
-      : a(a_), tp0(VTAIL ? (int)(a_.V / kTile) : 0), tiles_p(VTAIL ? 1 : (int)(a_.V / kTile)),
+      : a(a_), tp0(VTAIL ? (int)(a_.vw / kTile) : 0), tiles_p(VTAIL ? 1 : (int)(a_.vw / kTile)),
         tiles_q((int)(a_.Np / kTile)) {}
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void coords(int tile, int& tp, int& tq) const {
@@ -168,16 +169,16 @@ template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdPro
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     coords(tile, tp, tq);
-    p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile;
+    p = reinterpret_cast<const WSrc*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
     q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.V); }
+  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
   LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     coords(tile, tp, tq);
-    fwd_epilogue<T, VTAIL>(a, acc, tp, tq);
+    fwd_epilogue<T, VTAIL>(a, acc, (int)(a.v0 / kTile) + tp, tq);
   }
 };
 
@@ -345,14 +346,14 @@ hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
 
 // All full tile columns of the vocabulary, then the column that straddles V.
 template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
-  const int64_t tq = a.Np / kTile, full = a.V / kTile;
+  const int64_t tq = a.Np / kTile, full = a.vw / kTile;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
     hipError_t e = exact_k ? launch_one<T, XSrc, WSrc, false, false>(a, full * tq, s)
                            : launch_one<T, XSrc, WSrc, false, true>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (a.V % kTile) return launch_one<T, XSrc, WSrc, true, true>(a, tq, s);
+  if (a.vw % kTile) return launch_one<T, XSrc, WSrc, true, true>(a, tq, s);
   return hipSuccess;
 }
 
@@ -363,9 +364,8 @@ hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
   typedef elem_of<F16>::type hf;
   if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf, bf>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf, hf>(a, s);
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_F32) return launch_persistent<BF16, bf, float>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F32) return launch_persistent<F16, hf, float>(a, s);
-  if (a.x_dtype == DT_F32 && a.w_dtype == DT_F32) return launch_persistent<BF16, float, float>(a, s);
+  // an fp32 weight arrives here as a 16-bit slab copy; fp32 activations are converted on the way into LDS
+  if (a.x_dtype == DT_F32 && a.w_dtype == DT_BF16) return launch_persistent<BF16, float, bf>(a, s);
   return hipErrorInvalidValue;
 }
 

@@ -31,6 +31,10 @@ struct FwdArgs {
   const int64_t* y;
   int64_t N, H, V, ldx, ldw;
   int64_t Np, Vp;  // padded_tokens(N), padded_vocab(V)
+  // Vocabulary columns [v0, v0 + vw) covered by this launch (v0 a multiple of 256), and the
+  // window of W that the buffer `w` holds: columns [wv0, wv0 + Vw) of the weight, row stride ldw.
+  // (`w` is the caller's matrix, wv0 = 0, Vw = V -- or a 16-bit copy of one slab of an fp32 weight.)
+  int64_t v0, vw, wv0, Vw;
   int x_dtype, w_dtype;  // compute type = x_dtype (bf16 / f16)
   int64_t ignore_index;
   float scale, z_reg;
@@ -65,6 +69,7 @@ struct BwdArgs {
   // slab being processed
   int64_t v0, vs;   // first column and padded width (multiple of 256) of the vocabulary slab
   int64_t vw;       // columns of the slab that exist: min(vs, V - v0)
+  int64_t wv0, Vw;  // `w` holds columns [wv0, wv0 + Vw) of the weight (the whole matrix, or a 16-bit copy of this slab)
   void* dz;         // [Np][vs] staged dz in the compute type (exact zeros outside N x vw)
   float* dx_acc;    // [Np][Hp] fp32 running dx (null when there is a single slab)
   // dx with few output tiles: the K extent of a slab is cut into `dx_split` segments of `dx_kseg`
@@ -96,5 +101,9 @@ inline void dx_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* k
   *split = (int)((ktiles + seg - 1) / seg);
 }
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
+// dst[h][c] = 16-bit rounding of src[h * ld + v0 + c] for c < vw, 0 for vw <= c < dst_ld; h < H.
+// compute_dtype: DT_BF16 or DT_F16.
+hipError_t launch_convert_w_slab(const float* src, int64_t ld, int64_t H, int64_t v0, int64_t vw, void* dst,
+                                 int64_t dst_ld, int compute_dtype, hipStream_t s);
 
 }  // namespace lce

@@ -147,6 +147,22 @@ def test_backward_plan_is_consistent_with_workspace():
         assert Np * width * 2 <= max(1 << 30, Np * 256 * 2)   # dz stage capped at 1 GiB
 
 
+def test_fp32_weight_adds_one_16_bit_slab_copy_to_the_scratch():
+    """An fp32 (master) weight is rounded to the compute type one vocabulary slab at a time; the scratch of
+    both calls grows by that slab copy and stays within the N_chunk bound."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    N, H, V, nc = 65536, 8192, 262144, 8192
+    p16 = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc, x_dtype=torch.float16, w_dtype=torch.float16)
+    p32 = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc, x_dtype=torch.float16, w_dtype=torch.float32,
+                dw_dtype=torch.float32)
+    f16, b16 = _lib.workspace_bytes(p16)
+    f32, b32 = _lib.workspace_bytes(p32)
+    slabs, width = _lib.backward_plan(p32)
+    assert b32 - b16 == H * width * 2 and b32 <= nc * V * 4
+    assert 0 < f32 - f16 <= 256 << 20
+
+
 def test_null_and_small_workspace_are_rejected_without_touching_the_gpu(lib):
     from linear_cross_entropy_loss_amd import _lib
 
