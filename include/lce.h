@@ -67,7 +67,7 @@ typedef struct lce_problem {
   int64_t lddx;         /* row stride of dx, elements (backward only)          */
   int64_t lddw;         /* row stride of dw, elements (backward only)          */
   int32_t x_dtype;      /* LCE_BF16 | LCE_F16 | LCE_F32                        */
-  int32_t w_dtype;      /* same as x_dtype, or LCE_F32 (master weight, cast in-kernel) */
+  int32_t w_dtype;      /* same as x_dtype, or LCE_F32 (master weight, rounded slab by slab in ws) */
   int32_t dx_dtype;     /* x_dtype or LCE_F32                                  */
   int32_t dw_dtype;     /* w_dtype or LCE_F32                                  */
   int64_t ignore_index; /* any int64 (ops.py:674)                              */

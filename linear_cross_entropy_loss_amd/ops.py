@@ -154,7 +154,7 @@ class LinearXentImplementation(torch.autograd.Function):
         monitoring: bool = True,
     ):
         # Under autocast the activations take the autocast dtype; a float32 weight is NOT copied:
-        # the kernels read the fp32 master weight and round it on the way into LDS.
+        # the library rounds the fp32 master weight one vocabulary slab at a time, inside its workspace.
         if torch.is_autocast_enabled("cuda") and x_in.dtype == torch.float32:
             x_in = x_in.to(torch.get_autocast_dtype("cuda"))
         out5, lse, n_valid, x, y1, w = _forward_impl(
