@@ -368,3 +368,48 @@ def test_function_and_registered_operator_agree_bitwise():
         res.append((torch.stack([o.detach() for o in out]), xi.grad, wi.grad))
     for a, b in zip(*res):
         assert torch.equal(a, b)
+
+
+def test_forward_backward_can_be_captured_in_a_hip_graph():
+    """The library only enqueues kernels on the caller's stream (no synchronisation, no memset nodes, no
+    allocation of its own), so a whole loss + backward step can be captured once and replayed; every replay,
+    with eager work and synchronisations in between, must equal the eager result bit for bit."""
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    print("hip graph capture", flush=True)
+    N, H, V = 1024, 512, 10000
+    x, y, w = make_inputs(N, H, V, torch.bfloat16, seed=3, ignore_frac=0.1, device="cuda")
+    xs, ws, ys = x.clone().requires_grad_(True), w.clone().requires_grad_(True), y.clone()
+
+    def step(xi, yi, wi):
+        out = linear_cross_entropy(xi, yi, wi, -1, 1e-4, 1.0, 512, True)
+        out[0].backward()
+        return out
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            xs.grad = None
+            ws.grad = None
+            step(xs, ys, ws)
+    torch.cuda.current_stream().wait_stream(side)
+    xs.grad = None
+    ws.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = step(xs, ys, ws)
+    for trial in range(3):
+        x2, y2, w2 = make_inputs(N, H, V, torch.bfloat16, seed=10 + trial, ignore_frac=0.1, device="cuda")
+        with torch.no_grad():
+            xs.copy_(x2)
+            ws.copy_(w2)
+            ys.copy_(y2)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (torch.stack([o.detach() for o in out_g]).clone(), xs.grad.clone(), ws.grad.clone())
+        xe, we = x2.clone().requires_grad_(True), w2.clone().requires_grad_(True)
+        oe = step(xe, y2, we)
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], torch.stack([o.detach() for o in oe]))
+        assert torch.equal(got[1], xe.grad) and torch.equal(got[2], we.grad)
