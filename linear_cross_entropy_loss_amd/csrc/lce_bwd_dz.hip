@@ -152,7 +152,9 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
       // 5, 4, 7, 6 so that lanes l and l+32 always sit in rows of opposite parity (opposite bank halves)
       const int row = i * 8 + (lane >> 3) + ((lane >> 5) ? 1 - 2 * ((lane >> 3) & 1) : 0), chunk = lane & 7;
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * (kPassCols * 2) + ((chunk ^ (row & 7) ^ ((row >> 3) & 1)) << 4));
-      *reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + ph * kPassCols + chunk * 8) = v;
+      // streaming store: dz (1 GiB per slab) is read back from HBM by the next kernels anyway, and a
+      // normal store would evict the W / x tiles the following main loop is about to reuse from L2
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + ph * kPassCols + chunk * 8));
       if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most 4 rows in registers at a time
     }
   }
