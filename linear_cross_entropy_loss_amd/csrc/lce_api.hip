@@ -77,7 +77,7 @@ FwdPlan plan_fwd(const lce_problem* p) {
 
 struct BwdPlan {
   int64_t slabs, vs;
-  size_t dz, dx_acc, dx_part, w16, total;
+  size_t dz, dx_acc, dx_part, dw_part, w16, total;
 };
 
 // Bytes of the split-K partial sums of dx for slabs of `vs` columns (0 when dx is not split).
@@ -85,6 +85,19 @@ size_t dx_part_bytes(size_t Np, size_t Hp, int64_t vs) {
   int split, kseg;
   lce::dx_split_plan((int64_t)Np, (int64_t)Hp, vs, &split, &kseg);
   return split > 1 ? align_up((size_t)split * Np * Hp * 4) : 0;
+}
+
+// The same for dW (0 when dW is not split).  A narrower last slab has fewer output tiles and may be
+// split further, so both widths are sized.
+size_t dw_part_bytes(size_t Np, size_t Hp, int64_t vs, int64_t last_vs) {
+  size_t need = 0;
+  for (int64_t w : {vs, last_vs}) {
+    int split, kseg;
+    lce::dw_split_plan((int64_t)Np, (int64_t)Hp, w, &split, &kseg);
+    const size_t b = split > 1 ? align_up((size_t)split * Hp * (size_t)w * 4) : 0;
+    if (b > need) need = b;
+  }
+  return need;
 }
 
 // Fewest vocabulary slabs (of a width that is a multiple of 256 columns; the last
@@ -113,7 +126,9 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
       const int64_t slabs = (Vp + vs - 1) / vs;
       const size_t dz = align_up(Np * (size_t)vs * 2);
       const size_t acc = slabs > 1 ? align_up(Np * Hp * 4) : 0;
-      const size_t part = dx_part_bytes(Np, Hp, vs);  // at most 64 MiB
+      const int64_t last_vs = Vp - (slabs - 1) * vs;  // padded width of the last slab
+      const size_t dxp = dx_part_bytes(Np, Hp, vs), dwp = dw_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
+      const size_t part = dxp + dwp;
       const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2) : 0;  // 16-bit copy of the slab of W
       if ((dz + acc + part + w16 <= budget && (dz <= dz_cap || vs == 256)) || (pass == 1 && vs == 256)) {
         b->slabs = slabs;
@@ -121,6 +136,7 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
         b->dz = 0;
         b->dx_acc = dz;
         b->dx_part = dz + acc;
+        b->dw_part = dz + acc + dxp;
         b->w16 = dz + acc + part;
         b->total = dz + acc + part + w16;
         return LCE_OK;
@@ -280,6 +296,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.dz = base + b.dz;
   a.dx_acc = b.slabs > 1 ? (float*)(base + b.dx_acc) : nullptr;
   a.dx_part = (float*)(base + b.dx_part);
+  a.dw_part = (float*)(base + b.dw_part);
   rc = current_num_cus(&a.num_cus);
   if (rc != LCE_OK) return rc;
   const int ph = p->phases ? p->phases : ~0;
@@ -289,6 +306,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     a.vw = p->V - a.v0 < b.vs ? p->V - a.v0 : b.vs;   // columns of this slab that exist
     a.vs = lce::pad_to(a.vw, 256);                    // its padded width: dz row stride and K extent of dx
     lce::dx_split_plan(a.Np, a.Hp, a.vs, &a.dx_split, &a.dx_kseg);
+    lce::dw_split_plan(a.Np, a.Hp, a.vs, &a.dw_split, &a.dw_kseg);
     hipError_t e;
     if (p->w_dtype == LCE_F32) {
       // dz and dx of this slab read a 16-bit copy of its columns of the fp32 weight

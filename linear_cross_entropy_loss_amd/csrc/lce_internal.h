@@ -77,6 +77,10 @@ struct BwdArgs {
   // small kernel adds them in a fixed order.  dx_split == 1: no partials, the tile kernel finishes dx.
   int dx_split, dx_kseg;
   float* dx_part;
+  // The same for dW with few output tiles (small vocabulary slab x hidden size): K = tokens is cut into
+  // dw_split segments of dw_kseg K tiles; partial sums in dw_part [dw_split][Hp][vs] (fp32).
+  int dw_split, dw_kseg;
+  float* dw_part;
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
 };
@@ -86,12 +90,16 @@ hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s);
 hipError_t launch_fill_f32(float* p, int64_t n, float v, hipStream_t s);
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s);
+hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
+// dst[h][c] = 16-bit rounding of src[h * ld + v0 + c] for c < vw, 0 for vw <= c < dst_ld; h < H.
+// compute_dtype: DT_BF16 or DT_F16.
+hipError_t launch_convert_w_slab(const float* src, int64_t ld, int64_t H, int64_t v0, int64_t vw, void* dst,
+                                 int64_t dst_ld, int compute_dtype, hipStream_t s);
 
-// Split of the dx contraction of a slab of `vs` columns (host side, shared by planning and launch):
-// with T output tiles on a device assumed to run 256 workgroups, up to 256/T segments of at least
-// 16 K tiles each (a power of two, so that segments map onto XCDs evenly).
-inline void dx_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* kseg) {
-  const int64_t tiles = (Np / 256) * (Hp / 256), ktiles = vs / 64;
+// Split of a contraction with few output tiles along K (host side, shared by planning and launch):
+// with `tiles` output tiles on a device assumed to run 256 workgroups, up to 256/tiles segments of
+// at least 16 K tiles each (a power of two, so that segments map onto XCDs evenly).
+inline void k_split_plan(int64_t tiles, int64_t ktiles, int* split, int* kseg) {
   int s = 1;
   while (tiles * s * 2 <= 256 && ktiles / (s * 2) >= 16) s *= 2;
   int64_t seg = (ktiles + s - 1) / s;
@@ -100,10 +108,13 @@ inline void dx_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* k
   *kseg = (int)seg;
   *split = (int)((ktiles + seg - 1) / seg);
 }
-hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
-// dst[h][c] = 16-bit rounding of src[h * ld + v0 + c] for c < vw, 0 for vw <= c < dst_ld; h < H.
-// compute_dtype: DT_BF16 or DT_F16.
-hipError_t launch_convert_w_slab(const float* src, int64_t ld, int64_t H, int64_t v0, int64_t vw, void* dst,
-                                 int64_t dst_ld, int compute_dtype, hipStream_t s);
+// dx of one slab: (Np/256) x (Hp/256) tiles, K = vs columns
+inline void dx_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* kseg) {
+  k_split_plan((Np / 256) * (Hp / 256), vs / 64, split, kseg);
+}
+// dW of one slab: (vs/256) x (Hp/256) tiles, K = Np tokens
+inline void dw_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* kseg) {
+  k_split_plan((vs / 256) * (Hp / 256), Np / 64, split, kseg);
+}
 
 }  // namespace lce

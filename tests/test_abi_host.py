@@ -112,11 +112,13 @@ def test_budget_is_a_target_not_a_refusal():
         p = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc)
         assert _lib.backward_plan(p) == (1, V)
         _, bwd = _lib.workspace_bytes(p)
-        assert nc * V * 4 < bwd == N * V * 2 <= nc * V * 4 + N * H * 4   # 512 dx tiles: no K split
+        # dz for all tokens (+ the split-K partials of dW when V*H gives few dW tiles; dx has 512 tiles: no split)
+        assert nc * V * 4 < bwd <= nc * V * 4 + N * H * 4 and N * V * 2 <= bwd <= N * V * 2 + (64 << 20)
     p = _prob(N=65536, H=256, V=4096, ldx=256, ldw=4096, lddx=256, lddw=4096, n_chunk=64)   # nothing fits
     assert _lib.backward_plan(p) == (16, 256)
     _, bwd = _lib.workspace_bytes(p)
-    assert bwd == 65536 * 256 * 2 + 65536 * 256 * 4   # 256 dx tiles: no K split
+    # dz + fp32 running dx (256 dx tiles: no K split) + the split-K partials of the single dW tile
+    assert 0 < bwd - (65536 * 256 * 2 + 65536 * 256 * 4) <= 64 << 20
 
 
 def test_backward_plan_is_consistent_with_workspace():
@@ -124,14 +126,25 @@ def test_backward_plan_is_consistent_with_workspace():
 
     pad = lambda v, m: -(-v // m) * m
 
-    def dx_part_bytes(Np, Hp, vs):
-        # dx with few output tiles is split along K: up to 256/T segments of >= 16 K tiles (power of two)
-        tiles, ktiles, s = (Np // 256) * (Hp // 256), vs // 64, 1
+    def k_split(tiles, ktiles):
+        # a contraction with few output tiles is split along K: up to 256/tiles segments of >= 16 K tiles
+        # (a power of two), an even number of K tiles each
+        s = 1
         while tiles * s * 2 <= 256 and ktiles // (s * 2) >= 16:
             s *= 2
         seg = max(4, (-(-ktiles // s) + 1) & ~1)
-        split = -(-ktiles // seg)
+        return -(-ktiles // seg)
+
+    def dx_part_bytes(Np, Hp, vs):
+        split = k_split((Np // 256) * (Hp // 256), vs // 64)
         return split * Np * Hp * 4 if split > 1 else 0
+
+    def dw_part_bytes(Np, Hp, vs, last_vs):
+        need = 0
+        for w in (vs, last_vs):
+            split = k_split((w // 256) * (Hp // 256), Np // 64)
+            need = max(need, split * Hp * w * 4 if split > 1 else 0)
+        return need
 
     for N, H, V, nc in ((16384, 2048, 131072, 4096), (16384, 2048, 131072, 8192), (65536, 8192, 262144, 8192),
                         (512, 256, 4096, 512), (1000, 520, 50264, 512), (300, 104, 1008, 64), (16384, 768, 50264, 4096)):
@@ -142,8 +155,9 @@ def test_backward_plan_is_consistent_with_workspace():
         Np, Hp = pad(N, 256), pad(H, 256)
         _, bwd = _lib.workspace_bytes(p)
         part = dx_part_bytes(Np, Hp, width)
-        assert part <= 64 << 20
-        assert bwd == Np * width * 2 + (Np * Hp * 4 if slabs > 1 else 0) + part
+        partw = dw_part_bytes(Np, Hp, width, pad(V, 256) - (slabs - 1) * width)
+        assert part <= 64 << 20 and partw <= 64 << 20
+        assert bwd == Np * width * 2 + (Np * Hp * 4 if slabs > 1 else 0) + part + partw
         assert Np * width * 2 <= max(1 << 30, Np * 256 * 2)   # dz stage capped at 1 GiB
 
 
