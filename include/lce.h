@@ -13,7 +13,8 @@
  *     library keeps no state between calls: scratch comes in through `ws`.
  *   - x is (N, H) row-major with row stride ldx; w is the TRANSPOSED weight
  *     (H, V) row-major with row stride ldw (linear_cross_entropy/ops.py:913);
- *     y is N contiguous int64 labels (ops.py:210).
+ *     y is N contiguous int64 labels (ops.py:210), each ignore_index or in
+ *     [0, V); any other value makes the returned loss NaN.
  *   - Shapes: any N, H, V, n_chunk >= 1 (N, V <= 2^30, H <= 2^20).  The
  *     reference's divisibility rules (N % 512, H % 256, V % 4096,
  *     ops.py:689-691, 905-907) are lifted; shapes that obey them run at full

@@ -194,7 +194,7 @@ __global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const Fw
 __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
   __shared__ float sh_m[4][kMergeRows], sh_s[4][kMergeRows], sh_lse[kMergeRows];
   __shared__ float sh_pz[4][kMergeRows], sh_sq[4][kMergeRows], sh_mx[4][kMergeRows];
-  __shared__ double sh_red[6][kMergeRows];
+  __shared__ double sh_red[7][kMergeRows];
   const int r = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int64_t tok = (int64_t)blockIdx.x * kMergeRows + r;  // < Np; rows >= N only keep the block sums aligned
   const bool exists = tok < a.N;
@@ -280,9 +280,11 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
     sh_red[3][r] = nrm;
     sh_red[4][r] = mx;
     sh_red[5][r] = valid ? 1.0 : 0.0;
+    // a label that is neither ignore_index nor a column of W: poisons the loss (see fwd_final_kernel)
+    sh_red[6][r] = (valid && (a.y[tok] < 0 || a.y[tok] >= a.V)) ? 1.0 : 0.0;
   }
   __syncthreads();
-  if (threadIdx.x < 6) {
+  if (threadIdx.x < 7) {
     const int q = threadIdx.x;
     double acc = sh_red[q][0];
     for (int i = 1; i < kMergeRows; ++i) acc = (q == 4) ? fmax(acc, sh_red[q][i]) : acc + sh_red[q][i];
@@ -291,24 +293,24 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
 }
 
 __global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
-  __shared__ double sh[6][256];
+  __shared__ double sh[7][256];
   const int nblk = (int)(a.Np / kMergeRows);
   const double* blk = reinterpret_cast<const double*>(a.blk);
-  double v[6] = {0, 0, 0, 0, -INFINITY, 0};
+  double v[7] = {0, 0, 0, 0, -INFINITY, 0, 0};
   for (int b = threadIdx.x; b < nblk; b += 256) {
 #pragma unroll
-    for (int q = 0; q < 6; ++q) {
+    for (int q = 0; q < 7; ++q) {
       const double t = blk[(int64_t)b * 8 + q];
       v[q] = (q == 4) ? fmax(v[q], t) : v[q] + t;
     }
   }
 #pragma unroll
-  for (int q = 0; q < 6; ++q) sh[q][threadIdx.x] = v[q];
+  for (int q = 0; q < 7; ++q) sh[q][threadIdx.x] = v[q];
   __syncthreads();
   for (int w = 128; w > 0; w >>= 1) {
     if (threadIdx.x < w) {
 #pragma unroll
-      for (int q = 0; q < 6; ++q) {
+      for (int q = 0; q < 7; ++q) {
         const double t = sh[q][threadIdx.x + w];
         sh[q][threadIdx.x] = (q == 4) ? fmax(sh[q][threadIdx.x], t) : sh[q][threadIdx.x] + t;
       }
@@ -318,7 +320,11 @@ __global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
   if (threadIdx.x == 0) {
     const double R = sh[5][0];  // 0 valid labels -> 0/0 = NaN, as F.cross_entropy gives
     const double ce = sh[0][0] / R, zr = sh[1][0] / R;
-    a.out5[0] = (float)(ce + (double)a.z_reg * zr);
+    // Labels outside [0, V) that are not ignore_index have no column to match; the reference lets
+    // them contribute lse alone, silently.  Here they turn the loss into NaN (F.cross_entropy
+    // raises a device-side assert for them) -- visible to the caller, no synchronisation needed.
+    const bool bad_labels = sh[6][0] != 0.0;
+    a.out5[0] = bad_labels ? __builtin_nanf("") : (float)(ce + (double)a.z_reg * zr);
     a.out5[1] = (float)zr;
     a.out5[2] = a.monitoring ? (float)sh[4][0] : 0.f;
     a.out5[3] = a.monitoring ? (float)(sh[2][0] / R) : 0.f;

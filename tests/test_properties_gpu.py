@@ -166,6 +166,23 @@ def test_shape_errors_raise_value_error():
         linear_cross_entropy(x, y.to(torch.int32), w)  # labels must be int64
 
 
+def test_out_of_range_labels_poison_the_loss():
+    """A label outside [0, V) that is not ignore_index has no column to match.  The reference lets it through
+    silently (it then contributes lse alone); F.cross_entropy raises a device assert.  Here the loss is NaN."""
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    print("out-of-range labels", flush=True)
+    x, y, w = make_inputs(512, 256, 4096, torch.bfloat16, seed=6, ignore_frac=0.1, device="cuda")
+    assert torch.isfinite(linear_cross_entropy(x, y, w, -1)[0])
+    for bad in (4096, 10**12, -7):
+        yb = y.clone()
+        yb[3] = bad
+        assert torch.isnan(linear_cross_entropy(x, yb, w, -1)[0]), bad
+    yb = torch.where(y == -1, torch.full_like(y, -7), y)
+    assert torch.isfinite(linear_cross_entropy(x, yb, w, -7)[0])   # ... unless it is the ignore_index
+    assert torch.isnan(linear_cross_entropy(x, y, w, -7)[0])       # the -1 labels are now out of range
+
+
 def test_autocast_keeps_fp32_master_weight_and_returns_fp32_dw():
     from linear_cross_entropy_loss_amd import LinearCrossEntropyLoss
     from oracle import lce_forward_backward_fp64
