@@ -251,3 +251,48 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_header_is_plain_c_and_links_from_a_c_program(tmp_path):
+    """include/lce.h compiles as strict C99 and a C program linked against the library can call the
+    host-only entry points (no GPU involved: validation, planning, error strings)."""
+    import shutil
+    import subprocess
+
+    from linear_cross_entropy_loss_amd import _lib
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "lce.h"
+int main(void) {
+  lce_problem p;
+  size_t fwd = 0, bwd = 0;
+  int64_t slabs = 0, width = 0;
+  memset(&p, 0, sizeof p);
+  p.N = 16384; p.H = 2048; p.V = 131072; p.ldx = 2048; p.ldw = 131072; p.lddx = 2048; p.lddw = 131072;
+  p.x_dtype = LCE_BF16; p.w_dtype = LCE_BF16; p.dx_dtype = LCE_BF16; p.dw_dtype = LCE_BF16;
+  p.ignore_index = -100; p.logit_scale = 1.0f; p.z_reg = 0.0f; p.n_chunk = 4096;
+  if (lce_check_problem(&p) != LCE_OK) return 1;
+  if (lce_workspace_bytes(&p, &fwd, &bwd) != LCE_OK) return 2;
+  if (lce_backward_plan(&p, &slabs, &width) != LCE_OK) return 3;
+  p.N = 0;
+  if (lce_check_problem(&p) != LCE_EINVAL_SHAPE) return 4;
+  printf("%d %lu %lu %ld %ld %s\n", lce_version(), (unsigned long)fwd, (unsigned long)bwd, (long)slabs, (long)width,
+         lce_strerror(LCE_EWORKSPACE));
+  return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    libdir = str(_lib.LIB_PATH.parent)
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", inc, str(src), "-o", str(exe),
+                    "-L", libdir, "-l:" + _lib.LIB_PATH.name, "-Wl,-rpath," + libdir,
+                    "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split(None, 5)
+    assert int(out[0]) >= 100 and int(out[3]) == 4 and int(out[4]) == 32768
+    assert int(out[2]) <= 4096 * 131072 * 4 and "workspace" in out[5]
