@@ -240,10 +240,6 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
   const int ph = p->phases ? p->phases : ~0;
   hipError_t e;
   if (ph & LCE_PHASE_FWD_TILES) {
-    if (ph & LCE_PHASE_FWD_REDUCE) {  // a tiles-only (profiling) call reuses the zeroed buffer
-      e = lce::launch_fill_f32(a.tgt, a.Np, 0.f, s);
-      if (e != hipSuccess) return hip_fail(e, "fill");
-    }
     // One launch over the whole vocabulary, or -- fp32 weight -- one per slab, each on a
     // 16-bit copy of its columns made just before it (same stream, one buffer).
     for (int64_t v0 = 0; v0 < p->V; v0 += f.vs) {

@@ -274,6 +274,8 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
       ent = valid ? (double)(lse - pz) : 0.0;
       nrm = (double)sqrtf(sq);
     }
+    // tgt[tok] is written by the one tile that holds the target column; it is only read for a valid
+    // label (for a valid label outside [0, V) nothing wrote it -- and the loss is NaN anyway)
     sh_red[0][r] = valid ? l - (double)a.tgt[tok] : 0.0;
     sh_red[1][r] = valid ? l * l : 0.0;
     sh_red[2][r] = ent;
@@ -333,12 +335,6 @@ __global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
   }
 }
 
-__global__ void fill_f32_kernel(float* p, int64_t n, float v) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (; i < n; i += stride) p[i] = v;
-}
-
 template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK>
 hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
   auto kern = fwd_tiles_persistent_kernel<T, XSrc, WSrc, VTAIL, KMASK>;
@@ -380,14 +376,6 @@ hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(fwd_final_kernel, dim3(1), dim3(256), 0, s, a);
-  return hipGetLastError();
-}
-
-hipError_t launch_fill_f32(float* p, int64_t n, float v, hipStream_t s) {
-  if (n <= 0) return hipSuccess;
-  int64_t blocks = (n + 255) / 256;
-  if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p, n, v);
   return hipGetLastError();
 }
 

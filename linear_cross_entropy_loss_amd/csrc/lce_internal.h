@@ -48,7 +48,7 @@ struct FwdArgs {
   float* part_max;   // [Vp/128][Np]  per-slice max            (monitoring)
   float* part_pz;    // [Vp/128][Np]  per-slice sum softmax*z  (monitoring)
   float* part_sq;    // [Vp/128][Np]  per-slice sum z^2        (monitoring)
-  float* tgt;        // [Np]          target logit, pre-zeroed
+  float* tgt;        // [Np]          target logit (written for tokens whose label is a column of W)
   float* blk;        // [Np/64][8]    per-merge-block partial sums
 };
 
@@ -87,7 +87,6 @@ struct BwdArgs {
 
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s);
 hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s);
-hipError_t launch_fill_f32(float* p, int64_t n, float v, hipStream_t s);
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
