@@ -203,3 +203,36 @@ def test_gpt2_vocabulary_matches_fp64_oracle_evaluated_on_gpu():
         print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
         assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
     assert (xd.grad[y == -1] == 0).all()
+
+
+def test_randomized_shapes_and_options_match_oracle():
+    """Twenty seeded draws over token counts, hidden sizes, vocabularies (tile multiples, off-by-one,
+    non-multiples of 8), dtypes, fp32 master weight, ignore fraction, z-regularisation, scale, N_chunk_size
+    (forcing one or many slabs, split-K or not) and monitoring -- each against the fp64 oracle."""
+    import random
+
+    rng = random.Random(1234)
+    for it in range(20):
+        N = rng.choice([1, 7, 100, 255, 256, 257, 600, 1024, 1500, 3000])
+        H = rng.choice([8, 24, 100, 128, 136, 256, 264, 520, 777, 1024])
+        V = rng.choice([8, 9, 255, 256, 263, 1000, 1001, 4096, 5000, 10008, 12000])
+        dt = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+        wdt = rng.choice([None, torch.float32]) if dt != torch.float32 else None
+        ign, zreg, scale = rng.choice([0.0, 0.1, 0.5]), rng.choice([0.0, 1e-4, 1e-2]), rng.choice([1.0, 0.5, 2.0])
+        nc, mon = rng.choice([16, 64, 512, 4096]), rng.choice([False, True])
+        print(f"random case {it}: N={N} H={H} V={V} {dt} w={wdt} ign={ign} zreg={zreg} scale={scale} chunk={nc} "
+              f"mon={mon}", flush=True)
+        x, y, w = make_inputs(N, H, V, dt, seed=100 + it, ignore_frac=ign, w_dtype=wdt)
+        if (y != -1).sum() == 0:
+            y[0] = 0
+        out, dx, dw = _run(x, y, w, -1, zreg, scale, nc, mon, grad_output=1.3)
+        ref = _oracle(x, y, w, -1, zreg, scale, grad_output=1.3)
+        assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item()), it
+        if mon:
+            assert abs(out[2].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item()) + 1e-3, it
+            assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item()) + 1e-4, it
+            assert abs(out[4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item()), it
+        for got, want in ((dx, ref.dx), (dw, ref.dw)):
+            emax, el2 = rel_errors(got, want)
+            assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (it, emax, el2)
+        assert (dx.cpu()[y == -1] == 0).all(), it
