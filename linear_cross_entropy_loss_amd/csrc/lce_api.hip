@@ -110,7 +110,7 @@ size_t dw_part_bytes(size_t Np, size_t Hp, int64_t vs, int64_t last_vs) {
 // meet it (the fp32 running dx alone is larger, and a split into very narrow
 // slabs leaves the GPU idle); for those the bound is widened by N * H * 4 bytes,
 // the fp32 x_grad buffer the reference allocates next to its logits chunk
-// (ops.py:693) and this library does not.  If even that fails, the narrowest
+// (ops.py:693) and this library does not -- and by the split-K partial sums.  If even that fails, the narrowest
 // split is used: the bound is a target, the operator never refuses a shape.
 int plan_bwd(const lce_problem* p, BwdPlan* b) {
   const size_t strict = (size_t)p->n_chunk * (size_t)p->V * 4;
@@ -130,7 +130,10 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
       const size_t dxp = dx_part_bytes(Np, Hp, vs), dwp = dw_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
       const size_t part = dxp + dwp;
       const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2) : 0;  // 16-bit copy of the slab of W
-      if ((dz + acc + part + w16 <= budget && (dz <= dz_cap || vs == 256)) || (pass == 1 && vs == 256)) {
+      // the widened bound of the second pass is for the staging proper; the split-K partial sums
+      // (at most 64 MiB each for dx and dW) come on top of it there
+      const size_t counted = dz + acc + w16 + (pass == 0 ? part : 0);
+      if ((counted <= budget && (dz <= dz_cap || vs == 256)) || (pass == 1 && vs == 256)) {
         b->slabs = slabs;
         b->vs = vs;
         b->dz = 0;
