@@ -30,6 +30,12 @@ WORKLOADS = {
                                           z_reg=0.0, scale=1.0, monitoring=False, seed=2),
     "c1_small_N2048_H2048_V16384": dict(N=2048, H=2048, V=16384, dtype="bf16", ignore=0.0, n_chunk=4096,
                                          z_reg=0.0, scale=1.0, monitoring=False, seed=1),
+    # fp16 with every loss feature on, Zipf(1.1) labels, 10 % ignored
+    "c3_f16_N16384_H4096_V131072_all_features": dict(N=16384, H=4096, V=131072, dtype="f16", ignore=0.10, n_chunk=4096,
+                                                      z_reg=1e-4, scale=0.5, monitoring=True, seed=3, zipf=True),
+    # long sequence, fp16 activations, fp32 master weight (fp32 dW), Zipf(1.1) labels, 10 % ignored
+    "c5_f16_w32_N65536_H8192_V262144": dict(N=65536, H=8192, V=262144, dtype="f16", w_dtype="f32", ignore=0.10,
+                                             n_chunk=8192, z_reg=0.0, scale=1.0, monitoring=False, seed=5, zipf=True),
 }
 
 
@@ -41,8 +47,15 @@ def make_gpu_inputs(cfg, torch):
     std = 1.0 / math.sqrt(H)
     w = torch.empty(H, V, device="cuda", dtype=torch.float32)
     torch.nn.init.trunc_normal_(w, mean=0.0, std=std, a=-3 * std, b=3 * std, generator=g)
-    w = w.to(dt)
-    y = torch.randint(0, V, (N,), device="cuda", generator=g)
+    if cfg.get("w_dtype") != "f32":
+        w = w.to(dt)
+    if cfg.get("zipf"):
+        p = torch.arange(1, V + 1, dtype=torch.float64, device="cuda") ** -1.1
+        cdf = torch.cumsum(p, 0) / p.sum()
+        u = torch.rand(N, device="cuda", generator=g, dtype=torch.float64)
+        y = torch.searchsorted(cdf, u).clamp_(max=V - 1)
+    else:
+        y = torch.randint(0, V, (N,), device="cuda", generator=g)
     if cfg["ignore"] > 0:
         y[torch.rand(N, device="cuda", generator=g) < cfg["ignore"]] = -1
     return x, y, w
