@@ -198,7 +198,12 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs an AMD GPU (torch.cuda.is_available() is False)", file=sys.stderr)
         sys.exit(1)
-    from linear_cross_entropy_loss_amd import linear_cross_entropy
+    from linear_cross_entropy_loss_amd import _lib, linear_cross_entropy
+
+    if not _lib.LIB_PATH.exists():  # normally built beforehand and shipped with the tree
+        from linear_cross_entropy_loss_amd.build import build
+
+        build(force=True)
 
     cfg = WORKLOADS[args.workload]
     N, H, V = cfg["N"], cfg["H"], cfg["V"]

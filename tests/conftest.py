@@ -12,6 +12,16 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+def pytest_sessionstart(session):
+    """Load what is built; compile the library only when there is none (hipcc cross-compiles without a GPU)."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        from linear_cross_entropy_loss_amd.build import build
+
+        build(force=True)
+
+
 def pytest_collection_modifyitems(config, items):
     import torch
 
