@@ -179,6 +179,14 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
   static constexpr int kPReads = P_KC ? 4 : 8;  // LDS read instructions per k-step
   static constexpr int kQReads = Q_KC ? 4 : 8;
   static constexpr int kReads = kPReads + kQReads;
+  // Fragment reads of the next K step go out early in the current one, so that their data is
+  // back before its first matrix instruction: a quarter of them (2, 3 or 4) after each of the
+  // first four MFMAs.  (One per MFMA, or all of them in one go, both measure slower.)
+  static constexpr int kReadsPerSlot = kReads / 4;
+  // Rows of MFMAs of the last K step that run before the workgroup barrier.  The earlier the
+  // barrier, the more time the first fragment reads of the next K tile have; with 16 of them
+  // (both operands transposed) the barrier opens the step, otherwise one row precedes it.
+  static constexpr int kPreRows = kReads > 12 ? 0 : 1;
 
   LCE_DEV Pipe3(Problem& p) : prob(p) {}
 
@@ -217,9 +225,9 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
   }
   LCE_DEV void read_frags(int buf, const char* stage, int ks) {
 #pragma unroll
-    for (int b = 0; b < kNB; ++b) pf[buf][b] = pr.read(stage, b, ks);
-#pragma unroll
     for (int b = 0; b < kNB; ++b) qf[buf][b] = qr.read(stage + kTileBytes, b, ks);
+#pragma unroll
+    for (int b = 0; b < kNB; ++b) pf[buf][b] = pr.read(stage, b, ks);
   }
   template <bool ZERO> LCE_DEV void mfma_rows(f32x16_t (&acc)[kNB][kNB], int buf, int i0, int i1) {
 #pragma unroll
@@ -254,7 +262,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
-      if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
+      if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
       if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -267,7 +275,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
-      if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
+      if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
       if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
       if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 0..5: P
     }
@@ -281,24 +289,26 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
-      if (i < kReads) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, 1, 0);
+      if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
       if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
       if (i >= 6 && i < 10 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 6, 7: P
       if (i >= 10 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);           // chunks 8..10: Q
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    // k-step 3: first half with loads 11..15; barrier; reads for the next K tile's step 0; second half
-    load_chunks(sp, sq, 11, 16);
-    mfma_rows<false>(acc, 1, 0, kNB / 2);
+    // k-step 3: kPreRows rows of MFMAs with loads 11..; barrier; reads for the next K tile's step 0; the rest
+    constexpr int kPre = 4 * kPreRows, kPreLoads = kPre < 5 ? kPre : 5;
+    load_chunks(sp, sq, 11, 11 + kPreLoads);
+    mfma_rows<false>(acc, 1, 0, kPreRows);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kPre; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
-      if (i < 5) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);  // chunks 11..15: Q
+      if (i < kPreLoads) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);  // chunks 11..: Q
     }
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     if (!LAST) read_frags(0, nxt, 0);
+    load_chunks(sp, sq, 11 + kPreLoads, 16);
     // The fetch stream moves on to K tile t+3 (first needed by the next step's loads).  Its scalar
     // address / range arithmetic sits in this region so that it issues between the MFMAs below.
     if (WRAP) {
@@ -306,13 +316,12 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
     } else {
       stream_advance();
     }
-    mfma_rows<false>(acc, 1, kNB / 2, kNB);
-    if (!LAST) {
+    mfma_rows<false>(acc, 1, kPreRows, kNB);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
-        if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, (kReads + 3) / 4, 0);
-      }
+    for (int i = 0; i < 16 - kPre; ++i) {
+      __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
+      if (!LAST && i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
+      if (i >= 4 && i < 4 + 5 - kPreLoads) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
