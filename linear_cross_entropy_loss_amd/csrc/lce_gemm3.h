@@ -223,11 +223,18 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
     if (c0 < 8) ps.load(sp, c0, c1 < 8 ? c1 : 8);
     if (c1 > 8) qs.load(sq, c0 > 8 ? c0 - 8 : 0, c1 - 8);
   }
+  // The order of the two operands' reads is a measured choice (about 1 % either way).
   LCE_DEV void read_frags(int buf, const char* stage, int ks) {
+    if (kReads > 12) {
+#pragma unroll
+      for (int b = 0; b < kNB; ++b) pf[buf][b] = pr.read(stage, b, ks);
+    }
 #pragma unroll
     for (int b = 0; b < kNB; ++b) qf[buf][b] = qr.read(stage + kTileBytes, b, ks);
+    if (kReads <= 12) {
 #pragma unroll
-    for (int b = 0; b < kNB; ++b) pf[buf][b] = pr.read(stage, b, ks);
+      for (int b = 0; b < kNB; ++b) pf[buf][b] = pr.read(stage, b, ks);
+    }
   }
   template <bool ZERO> LCE_DEV void mfma_rows(f32x16_t (&acc)[kNB][kNB], int buf, int i0, int i1) {
 #pragma unroll
@@ -267,32 +274,32 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    // k-step 1: MFMAs on buffer 1; reads for step 2; stores 6..10; loads 0..5
+    // k-step 1: MFMAs on buffer 1; reads for step 2; stores 6..11 (in slots the reads leave free); loads 0..5
     read_frags(0, cur, 2);
-    store_chunks(sp, sq, nxt, 6, 11);
+    store_chunks(sp, sq, nxt, 6, 12);
     load_chunks(sp, sq, 0, 6);
     mfma_rows<false>(acc, 1, 0, kNB);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
-      if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
+      if (i >= 5 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
       if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 0..5: P
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    // k-step 2: MFMAs on buffer 0; reads for step 3; stores 11..15; loads 6..10
+    // k-step 2: MFMAs on buffer 0; reads for step 3; stores 12..15; loads 6..10
     read_frags(1, cur, 3);
-    store_chunks(sp, sq, nxt, 11, 16);
+    store_chunks(sp, sq, nxt, 12, 16);
     load_chunks(sp, sq, 6, 11);
     mfma_rows<false>(acc, 0, 0, kNB);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
-      if (i >= 1 && i < 11 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
-      if (i >= 6 && i < 10 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 6, 7: P
-      if (i >= 10 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);           // chunks 8..10: Q
+      if (i >= 4 && i < 12 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
+      if (i >= 5 && i < 9 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 6, 7: P
+      if (i >= 9 && i < 15 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);  // chunks 8..10: Q
     }
     __builtin_amdgcn_sched_barrier(0);
 
