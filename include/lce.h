@@ -19,6 +19,10 @@
  *     reference's divisibility rules (N % 512, H % 256, V % 4096,
  *     ops.py:689-691, 905-907) are lifted; shapes that obey them run at full
  *     speed, others pay for partly empty tiles.
+ *     256 rows of x, of a 16-bit w and of dx must span less than 2 GiB (row
+ *     stride in bytes <= 8 MiB, i.e. 4 Mi elements of 16-bit data), and
+ *     ceil(N/256) * ceil(V/256) <= 2^28; beyond that the calls return
+ *     LCE_EINVAL_ARG / LCE_EINVAL_SHAPE.
  *   - Row strides keep every row 16-byte aligned: ldx, ldw (and lddw for a
  *     16-bit dW) are multiples of 8 elements for 16-bit data, 4 for fp32; lddx
  *     is a multiple of 4.  A stride larger than the row length is fine.  When

@@ -34,11 +34,19 @@ int check(const lce_problem* p, bool backward) {
   if (!(p->logit_scale > 0.f) || !(p->z_reg >= 0.f)) return LCE_EINVAL_ARG;
   const int64_t xa = xd == LCE_F32 ? 4 : 8, wa = wd == LCE_F32 ? 4 : 8;  // 16-byte rows
   if (p->ldx < p->H || p->ldx % xa || p->ldw < p->V || p->ldw % wa) return LCE_EINVAL_ARG;
+  // The kernels address a 256-row tile of x, of a 16-bit W and of dx with 32-bit byte offsets: 256 rows must
+  // stay below 2 GiB.  (An fp32 W is only read by the slab conversion, which uses 64-bit addresses.)
+  const int64_t tile_limit = ((int64_t)1 << 31) / 256;
+  if (p->ldx * (xd == LCE_F32 ? 4 : 2) > tile_limit) return LCE_EINVAL_ARG;
+  if (is16(wd) && p->ldw * 2 > tile_limit) return LCE_EINVAL_ARG;
+  // tile and work-item counts are 32-bit
+  if (lce::padded_tokens(p->N) / 256 * (lce::padded_vocab(p->V) / 256) > (int64_t)1 << 28) return LCE_EINVAL_SHAPE;
   if (backward) {
     if (p->dx_dtype != xd && p->dx_dtype != LCE_F32) return LCE_EINVAL_DTYPE;
     if (p->dw_dtype != wd && p->dw_dtype != LCE_F32) return LCE_EINVAL_DTYPE;
     // dx is stored in 8-byte (16-bit types) or 16-byte pieces, dW in 16-byte pieces
     if (p->lddx < p->H || p->lddx % 4 || p->lddw < p->V || p->lddw % (p->dw_dtype == LCE_F32 ? 4 : 8)) return LCE_EINVAL_ARG;
+    if (p->lddx * (p->dx_dtype == LCE_F32 ? 4 : 2) > tile_limit) return LCE_EINVAL_ARG;
   }
   return LCE_OK;
 }

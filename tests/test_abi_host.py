@@ -73,6 +73,14 @@ def test_shape_contract(lib):
     assert lib.lce_check_problem(ctypes.byref(_prob(x_dtype=torch.bfloat16, w_dtype=torch.float16))) == _lib.LCE_EINVAL_DTYPE
     assert lib.lce_check_problem(ctypes.byref(_prob(x_dtype=torch.float32, w_dtype=torch.bfloat16))) == _lib.LCE_EINVAL_DTYPE
     assert lib.lce_check_problem(ctypes.byref(_prob(w_dtype=torch.float32, dw_dtype=torch.float32))) == _lib.LCE_OK
+    # 32-bit tile addressing: 256 rows of x, of a 16-bit w and of dx stay below 2 GiB; an fp32 w is exempt
+    big = (1 << 22) + 8
+    assert lib.lce_check_problem(ctypes.byref(_prob(V=4096, ldw=big, lddw=big))) == _lib.LCE_EINVAL_ARG
+    assert lib.lce_check_problem(ctypes.byref(_prob(V=4096, ldw=1 << 22, lddw=1 << 22))) == _lib.LCE_OK
+    assert lib.lce_check_problem(ctypes.byref(_prob(V=4096, ldw=big, lddw=big, w_dtype=torch.float32, dw_dtype=torch.float32))) == _lib.LCE_OK
+    assert lib.lce_check_problem(ctypes.byref(_prob(ldx=big))) == _lib.LCE_EINVAL_ARG
+    assert lib.lce_check_problem(ctypes.byref(_prob(lddx=big))) == _lib.LCE_EINVAL_ARG
+    assert lib.lce_check_problem(ctypes.byref(_prob(N=1 << 30, V=1 << 20, ldw=1 << 20, lddw=1 << 20))) == _lib.LCE_EINVAL_SHAPE
     assert lib.lce_check_problem(None) == _lib.LCE_EINVAL_ARG
 
 
