@@ -377,14 +377,19 @@ def test_function_and_registered_operator_agree_bitwise():
     print("Function vs operator", flush=True)
     x, y, w = make_inputs(777, 264, 10008, torch.float16, seed=10, ignore_frac=0.1, device="cuda")
     res = []
-    for fn in (LinearXentImplementation.apply, linear_cross_entropy):
+
+    def via_operator(x, y, w, *cfg):  # what linear_cross_entropy calls while torch.compile traces
+        return torch.ops.lce_amd.forward(x, y, w, *cfg)[0].unbind(0)
+
+    for fn in (LinearXentImplementation.apply, linear_cross_entropy, via_operator):
         xi = x.clone().requires_grad_(True)
         wi = w.clone().requires_grad_(True)
         out = fn(xi, y, wi, -1, 1e-4, 0.5, 512, True)
         out[0].backward()
         res.append((torch.stack([o.detach() for o in out]), xi.grad, wi.grad))
-    for a, b in zip(*res):
-        assert torch.equal(a, b)
+    for other in res[1:]:
+        for a, b in zip(res[0], other):
+            assert torch.equal(a, b)
 
 
 def test_forward_backward_can_be_captured_in_a_hip_graph():
