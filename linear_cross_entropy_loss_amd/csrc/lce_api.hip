@@ -179,12 +179,14 @@ const char* lce_strerror(int status) {
   switch (status) {
     case LCE_OK: return "ok";
     case LCE_EINVAL_SHAPE:
-      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N, V <= 2^30, H <= 2^20)";
+      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N, V <= 2^30, H <= 2^20; "
+             "ceil(N/256) * ceil(V/256) <= 2^28)";
     case LCE_EINVAL_DTYPE:
       return "unsupported dtype combination (x: bf16/f16/f32; w: x dtype or f32; grads: same dtype or f32)";
     case LCE_EINVAL_ARG:
       return "invalid argument (null or misaligned pointer; row strides must be >= the row length and multiples of 8 "
-             "elements for 16-bit data, 4 for fp32; logit_scale <= 0 or z_reg < 0)";
+             "elements for 16-bit data, 4 for fp32, and at most 8 MiB for x, a 16-bit w and dx; logit_scale <= 0 or "
+             "z_reg < 0)";
     case LCE_EWORKSPACE: return "workspace missing or too small for this problem and N_chunk_size";
     case LCE_EHIP: return "HIP error";
     default: return "unknown status";
