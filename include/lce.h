@@ -87,14 +87,15 @@ typedef struct lce_problem {
  * Profiling aid: a non-zero lce_problem.phases restricts a call to the named
  * kernels so that each can be bracketed by events.  Results of a restricted
  * call are only meaningful if the skipped phases ran before on the same
- * buffers.
+ * buffers and the same workspace (that of the same entry point).
  */
 enum {
   LCE_PHASE_FWD_TILES = 1,  /* lce_forward: the MFMA tile kernel            */
   LCE_PHASE_FWD_REDUCE = 2, /* lce_forward: row merge + final reduction     */
   LCE_PHASE_BWD_DZ = 4,     /* lce_backward: recompute + dz staging         */
   LCE_PHASE_BWD_DX = 8,     /* lce_backward: dx contraction                 */
-  LCE_PHASE_BWD_DW = 16     /* lce_backward: dW contraction                 */
+  LCE_PHASE_BWD_DW = 16,    /* lce_backward: dW contraction                 */
+  LCE_PHASE_PACK = 32       /* either call: packing of the tokens whose label is not ignore_index */
 };
 
 /* Library version: major*10000 + minor*100 + patch. */
@@ -136,7 +137,9 @@ int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width)
  * (ops.py:722-752) and the torch reductions around it (ops.py:705, 753-761,
  * 793-794, 802), without ever writing logits to memory.
  *
- *   lse     out, N floats: logsumexp of the scaled logits of every row
+ *   lse     out, N floats: logsumexp of the scaled logits of every row whose
+ *           label is not ignore_index (with monitoring == 0 the other rows
+ *           are not computed at all and get 0)
  *   out5    out, 5 floats: loss, z_reg, logit_max, logit_entropy, logit_norm
  *           (the 5-tuple of ops.py:802 with the meanings of ops.py:9-17; the
  *           last three are 0 when monitoring == 0)

@@ -11,7 +11,7 @@ LIB_PATH = _PKG_DIR / "liblce_gfx950.so"
 
 LCE_BF16, LCE_F16, LCE_F32 = 0, 1, 2
 LCE_OK = 0
-PHASE_FWD_TILES, PHASE_FWD_REDUCE, PHASE_BWD_DZ, PHASE_BWD_DX, PHASE_BWD_DW = 1, 2, 4, 8, 16
+PHASE_FWD_TILES, PHASE_FWD_REDUCE, PHASE_BWD_DZ, PHASE_BWD_DX, PHASE_BWD_DW, PHASE_PACK = 1, 2, 4, 8, 16, 32
 LCE_EINVAL_SHAPE, LCE_EINVAL_DTYPE, LCE_EINVAL_ARG, LCE_EWORKSPACE, LCE_EHIP = -1, -2, -3, -4, -5
 
 EXPORTS = (

@@ -15,7 +15,7 @@ CSRC = PKG_DIR / "csrc"
 LIB_NAME = "liblce_gfx950.so"
 LIB_PATH = PKG_DIR / LIB_NAME
 
-SOURCES = ["lce_api.hip", "lce_fwd.hip", "lce_bwd_dz.hip", "lce_bwd_dx.hip", "lce_bwd_dw.hip", "lce_convert.hip"]
+SOURCES = ["lce_api.hip", "lce_fwd.hip", "lce_bwd_dz.hip", "lce_bwd_dx.hip", "lce_bwd_dw.hip", "lce_convert.hip", "lce_compact.hip"]
 
 # Packed-fp32 VALU forms are disabled for all device code.
 HIPCC_FLAGS = [

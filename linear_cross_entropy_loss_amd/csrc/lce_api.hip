@@ -51,8 +51,29 @@ int check(const lce_problem* p, bool backward) {
   return LCE_OK;
 }
 
+// Buffers of the packing pre-pass (tokens with an ignored label dropped), relative to `base`.
+struct PackPlan {
+  size_t cnt, n_rows, perm, yc, xc, end;
+  int64_t ldxc;  // row stride of the packed copy of x, elements: rows of whole 16-byte pieces
+};
+
+PackPlan plan_pack(const lce_problem* p, size_t base) {
+  PackPlan k;
+  const size_t N = (size_t)p->N, es = p->x_dtype == LCE_F32 ? 4 : 2;
+  k.ldxc = lce::pad_to(p->H, (int64_t)(16 / es));
+  size_t o = base;
+  k.cnt = o; o += align_up((size_t)lce::compact_segments(p->N) * 4);
+  k.n_rows = o; o += 256;
+  k.perm = o; o += align_up(N * 4);
+  k.yc = o; o += align_up(N * 8);
+  k.xc = o; o += align_up(N * (size_t)k.ldxc * es);
+  k.end = o;
+  return k;
+}
+
 struct FwdPlan {
   size_t part_lse, part_max, part_pz, part_sq, tgt, blk, w16, total;
+  PackPlan pack;  // only when monitoring is off (the monitoring values are taken over all rows)
   int64_t vs;  // columns per forward launch: all of V, or the width of the 16-bit slab copy of an fp32 weight
 };
 
@@ -79,12 +100,19 @@ FwdPlan plan_fwd(const lce_problem* p) {
     if (cols < f.vs) f.vs = cols;
     o += align_up((size_t)p->H * (size_t)f.vs * 2);
   }
+  if (!p->monitoring) {
+    f.pack = plan_pack(p, o);
+    o = f.pack.end;
+  }
   f.total = o;
   return f;
 }
 
 struct BwdPlan {
   int64_t slabs, vs;
+  PackPlan pack;
+  size_t lse_c, dxc;  // lse of the packed rows; packed dx before it is moved to its place
+  int64_t lddxc;
   size_t dz, dx_acc, dx_part, dw_part, w16, total;
 };
 
@@ -126,6 +154,12 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   const size_t Np = (size_t)lce::padded_tokens(p->N), Hp = (size_t)lce::padded_hidden(p->H);
   const int64_t Vp = lce::padded_vocab(p->V);
   const int64_t cols = Vp / 256;
+  // buffers of the packed rows come first and count towards the bound
+  b->pack = plan_pack(p, 0);
+  b->lddxc = lce::pad_to(p->H, 8);
+  b->lse_c = b->pack.end;
+  b->dxc = b->lse_c + align_up((size_t)p->N * 4);
+  const size_t fixed = b->dxc + align_up((size_t)p->N * (size_t)b->lddxc * (p->dx_dtype == LCE_F32 ? 4 : 2));
   for (int pass = 0; pass < 2; ++pass) {
     const size_t budget = strict + (pass ? (size_t)p->N * (size_t)p->H * 4 : 0);
     for (int64_t s = 1; s <= cols; ++s) {
@@ -139,17 +173,17 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
       const size_t part = dxp + dwp;
       const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2) : 0;  // 16-bit copy of the slab of W
       // the widened bound of the second pass is for the staging proper; the split-K partial sums
-      // (at most 64 MiB each for dx and dW) come on top of it there
-      const size_t counted = dz + acc + w16 + (pass == 0 ? part : 0);
+      // (at most 64 MiB each for dx and dW) and the packed rows come on top of it there
+      const size_t counted = dz + acc + w16 + (pass == 0 ? fixed + part : 0);
       if ((counted <= budget && (dz <= dz_cap || vs == 256)) || (pass == 1 && vs == 256)) {
         b->slabs = slabs;
         b->vs = vs;
-        b->dz = 0;
-        b->dx_acc = dz;
-        b->dx_part = dz + acc;
-        b->dw_part = dz + acc + dxp;
-        b->w16 = dz + acc + part;
-        b->total = dz + acc + part + w16;
+        b->dz = fixed;
+        b->dx_acc = fixed + dz;
+        b->dx_part = fixed + dz + acc;
+        b->dw_part = fixed + dz + acc + dxp;
+        b->w16 = fixed + dz + acc + part;
+        b->total = fixed + dz + acc + part + w16;
         return LCE_OK;
       }
     }
@@ -252,6 +286,25 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
 
   const int ph = p->phases ? p->phases : ~0;
   hipError_t e;
+  if (!p->monitoring) {
+    // Tokens with an ignored label add nothing to the loss: the tile kernel runs on the others only.
+    const PackPlan& k = f.pack;
+    a.n_rows = (const int64_t*)(base + k.n_rows);
+    a.perm = (const int*)(base + k.perm);
+    a.xc = base + k.xc;
+    a.ldxc = k.ldxc;
+    a.y0 = y;
+    a.y = (const int64_t*)(base + k.yc);
+    if (ph & LCE_PHASE_PACK) {
+      e = lce::launch_compact_labels(y, p->N, p->ignore_index, (int*)(base + k.cnt), (int64_t*)(base + k.n_rows),
+                                     (int*)(base + k.perm), (int64_t*)(base + k.yc), s);
+      if (e != hipSuccess) return hip_fail(e, "compact_labels");
+      const int64_t es = p->x_dtype == LCE_F32 ? 4 : 2;
+      e = lce::launch_gather_rows(x, p->ldx * es, a.perm, a.n_rows, p->N, base + k.xc, k.ldxc * es, nullptr,
+                                  nullptr, a.num_cus, s);
+      if (e != hipSuccess) return hip_fail(e, "gather_rows");
+    }
+  }
   if (ph & LCE_PHASE_FWD_TILES) {
     // One launch over the whole vocabulary, or -- fp32 weight -- one per slab, each on a
     // 16-bit copy of its columns made just before it (same stream, one buffer).
@@ -310,6 +363,25 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   if (rc != LCE_OK) return rc;
   const int ph = p->phases ? p->phases : ~0;
 
+  // Tokens with an ignored label have dz == 0: the kernels run on the other rows only, packed to the front.
+  const PackPlan& k = b.pack;
+  const int64_t xes = p->x_dtype == LCE_F32 ? 4 : 2, dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
+  a.n_rows = (const int64_t*)(base + k.n_rows);
+  a.xc = base + k.xc;
+  a.ldxc = k.ldxc;
+  a.dxc = base + b.dxc;
+  a.lddxc = b.lddxc;
+  a.y = (const int64_t*)(base + k.yc);
+  a.lse = (const float*)(base + b.lse_c);
+  if (ph & LCE_PHASE_PACK) {
+    hipError_t e = lce::launch_compact_labels(y, p->N, p->ignore_index, (int*)(base + k.cnt), (int64_t*)(base + k.n_rows),
+                                              (int*)(base + k.perm), (int64_t*)(base + k.yc), s);
+    if (e != hipSuccess) return hip_fail(e, "compact_labels");
+    e = lce::launch_gather_rows(x, p->ldx * xes, (const int*)(base + k.perm), a.n_rows, p->N, base + k.xc, k.ldxc * xes,
+                                lse, (float*)(base + b.lse_c), a.num_cus, s);
+    if (e != hipSuccess) return hip_fail(e, "gather_rows");
+  }
+
   for (int64_t i = 0; i < b.slabs; ++i) {
     a.v0 = i * b.vs;
     a.vw = p->V - a.v0 < b.vs ? p->V - a.v0 : b.vs;   // columns of this slab that exist
@@ -341,6 +413,12 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
       e = lce::launch_bwd_dw(a, s);
       if (e != hipSuccess) return hip_fail(e, "bwd_dw");
     }
+  }
+  if (dx && (ph & LCE_PHASE_BWD_DX)) {
+    // packed dx rows go to their tokens, dropped tokens get exact zeros (nothing to do if none was dropped)
+    hipError_t e = lce::launch_scatter_rows(a.dxc, b.lddxc * dxes, (const int*)(base + k.perm), a.n_rows, p->N, y,
+                                            p->ignore_index, dx, p->lddx * dxes, p->H * dxes, a.num_cus, s);
+    if (e != hipSuccess) return hip_fail(e, "scatter_rows");
   }
   return LCE_OK;
 }

@@ -93,10 +93,22 @@ template <class T, class XSrc, bool SPLIT> struct DwProblem {
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
+  int64_t rows, ldx;  // token rows (the K extent): all of x, or the packed rows (see BwdArgs)
+  const XSrc* x;
   int tiles_p, tiles_q, split, kseg;
   LCE_DEV DwProblem(const BwdArgs& a_)
       : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.Hp / kTile)), split(SPLIT ? a_.dw_split : 1),
-        kseg(a_.dw_kseg) {}
+        kseg(a_.dw_kseg) {
+    rows = packed_rows(a.n_rows, a.N);
+    const bool packed = rows != a.N;
+    x = reinterpret_cast<const XSrc*>(packed ? a.xc : a.x);
+    ldx = packed ? a.ldxc : a.ldx;
+  }
+  // K tiles of an unsplit contraction: an even number, at least four, covering the rows
+  LCE_DEV int ktiles() const {
+    const int64_t kt = (rows + 2 * kBK - 1) / (2 * kBK) * 2;
+    return (int)(kt < 4 ? 4 : kt);
+  }
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q * split; }
   LCE_DEV void decode(int item, int& tp, int& tq, int& seg) const {
     seg = SPLIT ? item % split : 0;
@@ -107,11 +119,14 @@ template <class T, class XSrc, bool SPLIT> struct DwProblem {
     decode(item, tp, tq, seg);
     const int64_t k0 = (int64_t)seg * kseg * kBK;  // first token of the segment
     p = reinterpret_cast<const E*>(a.dz) + k0 * a.vs + (int64_t)tp * kTile;
-    q = reinterpret_cast<const XSrc*>(a.x) + k0 * a.ldx + (int64_t)tq * kTile;
+    q = x + k0 * ldx + (int64_t)tq * kTile;
   }
   // rows past the end of either operand (a last segment running past the tokens) read as zeros
-  LCE_DEV const void* p_end() const { return reinterpret_cast<const E*>(a.dz) + a.Np * a.vs; }
-  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
+  // dz is written for whole token tiles; x rows past the last one read as zeros
+  LCE_DEV const void* p_end() const {
+    return reinterpret_cast<const E*>(a.dz) + (rows + kTile - 1) / kTile * kTile * a.vs;
+  }
+  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.Np; }
   LCE_DEV void epilogue(int item, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq, seg;
@@ -130,7 +145,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdAr
   typedef typename elem_of<T>::type E;
   DwProblem<T, XSrc, SPLIT> prob(a);
   Pipe3<T, E, false, XSrc, false, DwProblem<T, XSrc, SPLIT>> pipe(prob);
-  pipe.run(a.vs, a.ldx, SPLIT ? a.dw_kseg : (int)(a.Np / kBK), lds);
+  pipe.run(a.vs, prob.ldx, SPLIT ? a.dw_kseg : prob.ktiles(), lds);
 }
 
 // Split mode, second step: dW[:, slab] = coef * sum over segments, in segment order.

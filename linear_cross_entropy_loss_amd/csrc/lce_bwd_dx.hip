@@ -17,8 +17,10 @@ namespace {
 // out-of-range offset (a quad that H cuts through is written whole: the row
 // stride is a multiple of 4, so it stays inside its row).  No branches: a branch
 // around accumulator reads makes the compiler read all of them up front.
+// `out` / `ldo` / `rows`: dx itself, or the packed copy when tokens were dropped (see BwdArgs).
 template <class T>
-LCE_DEV void dx_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
+LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo, f32x16_t (&acc)[kNB][kNB], int tp,
+                         int tq) {
   typedef typename elem_of<T>::type E;
   const int64_t h0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
   const int tid = opaque_tid();
@@ -27,17 +29,17 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
   const int es = a.dx_dtype == DT_F32 ? 4 : 2;
   // descriptor over the rows of this tile: base = first row, range = bytes to the end of dx
-  const char* tile_base = reinterpret_cast<const char*>(a.dx) + t0 * a.lddx * es;
+  const char* tile_base = reinterpret_cast<const char*>(out) + t0 * ldo * es;
   // whole dwords: with 16-bit data and an odd H the last row ends one element into its stride padding
   const int64_t hcols = es == 2 ? (a.H + 1) & ~(int64_t)1 : a.H;
-  const int64_t left = (reinterpret_cast<const char*>(a.dx) + ((a.N - 1) * a.lddx + hcols) * es) - tile_base;
+  const int64_t left = (reinterpret_cast<const char*>(out) + ((rows - 1) * ldo + hcols) * es) - tile_base;
   const unsigned range = left <= 0 ? 0u : (left > 0x7fffffff ? 0x7fffffffu : (unsigned)left);
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(tile_base), 0, (int)range, 0x00020000);
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
     const int row = wq * kWaveTile + qb * kBlk + (lane & 31);  // row inside the tile
     const int64_t tok = t0 + row;
-    const unsigned row_off = (unsigned)(row * a.lddx * es);
+    const unsigned row_off = (unsigned)(row * ldo * es);
 #pragma unroll
     for (int pb = 0; pb < kNB; ++pb)
 #pragma unroll
@@ -99,10 +101,12 @@ template <class T, class WSrc, bool SPLIT, bool KMASK> struct DxProblem {
   static constexpr bool kKMask = KMASK;
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
+  int64_t rows;  // token rows: all, or the packed ones (see BwdArgs)
   int tiles_p, tiles_q, split, kseg;
   LCE_DEV DxProblem(const BwdArgs& a_)
-      : a(a_), tiles_p((int)(a_.Hp / kTile)), tiles_q((int)(a_.Np / kTile)), split(SPLIT ? a_.dx_split : 1),
-        kseg(a_.dx_kseg) {}
+      : a(a_), rows(packed_rows(a_.n_rows, a_.N)), tiles_p((int)(a_.Hp / kTile)), split(SPLIT ? a_.dx_split : 1), kseg(a_.dx_kseg) {
+    tiles_q = (int)((rows + kTile - 1) / kTile);
+  }
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q * split; }
   LCE_DEV void decode(int item, int& tp, int& tq, int& seg) const {
     seg = SPLIT ? item % split : 0;
@@ -116,7 +120,7 @@ template <class T, class WSrc, bool SPLIT, bool KMASK> struct DxProblem {
     q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs + k0;
   }
   LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
-  LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + a.Np * a.vs; }
+  LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + (int64_t)tiles_q * kTile * a.vs; }
   LCE_DEV int k_valid(int item) const {
     const int seg = SPLIT ? item % split : 0;
     const int64_t left = a.vw - (int64_t)seg * kseg * kBK;
@@ -128,7 +132,8 @@ template <class T, class WSrc, bool SPLIT, bool KMASK> struct DxProblem {
     if (SPLIT) {
       dx_partial_epilogue(a, acc, tp, tq, seg);
     } else {
-      dx_epilogue<T>(a, acc, tp, tq);
+      const bool packed = rows != a.N;
+      dx_epilogue<T>(a, rows, packed ? a.dxc : a.dx, packed ? a.lddxc : a.lddx, acc, tp, tq);
     }
   }
 };
@@ -148,7 +153,11 @@ template <class T>
 __global__ __launch_bounds__(256) void dx_reduce_kernel(const BwdArgs a) {
   typedef typename elem_of<T>::type E;
   const int64_t quads_per_row = a.Hp / 4;
-  const int64_t total = a.N * quads_per_row;
+  const int64_t rows = packed_rows(a.n_rows, a.N);
+  const int64_t total = rows * quads_per_row;
+  const bool packed = rows != a.N;
+  void* out = packed ? a.dxc : a.dx;
+  const int64_t ldo = packed ? a.lddxc : a.lddx;
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t tok = i / quads_per_row, h = (i - tok * quads_per_row) * 4;
@@ -160,12 +169,12 @@ __global__ __launch_bounds__(256) void dx_reduce_kernel(const BwdArgs a) {
     if (!a.last) {
       *reinterpret_cast<f32x4_t*>(a.dx_acc + o) = v;
     } else if (a.dx_dtype == DT_F32) {
-      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dx) + tok * a.lddx + h) = v * coef;
+      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + tok * ldo + h) = v * coef;
     } else {
       u32x2_t b;
       b[0] = pack2<T>(v[0] * coef, v[1] * coef);
       b[1] = pack2<T>(v[2] * coef, v[3] * coef);
-      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dx) + tok * a.lddx + h) = b;
+      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(out) + tok * ldo + h) = b;
     }
   }
 }

@@ -45,7 +45,7 @@ static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must
 // one run that V cuts through is handled element by element.  Columns outside
 // are written as exact zeros.
 template <class T, bool ZREG, bool VTAIL>
-LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
+LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
   typedef typename elem_of<T>::type E;
   const int64_t v0 = a.v0 + (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
   const int tid = opaque_tid();
@@ -68,7 +68,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
     const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-    const bool exists = tok < a.N;  // rows past N are staged as zeros, like ignored tokens
+    const bool exists = tok < rows;  // rows past the last one are staged as zeros, like ignored tokens
     const int64_t yy = exists ? a.y[tok] : a.ignore_index;
     const int64_t rel = yy - slice_v0;
     const bool valid = yy != a.ignore_index;
@@ -170,10 +170,18 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int t
 template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK> struct DzProblem {
   static constexpr bool kKMask = KMASK;
   const BwdArgs& a;
+  int64_t rows, ldx;  // token rows: all of x, or the packed rows (see BwdArgs)
+  const XSrc* x;
   int tp0, tiles_p, tiles_q;
   LCE_DEV DzProblem(const BwdArgs& a_)
       : a(a_), tp0(VTAIL ? (int)(a_.vw / kTile) : 0),
-        tiles_p(VTAIL ? (int)(a_.vs / kTile - a_.vw / kTile) : (int)(a_.vw / kTile)), tiles_q((int)(a_.Np / kTile)) {}
+        tiles_p(VTAIL ? (int)(a_.vs / kTile - a_.vw / kTile) : (int)(a_.vw / kTile)) {
+    rows = packed_rows(a.n_rows, a.N);
+    const bool packed = rows != a.N;
+    x = reinterpret_cast<const XSrc*>(packed ? a.xc : a.x);
+    ldx = packed ? a.ldxc : a.ldx;
+    tiles_q = (int)((rows + kTile - 1) / kTile);
+  }
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void coords(int tile, int& tp, int& tq) const {
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
@@ -183,15 +191,15 @@ template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK> st
     int tp, tq;
     coords(tile, tp, tq);
     p = reinterpret_cast<const WSrc*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
-    q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
+    q = x + (int64_t)tq * kTile * ldx;
   }
   LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
-  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
+  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
     coords(tile, tp, tq);
-    dz_epilogue_impl<T, ZREG, VTAIL>(a, acc, tp, tq, scratch);
+    dz_epilogue_impl<T, ZREG, VTAIL>(a, rows, acc, tp, tq, scratch);
   }
 };
 
@@ -200,7 +208,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdAr
   extern __shared__ __attribute__((aligned(16))) char lds[];
   DzProblem<T, XSrc, WSrc, ZREG, VTAIL, KMASK> prob(a);
   Pipe3<T, WSrc, false, XSrc, true, DzProblem<T, XSrc, WSrc, ZREG, VTAIL, KMASK>> pipe(prob);
-  pipe.run(a.ldw, a.ldx, (int)(padded_k(a.H) / kBK), lds);
+  pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
 template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK>

@@ -1,0 +1,175 @@
+// Tokens whose label equals ignore_index contribute nothing to the loss or to
+// either gradient (linear_cross_entropy/ops.py:213, 314, 422), so the tile
+// kernels never look at them: the kept tokens are packed to the front, in
+// their original order, and the kernels run on the packed rows only.  The
+// number of kept tokens stays on the device (the kernels read it), so nothing
+// here synchronises with the host.  (The reference computes the ignored rows
+// and multiplies them away.)
+//
+//   compact_labels  perm[j] = original index of the j-th kept token, yc[j] its label, n_rows = how many
+//   gather_rows     xc[j] = x[perm[j]], lse_c[j] = lse[perm[j]]
+//   scatter_rows    dx[perm[j]] = dxc[j]; rows of dropped tokens = 0
+//
+// When no token is dropped (n_rows == N) the row copies are skipped and the
+// tile kernels read x and write dx in place.
+#include "lce_gemm.h"
+#include "lce_internal.h"
+
+namespace lce {
+
+namespace {
+
+constexpr int kSegTokens = 2048;  // tokens per workgroup of the counting / packing kernels
+constexpr int kPerThread = kSegTokens / 256;
+
+// Sum of `v` over the 256 threads of the workgroup; exclusive prefix of this thread in `excl`.
+LCE_DEV int block_scan(int v, int& excl, int* sh /* [4] */) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  if (lane == 63) sh[wave] = incl;
+  __syncthreads();
+  int before = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    if (w < wave) before += sh[w];
+    total += sh[w];
+  }
+  __syncthreads();  // sh may be reused by the caller
+  excl = before + incl - v;
+  return total;
+}
+
+__global__ __launch_bounds__(256) void count_kept_kernel(const int64_t* y, int64_t N, int64_t ignore_index, int* cnt) {
+  __shared__ int sh[4];
+  const int64_t base = (int64_t)blockIdx.x * kSegTokens + (int64_t)threadIdx.x * kPerThread;
+  int c = 0;
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) c += (base + k < N && y[base + k] != ignore_index) ? 1 : 0;
+  int excl;
+  const int total = block_scan(c, excl, sh);
+  if (threadIdx.x == 0) cnt[blockIdx.x] = total;
+}
+
+// One workgroup: cnt[] becomes its own exclusive prefix sum, n_rows the total.
+__global__ __launch_bounds__(256) void scan_counts_kernel(int* cnt, int64_t nseg, int64_t* n_rows) {
+  __shared__ int sh[4];
+  int64_t running = 0;
+  for (int64_t base = 0; base < nseg; base += 256) {
+    const int64_t i = base + threadIdx.x;
+    const int v = i < nseg ? cnt[i] : 0;
+    int excl;
+    const int total = block_scan(v, excl, sh);
+    if (i < nseg) cnt[i] = (int)(running + excl);
+    running += total;
+  }
+  if (threadIdx.x == 0) n_rows[0] = running;
+}
+
+__global__ __launch_bounds__(256) void pack_kept_kernel(const int64_t* y, int64_t N, int64_t ignore_index,
+                                                        const int* offs, int* perm, int64_t* yc) {
+  __shared__ int sh[4];
+  const int64_t base = (int64_t)blockIdx.x * kSegTokens + (int64_t)threadIdx.x * kPerThread;
+  int64_t lab[kPerThread];
+  int c = 0;
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) {
+    lab[k] = base + k < N ? y[base + k] : ignore_index;
+    c += lab[k] != ignore_index ? 1 : 0;
+  }
+  int excl;
+  block_scan(c, excl, sh);
+  int64_t j = (int64_t)offs[blockIdx.x] + excl;
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k)
+    if (lab[k] != ignore_index) {
+      perm[j] = (int)(base + k);
+      yc[j] = lab[k];
+      ++j;
+    }
+}
+
+// One workgroup per packed row (grid-stride).  Rows are moved in 16-byte pieces; `chunks` pieces per row.
+__global__ __launch_bounds__(256) void gather_rows_kernel(const char* x, int64_t ldx_bytes, const int* perm,
+                                                          const int64_t* n_rows, int64_t N, char* xc,
+                                                          int64_t ldxc_bytes, int chunks, const float* lse,
+                                                          float* lse_c) {
+  const int64_t rows = packed_rows(n_rows, N);
+  const bool copy_x = rows != N;
+  for (int64_t j = blockIdx.x; j < rows; j += gridDim.x) {
+    const int64_t src = packed_token(perm, j, N);
+    if (lse != nullptr && threadIdx.x == 0) lse_c[j] = lse[src];
+    if (copy_x) {
+      const u32x4_t* s = reinterpret_cast<const u32x4_t*>(x + src * ldx_bytes);
+      u32x4_t* d = reinterpret_cast<u32x4_t*>(xc + j * ldxc_bytes);
+      for (int c = threadIdx.x; c < chunks; c += 256) d[c] = s[c];
+    }
+  }
+}
+
+// One workgroup per token (grid-stride): token i moves packed row i to its place (if there is a packed
+// row i) and clears its own row of dx if it was dropped.  8-byte pieces, `chunks` per row.
+__global__ __launch_bounds__(256) void scatter_rows_kernel(const char* dxc, int64_t lddxc_bytes, const int* perm,
+                                                           const int64_t* n_rows, int64_t N, const int64_t* y,
+                                                           int64_t ignore_index, char* dx, int64_t lddx_bytes,
+                                                           int chunks) {
+  const int64_t rows = packed_rows(n_rows, N);
+  if (rows == N) return;  // nothing was dropped: the tile kernel wrote dx itself
+  for (int64_t i = blockIdx.x; i < N; i += gridDim.x) {
+    if (i < rows) {
+      const u32x2_t* s = reinterpret_cast<const u32x2_t*>(dxc + i * lddxc_bytes);
+      u32x2_t* d = reinterpret_cast<u32x2_t*>(dx + packed_token(perm, i, N) * lddx_bytes);
+      for (int c = threadIdx.x; c < chunks; c += 256) d[c] = s[c];
+    }
+    if (y[i] == ignore_index) {
+      u32x2_t* d = reinterpret_cast<u32x2_t*>(dx + i * lddx_bytes);
+      u32x2_t z;
+      z[0] = 0u;
+      z[1] = 0u;
+      for (int c = threadIdx.x; c < chunks; c += 256) d[c] = z;
+    }
+  }
+}
+
+unsigned row_grid(int64_t N, int num_cus) {
+  int64_t g = (int64_t)num_cus * 8;
+  if (g > N) g = N;
+  return (unsigned)(g < 1 ? 1 : g);
+}
+
+}  // namespace
+
+int64_t compact_segments(int64_t N) { return (N + kSegTokens - 1) / kSegTokens; }
+
+hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_index, int* cnt, int64_t* n_rows,
+                                 int* perm, int64_t* yc, hipStream_t s) {
+  const int64_t nseg = compact_segments(N);
+  hipLaunchKernelGGL(count_kept_kernel, dim3((unsigned)nseg), dim3(256), 0, s, y, N, ignore_index, cnt);
+  hipLaunchKernelGGL(scan_counts_kernel, dim3(1), dim3(256), 0, s, cnt, nseg, n_rows);
+  hipLaunchKernelGGL(pack_kept_kernel, dim3((unsigned)nseg), dim3(256), 0, s, y, N, ignore_index, cnt, perm, yc);
+  return hipGetLastError();
+}
+
+hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, const int* perm, const int64_t* n_rows, int64_t N,
+                              void* xc, int64_t ldxc_bytes, const float* lse, float* lse_c, int num_cus,
+                              hipStream_t s) {
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(row_grid(N, num_cus)), dim3(256), 0, s,
+                     reinterpret_cast<const char*>(x), ldx_bytes, perm, n_rows, N, reinterpret_cast<char*>(xc),
+                     ldxc_bytes, (int)(ldxc_bytes / 16), lse, lse_c);
+  return hipGetLastError();
+}
+
+hipError_t launch_scatter_rows(const void* dxc, int64_t lddxc_bytes, const int* perm, const int64_t* n_rows,
+                               int64_t N, const int64_t* y, int64_t ignore_index, void* dx, int64_t lddx_bytes,
+                               int64_t row_bytes, int num_cus, hipStream_t s) {
+  hipLaunchKernelGGL(scatter_rows_kernel, dim3(row_grid(N, num_cus)), dim3(256), 0, s,
+                     reinterpret_cast<const char*>(dxc), lddxc_bytes, perm, n_rows, N, y, ignore_index,
+                     reinterpret_cast<char*>(dx), lddx_bytes, (int)((row_bytes + 7) / 8));
+  return hipGetLastError();
+}
+
+}  // namespace lce

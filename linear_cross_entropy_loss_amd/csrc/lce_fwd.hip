@@ -36,7 +36,7 @@ LCE_DEV float fast_log(float v) { return __builtin_amdgcn_logf(v) * kLn2; }
 // whole, uniformly over the wave, and is taken or skipped with a scalar branch;
 // the one run that V cuts through is handled element by element.
 template <class T, bool VTAIL>
-LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
+LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   const int64_t v0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
   const int tid = opaque_tid();
   const int lane = tid & 63, wave = tid >> 6;
@@ -66,7 +66,7 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, i
       continue;
     }
     // Column of the target inside this wave's 128-wide slice, or -1.
-    const int64_t yy = tok < a.N ? a.y[tok] : a.ignore_index;
+    const int64_t yy = tok < rows ? a.y[tok] : a.ignore_index;
     const int64_t rel = yy - slice_v0;
     const int yl = (yy != a.ignore_index && rel >= 0 && rel < kWaveTile) ? (int)rel : -1;
 
@@ -153,14 +153,22 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, i
 // Persistent workgroups, operand stream pipelined across output tiles.  The
 // launch covers `tiles_p` tile columns of the vocabulary window [v0, v0 + vw)
 // starting at its column tile `tp0` (all full columns, or the one straddling V
-// for the VTAIL variant).
+// for the VTAIL variant).  The token rows are those of x, or -- when the tokens with ignored
+// labels were packed away -- the first `rows` rows of the packed copy (the count lives on the device).
 template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdProblem {
   static constexpr bool kKMask = KMASK;
   const FwdArgs& a;
+  int64_t rows, ldx;
+  const XSrc* x;
   int tp0, tiles_p, tiles_q;
   LCE_DEV FwdProblem(const FwdArgs& a_)
-      : a(a_), tp0(VTAIL ? (int)(a_.vw / kTile) : 0), tiles_p(VTAIL ? 1 : (int)(a_.vw / kTile)),
-        tiles_q((int)(a_.Np / kTile)) {}
+      : a(a_), tp0(VTAIL ? (int)(a_.vw / kTile) : 0), tiles_p(VTAIL ? 1 : (int)(a_.vw / kTile)) {
+    rows = a.n_rows ? packed_rows(a.n_rows, a.N) : a.N;
+    const bool packed = rows != a.N;
+    x = reinterpret_cast<const XSrc*>(packed ? a.xc : a.x);
+    ldx = packed ? a.ldxc : a.ldx;
+    tiles_q = (int)((rows + kTile - 1) / kTile);
+  }
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void coords(int tile, int& tp, int& tq) const {
     tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
@@ -170,15 +178,15 @@ template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdPro
     int tp, tq;
     coords(tile, tp, tq);
     p = reinterpret_cast<const WSrc*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
-    q = reinterpret_cast<const XSrc*>(a.x) + (int64_t)tq * kTile * a.ldx;
+    q = x + (int64_t)tq * kTile * ldx;
   }
   LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
-  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(a.x, a.N, a.ldx, a.H); }
+  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     coords(tile, tp, tq);
-    fwd_epilogue<T, VTAIL>(a, acc, (int)(a.v0 / kTile) + tp, tq);
+    fwd_epilogue<T, VTAIL>(a, rows, acc, (int)(a.v0 / kTile) + tp, tq);
   }
 };
 
@@ -187,7 +195,7 @@ __global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const Fw
   extern __shared__ __attribute__((aligned(16))) char lds[];
   FwdProblem<T, XSrc, WSrc, VTAIL, KMASK> prob(a);
   Pipe3<T, WSrc, false, XSrc, true, FwdProblem<T, XSrc, WSrc, VTAIL, KMASK>> pipe(prob);
-  pipe.run(a.ldw, a.ldx, (int)(padded_k(a.H) / kBK), lds);
+  pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
 // One workgroup = 64 tokens x 4 strided groups of slices.
@@ -196,8 +204,11 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
   __shared__ float sh_pz[4][kMergeRows], sh_sq[4][kMergeRows], sh_mx[4][kMergeRows];
   __shared__ double sh_red[7][kMergeRows];
   const int r = threadIdx.x & 63, g = threadIdx.x >> 6;
-  const int64_t tok = (int64_t)blockIdx.x * kMergeRows + r;  // < Np; rows >= N only keep the block sums aligned
-  const bool exists = tok < a.N;
+  const int64_t tok = (int64_t)blockIdx.x * kMergeRows + r;  // < Np; rows that do not exist only keep the block sums aligned
+  const int64_t rows = a.n_rows ? packed_rows(a.n_rows, a.N) : a.N;
+  const bool exists = tok < rows;
+  // packed rows: lse goes back to the token's own place; tokens that were dropped get 0
+  if (a.perm != nullptr && g == 1 && tok < a.N && a.y0[tok] == a.ignore_index) a.lse[tok] = 0.f;
   const int nslices = (int)(a.Vp / kChunkV);
 
   // Online (max, sum) merge of this group's slices, 8 at a time so that the loads of a
@@ -233,7 +244,7 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
       if (sh_s[i][r] != 0.f) St += sh_s[i][r] * fast_exp2((sh_m[i][r] - Mt) * kLog2e);
     const float lse = Mt + fast_log(St);
     sh_lse[r] = lse;
-    if (exists) a.lse[tok] = lse;
+    if (exists) a.lse[a.perm != nullptr ? packed_token(a.perm, tok, a.N) : tok] = lse;
   }
   __syncthreads();
   const float lse = sh_lse[r];

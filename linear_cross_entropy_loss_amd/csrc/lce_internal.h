@@ -39,6 +39,14 @@ struct FwdArgs {
   int64_t ignore_index;
   float scale, z_reg;
   int monitoring;
+  // Packed rows (tokens with an ignored label dropped; null / unused when the call works on all rows):
+  // *n_rows (device) rows are worked on; when *n_rows != N they are the rows of xc (row stride ldxc) and
+  // `y` holds their labels; perm[j] is the token that packed row j came from, y0 the labels of all tokens.
+  const int64_t* n_rows;
+  const void* xc;
+  int64_t ldxc;
+  const int* perm;
+  const int64_t* y0;
   int num_cus;  // compute units of the device: grid size of the persistent kernels
   // outputs / scratch
   float* lse;        // [N]
@@ -83,6 +91,14 @@ struct BwdArgs {
   float* dw_part;
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
+  // Packed rows (tokens with an ignored label dropped).  *n_rows (device) rows are worked on.  When
+  // *n_rows != N they are the rows of xc (row stride ldxc), dx goes to dxc (row stride lddxc, moved to
+  // its place afterwards), and in either case `y` and `lse` hold the labels / lse of the packed rows.
+  const int64_t* n_rows;
+  const void* xc;
+  int64_t ldxc;
+  void* dxc;
+  int64_t lddxc;
 };
 
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s);
@@ -94,6 +110,34 @@ hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
 // compute_dtype: DT_BF16 or DT_F16.
 hipError_t launch_convert_w_slab(const float* src, int64_t ld, int64_t H, int64_t v0, int64_t vw, void* dst,
                                  int64_t dst_ld, int compute_dtype, hipStream_t s);
+
+// Row count / row -> token map of the packed rows as the kernels read them from device memory, forced
+// into range: a call restricted to some phases on a workspace whose packing pre-pass did not run must
+// give wrong numbers, not wild addresses.
+__device__ __forceinline__ int64_t packed_rows(const int64_t* n_rows, int64_t N) {
+  const int64_t r = n_rows[0];
+  return r < 0 ? 0 : (r > N ? N : r);
+}
+__device__ __forceinline__ int64_t packed_token(const int* perm, int64_t j, int64_t N) {
+  const int64_t t = perm[j];
+  return t < 0 ? 0 : (t >= N ? N - 1 : t);
+}
+
+// Packing of the tokens whose label is not ignore_index (lce_compact.hip).  `cnt` holds one int per
+// compact_segments(N); perm and yc hold N entries each, of which the first *n_rows are written.
+int64_t compact_segments(int64_t N);
+hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_index, int* cnt, int64_t* n_rows,
+                                 int* perm, int64_t* yc, hipStream_t s);
+// xc[j] = x[perm[j]] for j < *n_rows, in 16-byte pieces of rows ldxc_bytes long (skipped when *n_rows == N);
+// lse_c[j] = lse[perm[j]] when lse is not null (always).
+hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, const int* perm, const int64_t* n_rows, int64_t N,
+                              void* xc, int64_t ldxc_bytes, const float* lse, float* lse_c, int num_cus,
+                              hipStream_t s);
+// dx[perm[j]] = dxc[j] for j < *n_rows and dx[i] = 0 for every token i with y[i] == ignore_index, in 8-byte
+// pieces covering row_bytes; nothing when *n_rows == N.
+hipError_t launch_scatter_rows(const void* dxc, int64_t lddxc_bytes, const int* perm, const int64_t* n_rows,
+                               int64_t N, const int64_t* y, int64_t ignore_index, void* dx, int64_t lddx_bytes,
+                               int64_t row_bytes, int num_cus, hipStream_t s);
 
 // Split of a contraction with few output tiles along K (host side, shared by planning and launch):
 // with `tiles` output tiles on a device assumed to run 256 workgroups, up to 256/tiles segments of

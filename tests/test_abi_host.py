@@ -109,6 +109,17 @@ def test_backward_scratch_within_n_chunk_bound(N, H, V, n_chunk):
     assert fwd >= (V // 128) * N * 4
 
 
+def _pack_bytes(N, H, es_x=2, es_dx=2, backward=True):
+    """Scratch of the packed rows (tokens with an ignored label dropped): segment counts, the row count, the
+    row -> token map, packed labels and the packed copy of x; for the backward also the packed lse and dx."""
+    al = lambda v: -(-v // 256) * 256
+    pad = lambda v, m: -(-v // m) * m
+    b = al(-(-N // 2048) * 4) + 256 + al(4 * N) + al(8 * N) + al(N * pad(H, 16 // es_x) * es_x)
+    if backward:
+        b += al(4 * N) + al(N * pad(H, 8) * es_dx)
+    return b
+
+
 def test_budget_is_a_target_not_a_refusal():
     """Small vocabulary with many tokens: the strict bound N_chunk*V*4 cannot be met (the fp32 running dx alone
     exceeds it).  The bound is then widened by N*H*4, the fp32 x_grad buffer the reference allocates beside
@@ -122,12 +133,12 @@ def test_budget_is_a_target_not_a_refusal():
         _, bwd = _lib.workspace_bytes(p)
         # dz for all tokens (+ the split-K partials of dW when V*H gives few dW tiles; dx has 512 tiles: no split)
         # dz for all tokens within the widened bound; on top: at most 64 MiB of dW partials
-        assert nc * V * 4 < N * V * 2 <= nc * V * 4 + N * H * 4 and 0 <= bwd - N * V * 2 <= 64 << 20
+        assert nc * V * 4 < N * V * 2 <= nc * V * 4 + N * H * 4 and 0 <= bwd - N * V * 2 - _pack_bytes(N, H) <= 64 << 20
     p = _prob(N=65536, H=256, V=4096, ldx=256, ldw=4096, lddx=256, lddw=4096, n_chunk=64)   # nothing fits
     assert _lib.backward_plan(p) == (16, 256)
     _, bwd = _lib.workspace_bytes(p)
     # dz + fp32 running dx (256 dx tiles: no K split) + the split-K partials of the single dW tile
-    assert 0 < bwd - (65536 * 256 * 2 + 65536 * 256 * 4) <= 64 << 20
+    assert 0 < bwd - (65536 * 256 * 2 + 65536 * 256 * 4) - _pack_bytes(65536, 256) <= 64 << 20
 
 
 def test_backward_plan_is_consistent_with_workspace():
@@ -166,7 +177,7 @@ def test_backward_plan_is_consistent_with_workspace():
         part = dx_part_bytes(Np, Hp, width)
         partw = dw_part_bytes(Np, Hp, width, pad(V, 256) - (slabs - 1) * width)
         assert part <= 64 << 20 and partw <= 64 << 20
-        assert bwd == Np * width * 2 + (Np * Hp * 4 if slabs > 1 else 0) + part + partw
+        assert bwd == _pack_bytes(N, H) + Np * width * 2 + (Np * Hp * 4 if slabs > 1 else 0) + part + partw
         assert Np * width * 2 <= max(1 << 30, Np * 256 * 2)   # dz stage capped at 1 GiB
 
 
