@@ -34,6 +34,49 @@ def test_masking_is_bit_exact_under_garbage_in_ignored_rows():
     assert (dx_a[y == -1].view(torch.int16) == 0).all()  # +0.0 bit pattern
 
 
+def test_ignored_rows_are_never_read_so_nan_in_them_is_harmless():
+    """Tokens with an ignored label are dropped before the tile kernels, so even NaN / Inf in their rows of
+    x leaves loss, dx and dW bit-identical (the reference's x^T dz would give NaN * 0 = NaN, ops.py:424).
+    With monitoring on, logit_max and logit_norm are taken over all rows (ops.py:15, 17) and do see them."""
+    print("NaN in ignored rows", flush=True)
+    x, y, w = make_inputs(1500, 264, 5000, torch.bfloat16, seed=31, ignore_frac=0.4, device="cuda")
+    out_a, dx_a, dw_a = _fb(x, y, w, z_reg=1e-3, n_chunk=64)
+    xg = x.clone()
+    xg[y == -1] = float("nan")
+    xg[(y == -1).nonzero()[::2, 0]] = float("inf")
+    out_b, dx_b, dw_b = _fb(xg, y, w, z_reg=1e-3, n_chunk=64)
+    assert torch.isfinite(out_b[0]) and torch.equal(out_a[0], out_b[0]) and torch.equal(out_a[1], out_b[1])
+    assert torch.equal(dx_a, dx_b) and torch.equal(dw_a, dw_b)
+    assert (dx_b[y == -1].view(torch.int16) == 0).all()
+    out_m, dx_m, dw_m = _fb(xg, y, w, z_reg=1e-3, n_chunk=64, mon=True)
+    assert torch.equal(out_m[0], out_a[0]) and torch.equal(dx_m, dx_a) and torch.equal(dw_m, dw_a)
+    assert not torch.isfinite(out_m[4])  # the norm over all rows meets the NaN rows
+
+
+@pytest.mark.parametrize("keep_every", [1, 2, 7, 300, 5000])
+def test_results_do_not_depend_on_where_the_ignored_tokens_sit(keep_every):
+    """Dropping ignored tokens packs the others to the front in their order: the kept tokens of a sparse
+    batch must give the loss, dW and dx rows of the dense batch made of those tokens alone."""
+    from oracle import lce_forward_backward_fp64
+
+    print(f"packed rows keep_every={keep_every}", flush=True)
+    N, H, V = 3000, 136, 3003
+    x, y, w = make_inputs(N, H, V, torch.float16, seed=40 + keep_every, ignore_frac=0.0, device="cuda")
+    keep = torch.zeros(N, dtype=torch.bool, device="cuda")
+    keep[::keep_every] = True
+    y = torch.where(keep, y, torch.full_like(y, -1))
+    # (a scratch bound wide enough for one vocabulary slab either way: the split depends on N, and with it
+    # the order in which dx is summed)
+    out, dx, dw = _fb(x, y, w, z_reg=1e-4, scale=0.5, n_chunk=4096, g=1.7)
+    dense, dxd, dwd = _fb(x[keep], y[keep], w, z_reg=1e-4, scale=0.5, n_chunk=4096, g=1.7)
+    # same rows in the same order through the same kernels: bit-identical
+    assert torch.equal(out[0], dense[0]) and torch.equal(dw, dwd) and torch.equal(dx[keep], dxd)
+    assert (dx[~keep].view(torch.int16) == 0).all()
+    ref = lce_forward_backward_fp64(x.cpu().double(), y.cpu(), w.cpu().double(), -1, 1e-4, 0.5, 1.7)
+    assert abs(out[0].item() - ref.loss.item()) <= 1e-3 * abs(ref.loss.item())
+    assert max(rel_errors(dx, ref.dx)) <= 2e-2 and max(rel_errors(dw, ref.dw)) <= 2e-2
+
+
 def test_valid_count_is_exact_and_nonnegative_ignore_index_is_honoured():
     from linear_cross_entropy_loss_amd import _lib
 
