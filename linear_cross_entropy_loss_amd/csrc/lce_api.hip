@@ -117,10 +117,9 @@ struct BwdPlan {
 };
 
 // Bytes of the split-K partial sums of dx for slabs of `vs` columns (0 when dx is not split).
-size_t dx_part_bytes(size_t Np, size_t Hp, int64_t vs) {
-  int split, kseg;
-  lce::dx_split_plan((int64_t)Np, (int64_t)Hp, vs, &split, &kseg);
-  return split > 1 ? align_up((size_t)split * Np * Hp * 4) : 0;
+size_t dx_part_bytes(size_t Np, size_t Hp, int64_t vs, int64_t last_vs) {
+  const int64_t b0 = lce::dx_tail_blocks((int64_t)Np, (int64_t)Hp, vs), b1 = lce::dx_tail_blocks((int64_t)Np, (int64_t)Hp, last_vs);
+  return (size_t)(b0 > b1 ? b0 : b1) * 256 * 256 * 4;
 }
 
 // The same for dW (0 when dW is not split).  A narrower last slab has fewer output tiles and may be
@@ -169,7 +168,7 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
       const size_t dz = align_up(Np * (size_t)vs * 2);
       const size_t acc = slabs > 1 ? align_up(Np * Hp * 4) : 0;
       const int64_t last_vs = Vp - (slabs - 1) * vs;  // padded width of the last slab
-      const size_t dxp = dx_part_bytes(Np, Hp, vs), dwp = dw_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
+      const size_t dxp = dx_part_bytes(Np, Hp, vs, last_vs), dwp = dw_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
       const size_t part = dxp + dwp;
       const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2) : 0;  // 16-bit copy of the slab of W
       // the widened bound of the second pass is for the staging proper; the split-K partial sums
@@ -386,7 +385,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     a.v0 = i * b.vs;
     a.vw = p->V - a.v0 < b.vs ? p->V - a.v0 : b.vs;   // columns of this slab that exist
     a.vs = lce::pad_to(a.vw, 256);                    // its padded width: dz row stride and K extent of dx
-    lce::dx_split_plan(a.Np, a.Hp, a.vs, &a.dx_split, &a.dx_kseg);
+    a.dx_grid = a.num_cus;
     lce::dw_split_plan(a.Np, a.Hp, a.vs, &a.dw_split, &a.dw_kseg);
     hipError_t e;
     if (p->w_dtype == LCE_F32) {

@@ -90,6 +90,7 @@ LCE_DEV void dw_partial_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], in
 
 // Work item = (output tile, K segment), segment fastest (see the dx kernel).
 template <class T, class XSrc, bool SPLIT> struct DwProblem {
+  static constexpr bool kVarK = false;
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;

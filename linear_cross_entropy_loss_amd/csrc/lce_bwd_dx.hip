@@ -18,9 +18,12 @@ namespace {
 // stride is a multiple of 4, so it stays inside its row).  No branches: a branch
 // around accumulator reads makes the compiler read all of them up front.
 // `out` / `ldo` / `rows`: dx itself, or the packed copy when tokens were dropped (see BwdArgs).
+// `part` != null: this is a K segment of a tail tile; its raw fp32 sum goes to that 256 x 256 block and
+// nothing else happens.  Both uses run through the same statements (a different fp32 destination and
+// row stride), because two separate code paths behind a branch would each read the accumulator.
 template <class T>
-LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo, f32x16_t (&acc)[kNB][kNB], int tp,
-                         int tq) {
+LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo, float* part,
+                         f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   typedef typename elem_of<T>::type E;
   const int64_t h0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
   const int tid = opaque_tid();
@@ -35,6 +38,11 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo,
   const int64_t left = (reinterpret_cast<const char*>(out) + ((rows - 1) * ldo + hcols) * es) - tile_base;
   const unsigned range = left <= 0 ? 0u : (left > 0x7fffffff ? 0x7fffffffu : (unsigned)left);
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(tile_base), 0, (int)range, 0x00020000);
+  const bool tail = part != nullptr;
+  const bool add_acc = !a.first && !tail, to_f32 = !a.last || tail;
+  // fp32 destination addressed as [token][hidden]: the running sum, or the segment's block shifted to this tile's origin
+  float* f32dst = tail ? part - (t0 * kTile + h0) : a.dx_acc;
+  const int64_t f32ld = tail ? kTile : a.Hp;
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
     const int row = wq * kWaveTile + qb * kBlk + (lane & 31);  // row inside the tile
@@ -49,9 +57,9 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo,
         f32x4_t v;
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = acc[pb][qb][rq * 4 + j];
-        if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + tok * a.Hp + h);
-        if (!a.last) {
-          *reinterpret_cast<f32x4_t*>(a.dx_acc + tok * a.Hp + h) = v;
+        if (add_acc) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + tok * a.Hp + h);
+        if (to_f32) {
+          *reinterpret_cast<f32x4_t*>(f32dst + tok * f32ld + h) = v;
         } else {
           const unsigned off = h < a.H ? row_off + (unsigned)(h * es) : 0x80000000u;
           if (a.dx_dtype == DT_F32) {
@@ -71,100 +79,121 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo,
   }
 }
 
-// Split mode: the raw fp32 partial sum of K segment `seg` goes to dx_part[seg][Np][Hp].
-LCE_DEV void dx_partial_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, int seg) {
-  const int64_t h0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
-  const int tid = opaque_tid();
-  const int lane = tid & 63, wave = tid >> 6;
-  const int wp = wave & 1, wq = wave >> 1;
-  float* part = a.dx_part + (int64_t)seg * a.Np * a.Hp;
-#pragma unroll
-  for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-#pragma unroll
-    for (int pb = 0; pb < kNB; ++pb)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int64_t h = h0 + wp * kWaveTile + pb * kBlk + 8 * rq + 4 * (lane >> 5);
-        f32x4_t v;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = acc[pb][qb][rq * 4 + j];
-        *reinterpret_cast<f32x4_t*>(part + tok * a.Hp + h) = v;
-      }
+// How one launch divides its work.  The output tiles (T of them, from the row count on the device) go to G
+// persistent workgroups in rounds of G.  A last round that would keep only r < G workgroups busy is cut along K
+// instead: its r tiles are split into `nseg` segments of `kseg` K tiles each (a power of two, r * nseg <= G, at
+// least 16 K tiles per segment), one work item per (tile, segment), so that the round is 1/nseg as long and
+// nearly all workgroups take part.  The segments' fp32 partial sums go to dx_part, one 256 x 256 block per
+// item, and dx_tail_kernel adds them in segment order -- deterministic, no atomics.  With few tiles in total
+// (small token counts) every tile is such a tail tile.
+struct DxPlan {
+  int tiles, full, tail_tiles, nseg, kseg;  // items [0, full) are whole tiles, then tail_tiles * nseg segment items
+};
+LCE_DEV DxPlan dx_plan(const BwdArgs& a, int tiles) {
+  DxPlan p;
+  const int G = a.dx_grid, kt = (int)(a.vs / kBK);
+  p.tiles = tiles;
+  p.full = tiles / G * G;
+  const int r = tiles - p.full, cap = G < kDxTailBlocks ? G : kDxTailBlocks;
+  int s = 1;
+  if (r > 0)
+    while (r * s * 2 <= cap && kt % (s * 4) == 0 && kt / (s * 2) >= 16) s *= 2;
+  if (s == 1) {
+    p.full = tiles;
+    p.tail_tiles = 0;
+    p.nseg = 1;
+    p.kseg = kt;
+  } else {
+    p.tail_tiles = r;
+    p.nseg = s;
+    p.kseg = kt / s;  // even: kt is a multiple of 2 s
   }
+  return p;
 }
 
-// Work item = (output tile, K segment); segment fastest, so that with a
-// power-of-two split the workgroups of one XCD work on the same segment and
-// share its W rows and dz columns in their L2.
-template <class T, class WSrc, bool SPLIT, bool KMASK> struct DxProblem {
+template <class T, class WSrc, bool KMASK> struct DxProblem {
   static constexpr bool kKMask = KMASK;
+  static constexpr bool kVarK = true;  // whole tiles and segment items have different K extents
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int64_t rows;  // token rows: all, or the packed ones (see BwdArgs)
-  int tiles_p, tiles_q, split, kseg;
-  LCE_DEV DxProblem(const BwdArgs& a_)
-      : a(a_), rows(packed_rows(a_.n_rows, a_.N)), tiles_p((int)(a_.Hp / kTile)), split(SPLIT ? a_.dx_split : 1), kseg(a_.dx_kseg) {
+  int tiles_p, tiles_q;
+  DxPlan plan;
+  LCE_DEV DxProblem(const BwdArgs& a_) : a(a_), rows(packed_rows(a_.n_rows, a_.N)), tiles_p((int)(a_.Hp / kTile)) {
     tiles_q = (int)((rows + kTile - 1) / kTile);
+    plan = dx_plan(a, tiles_p * tiles_q);
   }
-  LCE_DEV int num_tiles() const { return tiles_p * tiles_q * split; }
+  LCE_DEV int num_tiles() const { return plan.full + plan.tail_tiles * plan.nseg; }
+  // seg < 0: a whole tile
   LCE_DEV void decode(int item, int& tp, int& tq, int& seg) const {
-    seg = SPLIT ? item % split : 0;
-    tile_coords(SPLIT ? item / split : item, tiles_p * tiles_q, tiles_p, tiles_q, 8, tp, tq);
+    int tile = item;
+    seg = -1;
+    if (item >= plan.full) {
+      const int j = item - plan.full;
+      tile = plan.full + j / plan.nseg;
+      seg = j % plan.nseg;
+    }
+    tile_coords(tile, plan.tiles, tiles_p, tiles_q, 8, tp, tq);
   }
+  LCE_DEV int item_ktiles(int item) const { return item < plan.full ? (int)(a.vs / kBK) : plan.kseg; }
+  LCE_DEV int64_t k0_of(int seg) const { return seg < 0 ? 0 : (int64_t)seg * plan.kseg * kBK; }
   LCE_DEV void origins(int item, const void*& p, const void*& q) const {
     int tp, tq, seg;
     decode(item, tp, tq, seg);
-    const int64_t k0 = (int64_t)seg * kseg * kBK;
+    const int64_t k0 = k0_of(seg);
     p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + (a.v0 - a.wv0) + k0;
     q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs + k0;
   }
   LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
   LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + (int64_t)tiles_q * kTile * a.vs; }
   LCE_DEV int k_valid(int item) const {
-    const int seg = SPLIT ? item % split : 0;
-    const int64_t left = a.vw - (int64_t)seg * kseg * kBK;
+    int tp, tq, seg;
+    decode(item, tp, tq, seg);
+    const int64_t left = a.vw - k0_of(seg);
     return (int)(left < 0 ? 0 : left);
   }
   LCE_DEV void epilogue(int item, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq, seg;
     decode(item, tp, tq, seg);
-    if (SPLIT) {
-      dx_partial_epilogue(a, acc, tp, tq, seg);
-    } else {
-      const bool packed = rows != a.N;
-      dx_epilogue<T>(a, rows, packed ? a.dxc : a.dx, packed ? a.lddxc : a.lddx, acc, tp, tq);
-    }
+    const bool packed = rows != a.N;
+    float* part = seg >= 0 ? a.dx_part + (int64_t)(item - plan.full) * kTile * kTile : nullptr;
+    dx_epilogue<T>(a, rows, packed ? a.dxc : a.dx, packed ? a.lddxc : a.lddx, part, acc, tp, tq);
   }
 };
 
-template <class T, class WSrc, bool SPLIT, bool KMASK>
+template <class T, class WSrc, bool KMASK>
 __global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DxProblem<T, WSrc, SPLIT, KMASK> prob(a);
-  Pipe3<T, WSrc, true, E, true, DxProblem<T, WSrc, SPLIT, KMASK>> pipe(prob);
-  pipe.run(a.ldw, a.vs, SPLIT ? a.dx_kseg : (int)(a.vs / kBK), lds);
+  DxProblem<T, WSrc, KMASK> prob(a);
+  Pipe3<T, WSrc, true, E, true, DxProblem<T, WSrc, KMASK>> pipe(prob);
+  pipe.run(a.ldw, a.vs, (int)(a.vs / kBK), lds);
 }
 
-// Split mode, second step: dx (+)= sum over segments, in segment order; same
-// running-sum / final-store rules as the tile kernel's own epilogue.
+// Second step for the tail tiles: workgroup b finishes tail tile b -- sums its segments in order, then the
+// same running-sum / final-store rules as the tile kernel's own epilogue.
 template <class T>
-__global__ __launch_bounds__(256) void dx_reduce_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
   typedef typename elem_of<T>::type E;
-  const int64_t quads_per_row = a.Hp / 4;
   const int64_t rows = packed_rows(a.n_rows, a.N);
-  const int64_t total = rows * quads_per_row;
+  const int tiles_p = (int)(a.Hp / kTile), tiles_q = (int)((rows + kTile - 1) / kTile);
+  const DxPlan plan = dx_plan(a, tiles_p * tiles_q);
+  if ((int)blockIdx.x >= plan.tail_tiles) return;
+  int tp, tq;
+  tile_coords(plan.full + (int)blockIdx.x, plan.tiles, tiles_p, tiles_q, 8, tp, tq);
   const bool packed = rows != a.N;
   void* out = packed ? a.dxc : a.dx;
   const int64_t ldo = packed ? a.lddxc : a.lddx;
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t tok = i / quads_per_row, h = (i - tok * quads_per_row) * 4;
-    if (h >= a.H) continue;
+  const float* part = a.dx_part + (int64_t)blockIdx.x * plan.nseg * kTile * kTile;
+  for (int i = threadIdx.x; i < kTile * kTile / 4; i += 256) {
+    const int row = i / (kTile / 4), hl = (i - row * (kTile / 4)) * 4;
+    const int64_t tok = (int64_t)tq * kTile + row, h = (int64_t)tp * kTile + hl;
+    if (tok >= rows || h >= a.H) continue;
+    f32x4_t v = *reinterpret_cast<const f32x4_t*>(part + row * kTile + hl);
+    for (int s = 1; s < plan.nseg; ++s)
+      v += *reinterpret_cast<const f32x4_t*>(part + (int64_t)s * kTile * kTile + row * kTile + hl);
     const int64_t o = tok * a.Hp + h;
-    f32x4_t v = *reinterpret_cast<const f32x4_t*>(a.dx_part + o);
-    for (int s = 1; s < a.dx_split; ++s) v += *reinterpret_cast<const f32x4_t*>(a.dx_part + (int64_t)s * a.Np * a.Hp + o);
     if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + o);
     if (!a.last) {
       *reinterpret_cast<f32x4_t*>(a.dx_acc + o) = v;
@@ -179,27 +208,22 @@ __global__ __launch_bounds__(256) void dx_reduce_kernel(const BwdArgs a) {
   }
 }
 
-template <class T, class WSrc, bool SPLIT, bool KMASK> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dx_persistent_kernel<T, WSrc, SPLIT, KMASK>;
+template <class T, class WSrc, bool KMASK> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dx_persistent_kernel<T, WSrc, KMASK>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
-  const int64_t items = (a.Hp / kTile) * (a.Np / kTile) * (SPLIT ? a.dx_split : 1);
-  const int grid = (int)(items < a.num_cus ? items : a.num_cus);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
+  hipLaunchKernelGGL(kern, dim3(a.dx_grid), dim3(kThreads), kMainloopLds, s, a);
   return hipGetLastError();
 }
 
 template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  // the K mask is only needed when the K tiles of a work item run past the columns that exist
-  if (a.dx_split <= 1) return a.vw == a.vs ? launch_tiles<T, WSrc, false, false>(a, s) : launch_tiles<T, WSrc, false, true>(a, s);
-  const bool exact_k = a.vw == a.vs && (int64_t)a.dx_split * a.dx_kseg * kBK == a.vs;
-  hipError_t e = exact_k ? launch_tiles<T, WSrc, true, false>(a, s) : launch_tiles<T, WSrc, true, true>(a, s);
+  // the K mask is only needed when the K tiles run past the columns that exist (segments divide the K tiles evenly)
+  hipError_t e = a.vw == a.vs ? launch_tiles<T, WSrc, false>(a, s) : launch_tiles<T, WSrc, true>(a, s);
   if (e != hipSuccess) return e;
-  const int64_t quads = a.N * (a.Hp / 4);
-  int64_t blocks = (quads + 255) / 256;
-  if (blocks > 2048) blocks = 2048;
-  hipLaunchKernelGGL(dx_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, a);
+  if (dx_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // no shape of this launch can have a split tail
+  // at most dx_grid / 2 tail tiles can be split (two segments each)
+  hipLaunchKernelGGL(dx_tail_kernel<T>, dim3((unsigned)(a.dx_grid / 2 > 0 ? a.dx_grid / 2 : 1)), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 

@@ -169,6 +169,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
 // of the vocabulary to the end of the padded slab.
 template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK> struct DzProblem {
   static constexpr bool kKMask = KMASK;
+  static constexpr bool kVarK = false;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows: all of x, or the packed rows (see BwdArgs)
   const XSrc* x;

@@ -157,6 +157,7 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
 // labels were packed away -- the first `rows` rows of the packed copy (the count lives on the device).
 template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdProblem {
   static constexpr bool kKMask = KMASK;
+  static constexpr bool kVarK = false;
   const FwdArgs& a;
   int64_t rows, ldx;
   const XSrc* x;

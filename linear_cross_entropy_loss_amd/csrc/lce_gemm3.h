@@ -150,6 +150,8 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //        first element of the P / Q operand of that output tile:
 //        (row0, k=0) for a KC operand, (k=0, col0) for an MC operand
 //   const void* p_end(), q_end()                  one past the last valid byte of each operand
+//   static constexpr bool kVarK                   true if work items differ in their number of K tiles; then
+//   int  item_ktiles(int tile)                    gives it (even, at least 4) -- otherwise run() is told once
 //   static constexpr bool kKMask                  false if `ktiles * 64 == k_valid` for every tile of the launch
 //   int  k_valid(int tile)                        K extent of that tile's contraction; the K tiles of the
 //        loop may run past it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
@@ -354,6 +356,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
 
     f32x16_t acc[kNB][kNB];
     for (int tile = (int)blockIdx.x; tile < prob.num_tiles(); tile += (int)gridDim.x) {
+      if constexpr (Problem::kVarK) ktiles = prob.item_ktiles(tile);
       read_frags(0, lds, 0);
       step<0, true, false, false>(acc, sp, sq);
       if (ktiles > 4) {

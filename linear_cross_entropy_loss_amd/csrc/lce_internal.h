@@ -80,10 +80,10 @@ struct BwdArgs {
   int64_t wv0, Vw;  // `w` holds columns [wv0, wv0 + Vw) of the weight (the whole matrix, or a 16-bit copy of this slab)
   void* dz;         // [Np][vs] staged dz in the compute type (exact zeros outside N x vw)
   float* dx_acc;    // [Np][Hp] fp32 running dx (null when there is a single slab)
-  // dx with few output tiles: the K extent of a slab is cut into `dx_split` segments of `dx_kseg`
-  // K tiles, one work item each; the partial sums meet in dx_part [dx_split][Np][Hp] (fp32) and a
-  // small kernel adds them in a fixed order.  dx_split == 1: no partials, the tile kernel finishes dx.
-  int dx_split, dx_kseg;
+  // dx: tiles of a last, mostly idle round of workgroups are cut along K instead (planned on the device,
+  // see lce_bwd_dx.hip); the segments' partial sums meet in dx_part, dx_tail_blocks() blocks of 256 x 256
+  // floats, and a small kernel adds them in a fixed order.  dx_grid = workgroups of the tile kernel.
+  int dx_grid;
   float* dx_part;
   // The same for dW with few output tiles (small vocabulary slab x hidden size): K = tokens is cut into
   // dw_split segments of dw_kseg K tiles; partial sums in dw_part [dw_split][Hp][vs] (fp32).
@@ -151,9 +151,16 @@ inline void k_split_plan(int64_t tiles, int64_t ktiles, int* split, int* kseg) {
   *kseg = (int)seg;
   *split = (int)((ktiles + seg - 1) / seg);
 }
-// dx of one slab: (Np/256) x (Hp/256) tiles, K = vs columns
-inline void dx_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* kseg) {
-  k_split_plan((Np / 256) * (Hp / 256), vs / 64, split, kseg);
+// dx of one slab: at most (Np/256) x (Hp/256) tiles, K = vs columns.  Upper bound on the 256 x 256 fp32
+// blocks of partial sums that the device-side plan of the dx kernel can ask for (0: it never splits).
+constexpr int kDxTailBlocks = 256;
+inline int64_t dx_tail_blocks(int64_t Np, int64_t Hp, int64_t vs) {
+  const int64_t kt = vs / 64;
+  int64_t s = 1;  // most segments per tile: a power of two with at least 16 K tiles each, an even number
+  while (kt % (s * 4) == 0 && kt / (s * 2) >= 16) s *= 2;
+  if (s == 1) return 0;
+  const int64_t most = (Np / 256) * (Hp / 256) * s;
+  return most < kDxTailBlocks ? most : kDxTailBlocks;
 }
 // dW of one slab: (vs/256) x (Hp/256) tiles, K = Np tokens
 inline void dw_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* kseg) {
