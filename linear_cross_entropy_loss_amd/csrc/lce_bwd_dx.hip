@@ -170,29 +170,38 @@ __global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdAr
   pipe.run(a.ldw, a.vs, (int)(a.vs / kBK), lds);
 }
 
-// Second step for the tail tiles: workgroup b finishes tail tile b -- sums its segments in order, then the
-// same running-sum / final-store rules as the tile kernel's own epilogue.
+// Second step for the tail tiles: kTailParts workgroups share tail tile b (16 rows each) -- they sum its
+// segments in order, then apply the same running-sum / final-store rules as the tile kernel's own epilogue.
+constexpr int kTailParts = 16;
 template <class T>
 __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
   typedef typename elem_of<T>::type E;
   const int64_t rows = packed_rows(a.n_rows, a.N);
   const int tiles_p = (int)(a.Hp / kTile), tiles_q = (int)((rows + kTile - 1) / kTile);
   const DxPlan plan = dx_plan(a, tiles_p * tiles_q);
-  if ((int)blockIdx.x >= plan.tail_tiles) return;
+  const int b = (int)blockIdx.x / kTailParts, piece = (int)blockIdx.x % kTailParts;
+  if (b >= plan.tail_tiles) return;
   int tp, tq;
-  tile_coords(plan.full + (int)blockIdx.x, plan.tiles, tiles_p, tiles_q, 8, tp, tq);
+  tile_coords(plan.full + b, plan.tiles, tiles_p, tiles_q, 8, tp, tq);
   const bool packed = rows != a.N;
   void* out = packed ? a.dxc : a.dx;
   const int64_t ldo = packed ? a.lddxc : a.lddx;
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
-  const float* part = a.dx_part + (int64_t)blockIdx.x * plan.nseg * kTile * kTile;
-  for (int i = threadIdx.x; i < kTile * kTile / 4; i += 256) {
+  const float* part = a.dx_part + (int64_t)b * plan.nseg * kTile * kTile;
+  constexpr int kQuads = kTile * kTile / 4 / kTailParts;  // quads of this workgroup: 16 rows of the tile
+  for (int i = piece * kQuads + threadIdx.x; i < (piece + 1) * kQuads; i += 256) {
     const int row = i / (kTile / 4), hl = (i - row * (kTile / 4)) * 4;
     const int64_t tok = (int64_t)tq * kTile + row, h = (int64_t)tp * kTile + hl;
     if (tok >= rows || h >= a.H) continue;
+    // nseg is a power of two >= 2: two segments per step keep two loads in flight, the sum stays in segment order
     f32x4_t v = *reinterpret_cast<const f32x4_t*>(part + row * kTile + hl);
-    for (int s = 1; s < plan.nseg; ++s)
-      v += *reinterpret_cast<const f32x4_t*>(part + (int64_t)s * kTile * kTile + row * kTile + hl);
+    v += *reinterpret_cast<const f32x4_t*>(part + (int64_t)kTile * kTile + row * kTile + hl);
+    for (int s = 2; s < plan.nseg; s += 2) {
+      const f32x4_t u0 = *reinterpret_cast<const f32x4_t*>(part + (int64_t)s * kTile * kTile + row * kTile + hl);
+      const f32x4_t u1 = *reinterpret_cast<const f32x4_t*>(part + (int64_t)(s + 1) * kTile * kTile + row * kTile + hl);
+      v += u0;
+      v += u1;
+    }
     const int64_t o = tok * a.Hp + h;
     if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + o);
     if (!a.last) {
@@ -223,7 +232,8 @@ template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hi
   if (e != hipSuccess) return e;
   if (dx_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // no shape of this launch can have a split tail
   // at most dx_grid / 2 tail tiles can be split (two segments each)
-  hipLaunchKernelGGL(dx_tail_kernel<T>, dim3((unsigned)(a.dx_grid / 2 > 0 ? a.dx_grid / 2 : 1)), dim3(256), 0, s, a);
+  const unsigned tail_most = (unsigned)(a.dx_grid / 2 > 0 ? a.dx_grid / 2 : 1);
+  hipLaunchKernelGGL(dx_tail_kernel<T>, dim3(tail_most * kTailParts), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 
