@@ -55,11 +55,13 @@ int check(const lce_problem* p, bool backward) {
 struct PackPlan {
   size_t cnt, n_rows, perm, yc, xc, end;
   int64_t ldxc;  // row stride of the packed copy of x, elements: rows of whole 16-byte pieces
+  size_t xes;    // element size of the packed copy: that of x, or 2 for fp32 activations (stored rounded to bf16)
 };
 
 PackPlan plan_pack(const lce_problem* p, size_t base) {
   PackPlan k;
-  const size_t N = (size_t)p->N, es = p->x_dtype == LCE_F32 ? 4 : 2;
+  const size_t N = (size_t)p->N, es = 2;
+  k.xes = es;
   k.ldxc = lce::pad_to(p->H, (int64_t)(16 / es));
   size_t o = base;
   k.cnt = o; o += align_up((size_t)lce::compact_segments(p->N) * 4);
@@ -73,7 +75,9 @@ PackPlan plan_pack(const lce_problem* p, size_t base) {
 
 struct FwdPlan {
   size_t part_lse, part_max, part_pz, part_sq, tgt, blk, w16, total;
-  PackPlan pack;  // only when monitoring is off (the monitoring values are taken over all rows)
+  // When monitoring is off (the monitoring values are taken over all rows), and for fp32 activations, which
+  // reach the tile kernels through the packed copy (rounded to bf16 there).
+  PackPlan pack;
   int64_t vs;  // columns per forward launch: all of V, or the width of the 16-bit slab copy of an fp32 weight
 };
 
@@ -100,7 +104,7 @@ FwdPlan plan_fwd(const lce_problem* p) {
     if (cols < f.vs) f.vs = cols;
     o += align_up((size_t)p->H * (size_t)f.vs * 2);
   }
-  if (!p->monitoring) {
+  if (!p->monitoring || p->x_dtype == LCE_F32) {
     f.pack = plan_pack(p, o);
     o = f.pack.end;
   }
@@ -285,23 +289,34 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
 
   const int ph = p->phases ? p->phases : ~0;
   hipError_t e;
-  if (!p->monitoring) {
-    // Tokens with an ignored label add nothing to the loss: the tile kernel runs on the others only.
+  const bool pack = !p->monitoring, x32 = p->x_dtype == LCE_F32;
+  if (pack || x32) {
     const PackPlan& k = f.pack;
-    a.n_rows = (const int64_t*)(base + k.n_rows);
-    a.perm = (const int*)(base + k.perm);
+    if (pack) {
+      // Tokens with an ignored label add nothing to the loss: the tile kernel runs on the others only.
+      a.n_rows = (const int64_t*)(base + k.n_rows);
+      a.perm = (const int*)(base + k.perm);
+      a.y0 = y;
+      a.y = (const int64_t*)(base + k.yc);
+    }
     a.xc = base + k.xc;
     a.ldxc = k.ldxc;
-    a.y0 = y;
-    a.y = (const int64_t*)(base + k.yc);
     if (ph & LCE_PHASE_PACK) {
-      e = lce::launch_compact_labels(y, p->N, p->ignore_index, (int*)(base + k.cnt), (int64_t*)(base + k.n_rows),
-                                     (int*)(base + k.perm), (int64_t*)(base + k.yc), s);
-      if (e != hipSuccess) return hip_fail(e, "compact_labels");
-      const int64_t es = p->x_dtype == LCE_F32 ? 4 : 2;
-      e = lce::launch_gather_rows(x, p->ldx * es, a.perm, a.n_rows, p->N, base + k.xc, k.ldxc * es, nullptr,
-                                  nullptr, a.num_cus, s);
+      if (pack) {
+        e = lce::launch_compact_labels(y, p->N, p->ignore_index, (int*)(base + k.cnt), (int64_t*)(base + k.n_rows),
+                                       (int*)(base + k.perm), (int64_t*)(base + k.yc), s);
+        if (e != hipSuccess) return hip_fail(e, "compact_labels");
+      }
+      e = x32 ? lce::launch_gather_rows_f32((const float*)x, p->ldx, p->H, a.perm, a.n_rows, p->N, base + k.xc, k.ldxc,
+                                            nullptr, nullptr, a.num_cus, s)
+              : lce::launch_gather_rows(x, p->ldx * 2, a.perm, a.n_rows, p->N, base + k.xc, k.ldxc * 2, nullptr, nullptr,
+                                        a.num_cus, s);
       if (e != hipSuccess) return hip_fail(e, "gather_rows");
+    }
+    if (x32) {  // the tile kernels read the bf16 copy, whether or not rows were dropped
+      a.x = a.xc;
+      a.ldx = a.ldxc;
+      a.x_dtype = lce::DT_BF16;
     }
   }
   if (ph & LCE_PHASE_FWD_TILES) {
@@ -364,7 +379,8 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
 
   // Tokens with an ignored label have dz == 0: the kernels run on the other rows only, packed to the front.
   const PackPlan& k = b.pack;
-  const int64_t xes = p->x_dtype == LCE_F32 ? 4 : 2, dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
+  const bool x32 = p->x_dtype == LCE_F32;
+  const int64_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
   a.n_rows = (const int64_t*)(base + k.n_rows);
   a.xc = base + k.xc;
   a.ldxc = k.ldxc;
@@ -376,9 +392,16 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     hipError_t e = lce::launch_compact_labels(y, p->N, p->ignore_index, (int*)(base + k.cnt), (int64_t*)(base + k.n_rows),
                                               (int*)(base + k.perm), (int64_t*)(base + k.yc), s);
     if (e != hipSuccess) return hip_fail(e, "compact_labels");
-    e = lce::launch_gather_rows(x, p->ldx * xes, (const int*)(base + k.perm), a.n_rows, p->N, base + k.xc, k.ldxc * xes,
-                                lse, (float*)(base + b.lse_c), a.num_cus, s);
+    e = x32 ? lce::launch_gather_rows_f32((const float*)x, p->ldx, p->H, (const int*)(base + k.perm), a.n_rows, p->N,
+                                          base + k.xc, k.ldxc, lse, (float*)(base + b.lse_c), a.num_cus, s)
+            : lce::launch_gather_rows(x, p->ldx * 2, (const int*)(base + k.perm), a.n_rows, p->N, base + k.xc, k.ldxc * 2,
+                                      lse, (float*)(base + b.lse_c), a.num_cus, s);
     if (e != hipSuccess) return hip_fail(e, "gather_rows");
+  }
+  if (x32) {  // fp32 activations reach the tile kernels as the bf16 packed copy, whether or not rows were dropped
+    a.x = a.xc;
+    a.ldx = a.ldxc;
+    a.x_dtype = lce::DT_BF16;
   }
 
   for (int64_t i = 0; i < b.slabs; ++i) {

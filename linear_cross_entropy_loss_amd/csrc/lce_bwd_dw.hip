@@ -203,7 +203,6 @@ hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<F16>::type hf;
   if (a.x_dtype == DT_BF16) return launch_persistent<BF16, bf>(a, s);
   if (a.x_dtype == DT_F16) return launch_persistent<F16, hf>(a, s);
-  if (a.x_dtype == DT_F32) return launch_persistent<BF16, float>(a, s);
   return hipErrorInvalidValue;
 }
 

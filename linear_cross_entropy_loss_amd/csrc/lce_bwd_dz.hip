@@ -248,8 +248,7 @@ hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
   typedef elem_of<F16>::type hf;
   if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf, bf>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf, hf>(a, s);
-  // an fp32 weight arrives here as a 16-bit slab copy; fp32 activations are converted on the way into LDS
-  if (a.x_dtype == DT_F32 && a.w_dtype == DT_BF16) return launch_persistent<BF16, float, bf>(a, s);
+  // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as the bf16 packed copy)
   return hipErrorInvalidValue;
 }
 

@@ -111,6 +111,35 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const char* x, int64_t
   }
 }
 
+// fp32 activations: the packed copy is made in the 16-bit compute type (round to nearest even), so the tile
+// kernels only ever read 16-bit operands.  The copy is made even when no token is dropped, and `perm` /
+// `n_rows` may be null (all rows, in place order).  One thread converts 8 consecutive elements.
+template <class T>
+__global__ __launch_bounds__(256) void gather_rows_f32_kernel(const float* x, int64_t ldx, int64_t H, const int* perm,
+                                                              const int64_t* n_rows, int64_t N, unsigned short* xc,
+                                                              int64_t ldxc, const float* lse, float* lse_c) {
+  const int64_t rows = n_rows != nullptr ? packed_rows(n_rows, N) : N;
+  const int chunks = (int)(ldxc / 8);
+  for (int64_t j = blockIdx.x; j < rows; j += gridDim.x) {
+    const int64_t src = perm != nullptr ? packed_token(perm, j, N) : j;
+    if (lse != nullptr && threadIdx.x == 0) lse_c[j] = lse[src];
+    const float* s = x + src * ldx;
+    for (int c = threadIdx.x; c < chunks; c += 256) {
+      // the row stride is a multiple of 4: a quad that starts inside the row may be read whole
+      f32x4_t lo, hi;
+      for (int e = 0; e < 4; ++e) lo[e] = hi[e] = 0.f;
+      if (8 * c < H) lo = *reinterpret_cast<const f32x4_t*>(s + 8 * c);
+      if (8 * c + 4 < H) hi = *reinterpret_cast<const f32x4_t*>(s + 8 * c + 4);
+      u32x4_t o;
+      o[0] = pack2<T>(lo[0], lo[1]);
+      o[1] = pack2<T>(lo[2], lo[3]);
+      o[2] = pack2<T>(hi[0], hi[1]);
+      o[3] = pack2<T>(hi[2], hi[3]);
+      *reinterpret_cast<u32x4_t*>(xc + j * ldxc + 8 * c) = o;
+    }
+  }
+}
+
 // One workgroup per token (grid-stride): token i moves packed row i to its place (if there is a packed
 // row i) and clears its own row of dx if it was dropped.  8-byte pieces, `chunks` per row.
 __global__ __launch_bounds__(256) void scatter_rows_kernel(const char* dxc, int64_t lddxc_bytes, const int* perm,
@@ -151,6 +180,14 @@ hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_ind
   hipLaunchKernelGGL(count_kept_kernel, dim3((unsigned)nseg), dim3(256), 0, s, y, N, ignore_index, cnt);
   hipLaunchKernelGGL(scan_counts_kernel, dim3(1), dim3(256), 0, s, cnt, nseg, n_rows);
   hipLaunchKernelGGL(pack_kept_kernel, dim3((unsigned)nseg), dim3(256), 0, s, y, N, ignore_index, cnt, perm, yc);
+  return hipGetLastError();
+}
+
+hipError_t launch_gather_rows_f32(const float* x, int64_t ldx, int64_t H, const int* perm, const int64_t* n_rows,
+                                  int64_t N, void* xc, int64_t ldxc, const float* lse, float* lse_c, int num_cus,
+                                  hipStream_t s) {
+  hipLaunchKernelGGL(gather_rows_f32_kernel<BF16>, dim3(row_grid(N, num_cus)), dim3(256), 0, s, x, ldx, H, perm, n_rows,
+                     N, reinterpret_cast<unsigned short*>(xc), ldxc, lse, lse_c);
   return hipGetLastError();
 }
 

@@ -82,10 +82,6 @@ LCE_DEV int opaque_tid() {
   return t;
 }
 
-// Bit pattern -> float.  Takes the word by value on purpose: bit-casting a
-// vector element expression directly reads element 0 for every index.
-LCE_DEV float as_f32(unsigned int u) { return __builtin_bit_cast(float, u); }
-
 // ---------------------------------------------------------------------------
 // Workgroup -> tile mapping.  Workgroups are dealt round-robin to the 8 XCDs,
 // each with its own L2, so consecutive ids are first regrouped per XCD and

@@ -1,5 +1,5 @@
-// Persistent, software-pipelined contraction.  Operands are 16-bit in LDS; in memory
-// they are either already 16-bit or fp32 (converted on the way into LDS).
+// Persistent, software-pipelined contraction of 16-bit operands (fp32 inputs are
+// rounded to the compute type by copy kernels before a tile kernel sees them).
 //
 // One workgroup per CU walks a list of 256 x 256 output tiles.  The operand
 // fetch is one continuous stream of K tiles that runs THROUGH output-tile
@@ -29,10 +29,11 @@
 
 namespace lce {
 
-// Register staging of one operand tile: 8 chunks of 8 elements per thread; a chunk
-// is one 16-byte register quad for 16-bit sources and two for fp32 sources.
-template <bool WIDE> struct StageRegs {
-  u32x4_t v[WIDE ? 16 : 8];
+// Register staging of one operand tile: 8 chunks of 8 elements (one 16-byte register quad) per thread.
+// Operands are always 16-bit in memory: fp32 activations and weights are rounded to the compute type by
+// copy kernels before the tile kernels run.
+struct StageRegs {
+  u32x4_t v[8];
 };
 
 #define LCE_SG_MFMA 0x008
@@ -46,9 +47,9 @@ template <bool WIDE> struct StageRegs {
 // load costs one instruction and no vector address arithmetic.
 // KMASK = false compiles the K mask out, for launches whose K tiles cover the K extent exactly.
 template <class T, class SrcT, bool KC, bool KMASK> struct Stager3 {
-  static constexpr bool kWide = sizeof(SrcT) == 4;
+  static_assert(sizeof(SrcT) == 2, "operands are staged as 16-bit data");
   static constexpr int kEs = (int)sizeof(SrcT);
-  typedef StageRegs<kWide> Regs;
+  typedef StageRegs Regs;
   const char* base;      // uniform: first byte of the K tile being loaded
   const char* end;       // uniform: one past the last valid byte of the operand (loads beyond return 0)
   unsigned range;        // uniform: bytes from `base` to `end`, clamped to [0, 2^31)
@@ -106,31 +107,13 @@ template <class T, class SrcT, bool KC, bool KMASK> struct Stager3 {
     const __amdgpu_buffer_rsrc_t rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, (int)range, 0x00020000);
 #pragma unroll
-    for (int i = i0; i < i1; ++i) {
-      if (kWide) {
-        r.v[2 * i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff_cur, (int)(i * iter_stride), 0);
-        r.v[2 * i + 1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff_cur + 16, (int)(i * iter_stride), 0);
-      } else {
-        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff_cur, (int)(i * iter_stride), 0);
-      }
-    }
+    for (int i = i0; i < i1; ++i)
+      r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff_cur, (int)(i * iter_stride), 0);
   }
   LCE_DEV void store(const Regs& r, char* tile, int i0, int i1) const {
     constexpr int step = KC ? 32 * 128 : 8 * 512;
 #pragma unroll
-    for (int i = i0; i < i1; ++i) {
-      u32x4_t v;
-      if (kWide) {
-        const u32x4_t a = r.v[2 * i], b = r.v[2 * i + 1];
-        v[0] = pack2<T>(as_f32(a[0]), as_f32(a[1]));
-        v[1] = pack2<T>(as_f32(a[2]), as_f32(a[3]));
-        v[2] = pack2<T>(as_f32(b[0]), as_f32(b[1]));
-        v[3] = pack2<T>(as_f32(b[2]), as_f32(b[3]));
-      } else {
-        v = r.v[i];
-      }
-      *reinterpret_cast<u32x4_t*>(tile + lds_off + i * step) = v;
-    }
+    for (int i = i0; i < i1; ++i) *reinterpret_cast<u32x4_t*>(tile + lds_off + i * step) = r.v[i];
   }
 };
 
@@ -165,8 +148,6 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
   typedef Stager3<T, QSrc, Q_KC, Problem::kKMask> QStager;
   typedef typename PStager::Regs PRegs;
   typedef typename QStager::Regs QRegs;
-  static constexpr int kPW = PStager::kWide ? 2 : 1;  // load instructions per chunk
-  static constexpr int kQW = QStager::kWide ? 2 : 1;
   PStager ps;
   QStager qs;
   FragReader<P_KC> pr;
@@ -286,7 +267,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
       if (i >= 5 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
-      if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 0..5: P
+      if (i >= 4 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);  // chunks 0..5: P
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -300,8 +281,8 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
       if (i >= 4 && i < 12 && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_WR, 1, 0);
-      if (i >= 5 && i < 9 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kPW, 0);  // chunks 6, 7: P
-      if (i >= 9 && i < 15 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);  // chunks 8..10: Q
+      if (i >= 5 && i < 9 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);  // chunks 6, 7: P
+      if (i >= 9 && i < 15 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);  // chunks 8..10: Q
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -312,7 +293,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
 #pragma unroll
     for (int i = 0; i < kPre; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
-      if (i < kPreLoads) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);  // chunks 11..: Q
+      if (i < kPreLoads) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);  // chunks 11..: Q
     }
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
@@ -330,7 +311,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
     for (int i = 0; i < 16 - kPre; ++i) {
       __builtin_amdgcn_sched_group_barrier(LCE_SG_MFMA, 1, 0);
       if (!LAST && i < 4) __builtin_amdgcn_sched_group_barrier(LCE_SG_DS_RD, kReadsPerSlot, 0);
-      if (i >= 4 && i < 4 + 5 - kPreLoads) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, kQW, 0);
+      if (i >= 4 && i < 4 + 5 - kPreLoads) __builtin_amdgcn_sched_group_barrier(LCE_SG_VMEM_RD, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   }

@@ -133,6 +133,11 @@ hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_ind
 hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, const int* perm, const int64_t* n_rows, int64_t N,
                               void* xc, int64_t ldxc_bytes, const float* lse, float* lse_c, int num_cus,
                               hipStream_t s);
+// The same for fp32 activations: xc is written in bf16 (the compute type of fp32 inputs), always, also when
+// no token is dropped; perm / n_rows may be null (all N rows in their order).  ldx, ldxc in elements.
+hipError_t launch_gather_rows_f32(const float* x, int64_t ldx, int64_t H, const int* perm, const int64_t* n_rows,
+                                  int64_t N, void* xc, int64_t ldxc, const float* lse, float* lse_c, int num_cus,
+                                  hipStream_t s);
 // dx[perm[j]] = dxc[j] for j < *n_rows and dx[i] = 0 for every token i with y[i] == ignore_index, in 8-byte
 // pieces covering row_bytes; nothing when *n_rows == N.
 hipError_t launch_scatter_rows(const void* dxc, int64_t lddxc_bytes, const int* perm, const int64_t* n_rows,
