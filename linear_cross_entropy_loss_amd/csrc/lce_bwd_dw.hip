@@ -89,20 +89,20 @@ LCE_DEV void dw_partial_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], in
 }
 
 // Work item = (output tile, K segment), segment fastest (see the dx kernel).
-template <class T, class XSrc, bool SPLIT> struct DwProblem {
+template <class T, bool SPLIT> struct DwProblem {
   static constexpr bool kVarK = false;
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows (the K extent): all of x, or the packed rows (see BwdArgs)
-  const XSrc* x;
+  const E* x;
   int tiles_p, tiles_q, split, kseg;
   LCE_DEV DwProblem(const BwdArgs& a_)
       : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.Hp / kTile)), split(SPLIT ? a_.dw_split : 1),
         kseg(a_.dw_kseg) {
     rows = packed_rows(a.n_rows, a.N);
     const bool packed = rows != a.N;
-    x = reinterpret_cast<const XSrc*>(packed ? a.xc : a.x);
+    x = reinterpret_cast<const E*>(packed ? a.xc : a.x);
     ldx = packed ? a.ldxc : a.ldx;
   }
   // K tiles of an unsplit contraction: an even number, at least four, covering the rows
@@ -127,7 +127,7 @@ template <class T, class XSrc, bool SPLIT> struct DwProblem {
   LCE_DEV const void* p_end() const {
     return reinterpret_cast<const E*>(a.dz) + (rows + kTile - 1) / kTile * kTile * a.vs;
   }
-  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(x, rows, ldx, a.H); }
+  LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.Np; }
   LCE_DEV void epilogue(int item, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq, seg;
@@ -140,12 +140,12 @@ template <class T, class XSrc, bool SPLIT> struct DwProblem {
   }
 };
 
-template <class T, class XSrc, bool SPLIT>
+template <class T, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DwProblem<T, XSrc, SPLIT> prob(a);
-  Pipe3<T, E, false, XSrc, false, DwProblem<T, XSrc, SPLIT>> pipe(prob);
+  DwProblem<T, SPLIT> prob(a);
+  Pipe3<T, E, false, E, false, DwProblem<T, SPLIT>> pipe(prob);
   pipe.run(a.vs, prob.ldx, SPLIT ? a.dw_kseg : prob.ktiles(), lds);
 }
 
@@ -174,8 +174,8 @@ __global__ __launch_bounds__(256) void dw_reduce_kernel(const BwdArgs a) {
   }
 }
 
-template <class T, class XSrc, bool SPLIT> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dw_persistent_kernel<T, XSrc, SPLIT>;
+template <class T, bool SPLIT> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dw_persistent_kernel<T, SPLIT>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -185,9 +185,9 @@ template <class T, class XSrc, bool SPLIT> hipError_t launch_tiles(const BwdArgs
   return hipGetLastError();
 }
 
-template <class T, class XSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  if (a.dw_split <= 1) return launch_tiles<T, XSrc, false>(a, s);
-  hipError_t e = launch_tiles<T, XSrc, true>(a, s);
+template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  if (a.dw_split <= 1) return launch_tiles<T, false>(a, s);
+  hipError_t e = launch_tiles<T, true>(a, s);
   if (e != hipSuccess) return e;
   const int64_t quads = a.H * (a.vs / 4);
   int64_t blocks = (quads + 255) / 256;
@@ -199,10 +199,8 @@ template <class T, class XSrc> hipError_t launch_persistent(const BwdArgs& a, hi
 }  // namespace
 
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s) {
-  typedef elem_of<BF16>::type bf;
-  typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16) return launch_persistent<BF16, bf>(a, s);
-  if (a.x_dtype == DT_F16) return launch_persistent<F16, hf>(a, s);
+  if (a.x_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
+  if (a.x_dtype == DT_F16) return launch_persistent<F16>(a, s);
   return hipErrorInvalidValue;
 }
 

@@ -111,7 +111,7 @@ LCE_DEV DxPlan dx_plan(const BwdArgs& a, int tiles) {
   return p;
 }
 
-template <class T, class WSrc, bool KMASK> struct DxProblem {
+template <class T, bool KMASK> struct DxProblem {
   static constexpr bool kKMask = KMASK;
   static constexpr bool kVarK = true;  // whole tiles and segment items have different K extents
   typedef typename elem_of<T>::type E;
@@ -141,10 +141,10 @@ template <class T, class WSrc, bool KMASK> struct DxProblem {
     int tp, tq, seg;
     decode(item, tp, tq, seg);
     const int64_t k0 = k0_of(seg);
-    p = reinterpret_cast<const WSrc*>(a.w) + (int64_t)tp * kTile * a.ldw + (a.v0 - a.wv0) + k0;
+    p = reinterpret_cast<const E*>(a.w) + (int64_t)tp * kTile * a.ldw + (a.v0 - a.wv0) + k0;
     q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs + k0;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
+  LCE_DEV const void* p_end() const { return matrix_end<E>(a.w, a.H, a.ldw, a.Vw); }
   LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + (int64_t)tiles_q * kTile * a.vs; }
   LCE_DEV int k_valid(int item) const {
     int tp, tq, seg;
@@ -161,12 +161,12 @@ template <class T, class WSrc, bool KMASK> struct DxProblem {
   }
 };
 
-template <class T, class WSrc, bool KMASK>
+template <class T, bool KMASK>
 __global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DxProblem<T, WSrc, KMASK> prob(a);
-  Pipe3<T, WSrc, true, E, true, DxProblem<T, WSrc, KMASK>> pipe(prob);
+  DxProblem<T, KMASK> prob(a);
+  Pipe3<T, E, true, E, true, DxProblem<T, KMASK>> pipe(prob);
   pipe.run(a.ldw, a.vs, (int)(a.vs / kBK), lds);
 }
 
@@ -217,8 +217,8 @@ __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
   }
 }
 
-template <class T, class WSrc, bool KMASK> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dx_persistent_kernel<T, WSrc, KMASK>;
+template <class T, bool KMASK> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dx_persistent_kernel<T, KMASK>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -226,9 +226,9 @@ template <class T, class WSrc, bool KMASK> hipError_t launch_tiles(const BwdArgs
   return hipGetLastError();
 }
 
-template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
   // the K mask is only needed when the K tiles run past the columns that exist (segments divide the K tiles evenly)
-  hipError_t e = a.vw == a.vs ? launch_tiles<T, WSrc, false>(a, s) : launch_tiles<T, WSrc, true>(a, s);
+  hipError_t e = a.vw == a.vs ? launch_tiles<T, false>(a, s) : launch_tiles<T, true>(a, s);
   if (e != hipSuccess) return e;
   if (dx_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // no shape of this launch can have a split tail
   // at most dx_grid / 2 tail tiles can be split (two segments each)
@@ -240,12 +240,9 @@ template <class T, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hi
 }  // namespace
 
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s) {
-  typedef elem_of<BF16>::type bf;
-  typedef elem_of<F16>::type hf;
-  const bool bf_compute = a.x_dtype == DT_BF16 || a.x_dtype == DT_F32;
-  // an fp32 weight arrives here as a 16-bit slab copy
-  if (bf_compute && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf>(a, s);
+  // (an fp32 weight arrives here as a 16-bit slab copy; x_dtype is the compute type by now)
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
   return hipErrorInvalidValue;
 }
 

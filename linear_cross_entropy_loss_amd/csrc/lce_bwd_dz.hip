@@ -167,19 +167,20 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
 // The launch covers `tiles_p` tile columns of the slab starting at column tile
 // `tp0`: all the full ones, or (VTAIL) those from the one straddling the end
 // of the vocabulary to the end of the padded slab.
-template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK> struct DzProblem {
+template <class T, bool ZREG, bool VTAIL, bool KMASK> struct DzProblem {
+  typedef typename elem_of<T>::type E;
   static constexpr bool kKMask = KMASK;
   static constexpr bool kVarK = false;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows: all of x, or the packed rows (see BwdArgs)
-  const XSrc* x;
+  const E* x;
   int tp0, tiles_p, tiles_q;
   LCE_DEV DzProblem(const BwdArgs& a_)
       : a(a_), tp0(VTAIL ? (int)(a_.vw / kTile) : 0),
         tiles_p(VTAIL ? (int)(a_.vs / kTile - a_.vw / kTile) : (int)(a_.vw / kTile)) {
     rows = packed_rows(a.n_rows, a.N);
     const bool packed = rows != a.N;
-    x = reinterpret_cast<const XSrc*>(packed ? a.xc : a.x);
+    x = reinterpret_cast<const E*>(packed ? a.xc : a.x);
     ldx = packed ? a.ldxc : a.ldx;
     tiles_q = (int)((rows + kTile - 1) / kTile);
   }
@@ -191,11 +192,11 @@ template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK> st
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     coords(tile, tp, tq);
-    p = reinterpret_cast<const WSrc*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
+    p = reinterpret_cast<const E*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
     q = x + (int64_t)tq * kTile * ldx;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
-  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(x, rows, ldx, a.H); }
+  LCE_DEV const void* p_end() const { return matrix_end<E>(a.w, a.H, a.ldw, a.Vw); }
+  LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
@@ -204,17 +205,18 @@ template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK> st
   }
 };
 
-template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK>
+template <class T, bool ZREG, bool VTAIL, bool KMASK>
 __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  DzProblem<T, XSrc, WSrc, ZREG, VTAIL, KMASK> prob(a);
-  Pipe3<T, WSrc, false, XSrc, true, DzProblem<T, XSrc, WSrc, ZREG, VTAIL, KMASK>> pipe(prob);
+  typedef typename elem_of<T>::type E;
+  DzProblem<T, ZREG, VTAIL, KMASK> prob(a);
+  Pipe3<T, E, false, E, true, DzProblem<T, ZREG, VTAIL, KMASK>> pipe(prob);
   pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
-template <class T, class XSrc, class WSrc, bool ZREG, bool VTAIL, bool KMASK>
+template <class T, bool ZREG, bool VTAIL, bool KMASK>
 hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = bwd_dz_persistent_kernel<T, XSrc, WSrc, ZREG, VTAIL, KMASK>;
+  auto kern = bwd_dz_persistent_kernel<T, ZREG, VTAIL, KMASK>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e != hipSuccess) return e;
@@ -224,30 +226,28 @@ hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
 }
 
 // All full tile columns of the slab, then the column that straddles the end of the vocabulary.
-template <class T, class XSrc, class WSrc, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
+template <class T, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
   const int64_t tq = a.Np / kTile, full = a.vw / kTile, tail = a.vs / kTile - full;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = exact_k ? launch_one<T, XSrc, WSrc, ZREG, false, false>(a, full * tq, s)
-                           : launch_one<T, XSrc, WSrc, ZREG, false, true>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, ZREG, false, false>(a, full * tq, s)
+                           : launch_one<T, ZREG, false, true>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (tail > 0) return launch_one<T, XSrc, WSrc, ZREG, true, true>(a, tail * tq, s);
+  if (tail > 0) return launch_one<T, ZREG, true, true>(a, tail * tq, s);
   return hipSuccess;
 }
 
-template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  return a.z_reg != 0.f ? launch_persistent_z<T, XSrc, WSrc, true>(a, s)
-                        : launch_persistent_z<T, XSrc, WSrc, false>(a, s);
+template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  return a.z_reg != 0.f ? launch_persistent_z<T, true>(a, s)
+                        : launch_persistent_z<T, false>(a, s);
 }
 
 }  // namespace
 
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
-  typedef elem_of<BF16>::type bf;
-  typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf, bf>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf, hf>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
   // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as the bf16 packed copy)
   return hipErrorInvalidValue;
 }

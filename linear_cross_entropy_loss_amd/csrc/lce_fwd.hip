@@ -155,18 +155,19 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
 // starting at its column tile `tp0` (all full columns, or the one straddling V
 // for the VTAIL variant).  The token rows are those of x, or -- when the tokens with ignored
 // labels were packed away -- the first `rows` rows of the packed copy (the count lives on the device).
-template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdProblem {
+template <class T, bool VTAIL, bool KMASK> struct FwdProblem {
+  typedef typename elem_of<T>::type E;
   static constexpr bool kKMask = KMASK;
   static constexpr bool kVarK = false;
   const FwdArgs& a;
   int64_t rows, ldx;
-  const XSrc* x;
+  const E* x;
   int tp0, tiles_p, tiles_q;
   LCE_DEV FwdProblem(const FwdArgs& a_)
       : a(a_), tp0(VTAIL ? (int)(a_.vw / kTile) : 0), tiles_p(VTAIL ? 1 : (int)(a_.vw / kTile)) {
     rows = a.n_rows ? packed_rows(a.n_rows, a.N) : a.N;
     const bool packed = rows != a.N;
-    x = reinterpret_cast<const XSrc*>(packed ? a.xc : a.x);
+    x = reinterpret_cast<const E*>(packed ? a.xc : a.x);
     ldx = packed ? a.ldxc : a.ldx;
     tiles_q = (int)((rows + kTile - 1) / kTile);
   }
@@ -178,11 +179,11 @@ template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdPro
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     coords(tile, tp, tq);
-    p = reinterpret_cast<const WSrc*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
+    p = reinterpret_cast<const E*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
     q = x + (int64_t)tq * kTile * ldx;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<WSrc>(a.w, a.H, a.ldw, a.Vw); }
-  LCE_DEV const void* q_end() const { return matrix_end<XSrc>(x, rows, ldx, a.H); }
+  LCE_DEV const void* p_end() const { return matrix_end<E>(a.w, a.H, a.ldw, a.Vw); }
+  LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
@@ -191,11 +192,12 @@ template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK> struct FwdPro
   }
 };
 
-template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK>
+template <class T, bool VTAIL, bool KMASK>
 __global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  FwdProblem<T, XSrc, WSrc, VTAIL, KMASK> prob(a);
-  Pipe3<T, WSrc, false, XSrc, true, FwdProblem<T, XSrc, WSrc, VTAIL, KMASK>> pipe(prob);
+  typedef typename elem_of<T>::type E;
+  FwdProblem<T, VTAIL, KMASK> prob(a);
+  Pipe3<T, E, false, E, true, FwdProblem<T, VTAIL, KMASK>> pipe(prob);
   pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
@@ -347,9 +349,9 @@ __global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
   }
 }
 
-template <class T, class XSrc, class WSrc, bool VTAIL, bool KMASK>
+template <class T, bool VTAIL, bool KMASK>
 hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = fwd_tiles_persistent_kernel<T, XSrc, WSrc, VTAIL, KMASK>;
+  auto kern = fwd_tiles_persistent_kernel<T, VTAIL, KMASK>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -359,25 +361,23 @@ hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
 }
 
 // All full tile columns of the vocabulary, then the column that straddles V.
-template <class T, class XSrc, class WSrc> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
+template <class T> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
   const int64_t tq = a.Np / kTile, full = a.vw / kTile;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = exact_k ? launch_one<T, XSrc, WSrc, false, false>(a, full * tq, s)
-                           : launch_one<T, XSrc, WSrc, false, true>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, false, false>(a, full * tq, s)
+                           : launch_one<T, false, true>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (a.vw % kTile) return launch_one<T, XSrc, WSrc, true, true>(a, tq, s);
+  if (a.vw % kTile) return launch_one<T, true, true>(a, tq, s);
   return hipSuccess;
 }
 
 }  // namespace
 
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
-  typedef elem_of<BF16>::type bf;
-  typedef elem_of<F16>::type hf;
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16, bf, bf>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, hf, hf>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
   // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as the bf16 packed copy)
   return hipErrorInvalidValue;
 }
