@@ -81,7 +81,26 @@ typedef struct lce_problem {
   int64_t n_chunk;      /* N_chunk_size: scratch bound n_chunk*V*4 bytes (ops.py:677) */
   int32_t monitoring;   /* 0/1: also produce max / entropy / norm (ops.py:678) */
   int32_t phases;       /* 0 = everything; otherwise a mask of LCE_PHASE_* (profiling aid) */
+  int32_t pack_rows;    /* LCE_PACK_AUTO | LCE_PACK_ALWAYS | LCE_PACK_NEVER: see below        */
+  int32_t reserved;     /* 0                                                                  */
 } lce_problem;
+
+/*
+ * Tokens whose label equals ignore_index add nothing to the loss or to either
+ * gradient (ops.py:213, 314, 422).  With packing the kept rows are gathered to
+ * the front on the device and the tile kernels run on them only, so time
+ * scales with the number of labelled tokens; the pre-pass costs a few small
+ * launches (about 0.07 ms per forward + backward), which a small problem does
+ * not earn back.  LCE_PACK_AUTO packs when 8*N*H*V >= 2^41 FLOPs; results are
+ * the same either way up to the summation order of dW and the loss, and lse of
+ * an ignored row (see lce_forward).  Use the same value in lce_workspace_bytes,
+ * lce_forward and lce_backward of one problem.
+ */
+enum {
+  LCE_PACK_AUTO = 0,
+  LCE_PACK_ALWAYS = 1,
+  LCE_PACK_NEVER = 2
+};
 
 /*
  * Profiling aid: a non-zero lce_problem.phases restricts a call to the named
@@ -138,8 +157,8 @@ int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width)
  * 793-794, 802), without ever writing logits to memory.
  *
  *   lse     out, N floats: logsumexp of the scaled logits of every row whose
- *           label is not ignore_index (with monitoring == 0 the other rows
- *           are not computed at all and get 0)
+ *           label is not ignore_index (when rows are packed and monitoring
+ *           == 0 the other rows are not computed at all and get 0)
  *   out5    out, 5 floats: loss, z_reg, logit_max, logit_entropy, logit_norm
  *           (the 5-tuple of ops.py:802 with the meanings of ops.py:9-17; the
  *           last three are 0 when monitoring == 0)

@@ -32,6 +32,7 @@ int check(const lce_problem* p, bool backward) {
   const bool ok = (is16(xd) && (wd == xd || wd == LCE_F32)) || (xd == LCE_F32 && wd == LCE_F32);
   if (!ok) return LCE_EINVAL_DTYPE;
   if (!(p->logit_scale > 0.f) || !(p->z_reg >= 0.f)) return LCE_EINVAL_ARG;
+  if (p->pack_rows != LCE_PACK_AUTO && p->pack_rows != LCE_PACK_ALWAYS && p->pack_rows != LCE_PACK_NEVER) return LCE_EINVAL_ARG;
   const int64_t xa = xd == LCE_F32 ? 4 : 8, wa = wd == LCE_F32 ? 4 : 8;  // 16-byte rows
   if (p->ldx < p->H || p->ldx % xa || p->ldw < p->V || p->ldw % wa) return LCE_EINVAL_ARG;
   // The kernels address a 256-row tile of x, of a 16-bit W and of dx with 32-bit byte offsets: 256 rows must
@@ -57,6 +58,13 @@ struct PackPlan {
   int64_t ldxc;  // row stride of the packed copy of x, elements: rows of whole 16-byte pieces
   size_t xes;    // element size of the packed copy: that of x, or 2 for fp32 activations (stored rounded to bf16)
 };
+
+// Whether the tokens with an ignored label are packed away before the tile kernels run (lce.h).
+bool packs_rows(const lce_problem* p) {
+  if (p->pack_rows == LCE_PACK_ALWAYS) return true;
+  if (p->pack_rows == LCE_PACK_NEVER) return false;
+  return 8.0 * (double)p->N * (double)p->H * (double)p->V >= 2199023255552.0;  // 2^41
+}
 
 PackPlan plan_pack(const lce_problem* p, size_t base) {
   PackPlan k;
@@ -104,7 +112,7 @@ FwdPlan plan_fwd(const lce_problem* p) {
     if (cols < f.vs) f.vs = cols;
     o += align_up((size_t)p->H * (size_t)f.vs * 2);
   }
-  if (!p->monitoring || p->x_dtype == LCE_F32) {
+  if ((!p->monitoring && packs_rows(p)) || p->x_dtype == LCE_F32) {
     f.pack = plan_pack(p, o);
     o = f.pack.end;
   }
@@ -126,17 +134,10 @@ size_t dx_part_bytes(size_t Np, size_t Hp, int64_t vs, int64_t last_vs) {
   return (size_t)(b0 > b1 ? b0 : b1) * 256 * 256 * 4;
 }
 
-// The same for dW (0 when dW is not split).  A narrower last slab has fewer output tiles and may be
-// split further, so both widths are sized.
+// The same for dW.
 size_t dw_part_bytes(size_t Np, size_t Hp, int64_t vs, int64_t last_vs) {
-  size_t need = 0;
-  for (int64_t w : {vs, last_vs}) {
-    int split, kseg;
-    lce::dw_split_plan((int64_t)Np, (int64_t)Hp, w, &split, &kseg);
-    const size_t b = split > 1 ? align_up((size_t)split * Hp * (size_t)w * 4) : 0;
-    if (b > need) need = b;
-  }
-  return need;
+  const int64_t b0 = lce::dw_tail_blocks((int64_t)Np, (int64_t)Hp, vs), b1 = lce::dw_tail_blocks((int64_t)Np, (int64_t)Hp, last_vs);
+  return (size_t)(b0 > b1 ? b0 : b1) * 256 * 256 * 4;
 }
 
 // Fewest vocabulary slabs (of a width that is a multiple of 256 columns; the last
@@ -158,11 +159,14 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   const int64_t Vp = lce::padded_vocab(p->V);
   const int64_t cols = Vp / 256;
   // buffers of the packed rows come first and count towards the bound
+  const bool pack = packs_rows(p);
   b->pack = plan_pack(p, 0);
   b->lddxc = lce::pad_to(p->H, 8);
   b->lse_c = b->pack.end;
   b->dxc = b->lse_c + align_up((size_t)p->N * 4);
-  const size_t fixed = b->dxc + align_up((size_t)p->N * (size_t)b->lddxc * (p->dx_dtype == LCE_F32 ? 4 : 2));
+  size_t fixed = 0;  // (fp32 activations need the packed copy of x even when rows are not packed)
+  if (pack) fixed = b->dxc + align_up((size_t)p->N * (size_t)b->lddxc * (p->dx_dtype == LCE_F32 ? 4 : 2));
+  else if (p->x_dtype == LCE_F32) fixed = b->pack.end;
   for (int pass = 0; pass < 2; ++pass) {
     const size_t budget = strict + (pass ? (size_t)p->N * (size_t)p->H * 4 : 0);
     for (int64_t s = 1; s <= cols; ++s) {
@@ -289,7 +293,7 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
 
   const int ph = p->phases ? p->phases : ~0;
   hipError_t e;
-  const bool pack = !p->monitoring, x32 = p->x_dtype == LCE_F32;
+  const bool pack = !p->monitoring && packs_rows(p), x32 = p->x_dtype == LCE_F32;
   if (pack || x32) {
     const PackPlan& k = f.pack;
     if (pack) {
@@ -379,23 +383,30 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
 
   // Tokens with an ignored label have dz == 0: the kernels run on the other rows only, packed to the front.
   const PackPlan& k = b.pack;
-  const bool x32 = p->x_dtype == LCE_F32;
+  const bool pack = packs_rows(p), x32 = p->x_dtype == LCE_F32;
   const int64_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
-  a.n_rows = (const int64_t*)(base + k.n_rows);
   a.xc = base + k.xc;
   a.ldxc = k.ldxc;
-  a.dxc = base + b.dxc;
-  a.lddxc = b.lddxc;
-  a.y = (const int64_t*)(base + k.yc);
-  a.lse = (const float*)(base + b.lse_c);
-  if (ph & LCE_PHASE_PACK) {
-    hipError_t e = lce::launch_compact_labels(y, p->N, p->ignore_index, (int*)(base + k.cnt), (int64_t*)(base + k.n_rows),
-                                              (int*)(base + k.perm), (int64_t*)(base + k.yc), s);
-    if (e != hipSuccess) return hip_fail(e, "compact_labels");
-    e = x32 ? lce::launch_gather_rows_f32((const float*)x, p->ldx, p->H, (const int*)(base + k.perm), a.n_rows, p->N,
-                                          base + k.xc, k.ldxc, lse, (float*)(base + b.lse_c), a.num_cus, s)
-            : lce::launch_gather_rows(x, p->ldx * 2, (const int*)(base + k.perm), a.n_rows, p->N, base + k.xc, k.ldxc * 2,
-                                      lse, (float*)(base + b.lse_c), a.num_cus, s);
+  if (pack) {
+    a.n_rows = (const int64_t*)(base + k.n_rows);
+    a.dxc = base + b.dxc;
+    a.lddxc = b.lddxc;
+    a.y = (const int64_t*)(base + k.yc);
+    a.lse = (const float*)(base + b.lse_c);
+  }
+  if ((pack || x32) && (ph & LCE_PHASE_PACK)) {
+    const int* perm = pack ? (const int*)(base + k.perm) : nullptr;
+    hipError_t e;
+    if (pack) {
+      e = lce::launch_compact_labels(y, p->N, p->ignore_index, (int*)(base + k.cnt), (int64_t*)(base + k.n_rows),
+                                     (int*)(base + k.perm), (int64_t*)(base + k.yc), s);
+      if (e != hipSuccess) return hip_fail(e, "compact_labels");
+    }
+    float* lse_c = pack ? (float*)(base + b.lse_c) : nullptr;
+    e = x32 ? lce::launch_gather_rows_f32((const float*)x, p->ldx, p->H, perm, a.n_rows, p->N, base + k.xc, k.ldxc,
+                                          pack ? lse : nullptr, lse_c, a.num_cus, s)
+            : lce::launch_gather_rows(x, p->ldx * 2, perm, a.n_rows, p->N, base + k.xc, k.ldxc * 2, lse, lse_c,
+                                      a.num_cus, s);
     if (e != hipSuccess) return hip_fail(e, "gather_rows");
   }
   if (x32) {  // fp32 activations reach the tile kernels as the bf16 packed copy, whether or not rows were dropped
@@ -409,7 +420,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     a.vw = p->V - a.v0 < b.vs ? p->V - a.v0 : b.vs;   // columns of this slab that exist
     a.vs = lce::pad_to(a.vw, 256);                    // its padded width: dz row stride and K extent of dx
     a.dx_grid = a.num_cus;
-    lce::dw_split_plan(a.Np, a.Hp, a.vs, &a.dw_split, &a.dw_kseg);
+    a.dw_grid = a.num_cus;
     hipError_t e;
     if (p->w_dtype == LCE_F32) {
       // dz and dx of this slab read a 16-bit copy of its columns of the fp32 weight
@@ -436,7 +447,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
       if (e != hipSuccess) return hip_fail(e, "bwd_dw");
     }
   }
-  if (dx && (ph & LCE_PHASE_BWD_DX)) {
+  if (pack && dx && (ph & LCE_PHASE_BWD_DX)) {
     // packed dx rows go to their tokens, dropped tokens get exact zeros (nothing to do if none was dropped)
     hipError_t e = lce::launch_scatter_rows(a.dxc, b.lddxc * dxes, (const int*)(base + k.perm), a.n_rows, p->N, y,
                                             p->ignore_index, dx, p->lddx * dxes, p->H * dxes, a.num_cus, s);

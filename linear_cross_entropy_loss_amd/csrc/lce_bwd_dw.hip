@@ -12,14 +12,21 @@ namespace lce {
 
 namespace {
 
+// `part` != null: this is a K segment of a tail tile (see DwPlan); its raw fp32 sum goes to that
+// 256(h) x 256(v) block, through the statements of the fp32 output path (another destination, row
+// stride and factor, no bounds) -- a separate code path behind a branch would read the accumulator twice.
 template <class T>
-LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
+LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   typedef typename elem_of<T>::type E;
   const int64_t vl0 = (int64_t)tp * kTile, h0 = (int64_t)tq * kTile;
   const int tid = opaque_tid();
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
-  const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
+  const bool tail = part != nullptr;
+  const float coef = tail ? 1.f : a.grad_out[0] * a.scale / (float)a.n_valid[0];
+  // fp32 destination addressed as [h][v] with v counted over the whole vocabulary
+  float* f32dst = tail ? part - (h0 * kTile + a.v0 + vl0) : reinterpret_cast<float*>(a.dw);
+  const int64_t f32ld = tail ? kTile : a.lddw;
   const int half = lane >> 5;
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
@@ -30,14 +37,14 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
       const int64_t vb = a.v0 + vl0 + wp * kWaveTile + pb * kBlk;
       // Pieces (4 columns in fp32, 8 in the 16-bit types) that start at or past V are not
       // stored; one that V cuts through is written whole, into the stride padding of its row.
-      if (a.dw_dtype == DT_F32) {
+      if (a.dw_dtype == DT_F32 || tail) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-          if (vb + 8 * rq + 4 * half >= a.V || !row_exists) continue;
+          if (!tail && (vb + 8 * rq + 4 * half >= a.V || !row_exists)) continue;
           f32x4_t o;
 #pragma unroll
           for (int j = 0; j < 4; ++j) o[j] = acc[pb][qb][rq * 4 + j] * coef;
-          *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + h * a.lddw + vb + 8 * rq + 4 * half) = o;
+          *reinterpret_cast<f32x4_t*>(f32dst + h * f32ld + vb + 8 * rq + 4 * half) = o;
         }
       } else {
         // Lanes l and l+32 hold the two halves of every run of 8 columns; one
@@ -65,64 +72,76 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, in
   }
 }
 
-// Split mode: the raw fp32 partial sum of K segment `seg` goes to dw_part[seg][Hp][vs].
-LCE_DEV void dw_partial_epilogue(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, int seg) {
-  const int64_t vl0 = (int64_t)tp * kTile, h0 = (int64_t)tq * kTile;
-  const int tid = opaque_tid();
-  const int lane = tid & 63, wave = tid >> 6;
-  const int wp = wave & 1, wq = wave >> 1;
-  float* part = a.dw_part + (int64_t)seg * a.Hp * a.vs;
-#pragma unroll
-  for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t h = h0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-#pragma unroll
-    for (int pb = 0; pb < kNB; ++pb)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int64_t vl = vl0 + wp * kWaveTile + pb * kBlk + 8 * rq + 4 * (lane >> 5);
-        f32x4_t v;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = acc[pb][qb][rq * 4 + j];
-        *reinterpret_cast<f32x4_t*>(part + h * a.vs + vl) = v;
-      }
+// How one launch divides its work: as for dx (lce_bwd_dx.hip).  The T = (vs/256) x (Hp/256) output tiles
+// go to G persistent workgroups in rounds; a last round with r <= G/2 tiles is cut along K = tokens into
+// `nseg` segments of `kseg` K tiles (r * nseg <= G, at least 16 K tiles each), whose fp32 sums meet in
+// 256 x 256 blocks of dw_part and are added, in segment order, by dw_tail_kernel.  With few tiles in all
+// (a small vocabulary slab times a small hidden size) every tile is a tail tile.  The K extent comes from
+// the row count on the device, so the plan is made there; a last segment that runs past the rows reads zeros.
+struct DwPlan {
+  int tiles, full, tail_tiles, nseg, kseg, kt;
+};
+LCE_DEV DwPlan dw_plan(const BwdArgs& a, int64_t rows) {
+  DwPlan p;
+  const int G = a.dw_grid;
+  const int64_t kt2 = (rows + 2 * kBK - 1) / (2 * kBK) * 2;  // K tiles: an even number, at least four, covering the rows
+  p.kt = (int)(kt2 < 4 ? 4 : kt2);
+  p.tiles = (int)(a.vs / kTile) * (int)(a.Hp / kTile);
+  p.full = p.tiles / G * G;
+  const int r = p.tiles - p.full, cap = G < kTailBlocks ? G : kTailBlocks;
+  int s = 1;
+  if (r > 0)
+    while (r * s * 2 <= cap && p.kt / (s * 2) >= 16) s *= 2;
+  if (s == 1) {
+    p.full = p.tiles;
+    p.tail_tiles = 0;
+    p.nseg = 1;
+    p.kseg = p.kt;
+  } else {
+    const int seg = ((p.kt + s - 1) / s + 1) & ~1;  // even
+    p.tail_tiles = r;
+    p.kseg = seg;
+    p.nseg = (p.kt + seg - 1) / seg;
   }
+  return p;
 }
 
-// Work item = (output tile, K segment), segment fastest (see the dx kernel).
-template <class T, bool SPLIT> struct DwProblem {
-  static constexpr bool kVarK = false;
+template <class T> struct DwProblem {
+  static constexpr bool kVarK = true;    // whole tiles and segment items have different K extents
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows (the K extent): all of x, or the packed rows (see BwdArgs)
   const E* x;
-  int tiles_p, tiles_q, split, kseg;
-  LCE_DEV DwProblem(const BwdArgs& a_)
-      : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.Hp / kTile)), split(SPLIT ? a_.dw_split : 1),
-        kseg(a_.dw_kseg) {
+  int tiles_p, tiles_q;
+  DwPlan plan;
+  LCE_DEV DwProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.Hp / kTile)) {
     rows = packed_rows(a.n_rows, a.N);
     const bool packed = rows != a.N;
     x = reinterpret_cast<const E*>(packed ? a.xc : a.x);
     ldx = packed ? a.ldxc : a.ldx;
+    plan = dw_plan(a, rows);
   }
-  // K tiles of an unsplit contraction: an even number, at least four, covering the rows
-  LCE_DEV int ktiles() const {
-    const int64_t kt = (rows + 2 * kBK - 1) / (2 * kBK) * 2;
-    return (int)(kt < 4 ? 4 : kt);
-  }
-  LCE_DEV int num_tiles() const { return tiles_p * tiles_q * split; }
+  LCE_DEV int num_tiles() const { return plan.full + plan.tail_tiles * plan.nseg; }
+  // seg < 0: a whole tile
   LCE_DEV void decode(int item, int& tp, int& tq, int& seg) const {
-    seg = SPLIT ? item % split : 0;
-    tile_coords(SPLIT ? item / split : item, tiles_p * tiles_q, tiles_p, tiles_q, 4, tp, tq);
+    int tile = item;
+    seg = -1;
+    if (item >= plan.full) {
+      const int j = item - plan.full;
+      tile = plan.full + j / plan.nseg;
+      seg = j % plan.nseg;
+    }
+    tile_coords(tile, plan.tiles, tiles_p, tiles_q, 4, tp, tq);
   }
+  LCE_DEV int item_ktiles(int item) const { return item < plan.full ? plan.kt : plan.kseg; }
   LCE_DEV void origins(int item, const void*& p, const void*& q) const {
     int tp, tq, seg;
     decode(item, tp, tq, seg);
-    const int64_t k0 = (int64_t)seg * kseg * kBK;  // first token of the segment
+    const int64_t k0 = seg < 0 ? 0 : (int64_t)seg * plan.kseg * kBK;  // first token of the segment
     p = reinterpret_cast<const E*>(a.dz) + k0 * a.vs + (int64_t)tp * kTile;
     q = x + k0 * ldx + (int64_t)tq * kTile;
   }
-  // rows past the end of either operand (a last segment running past the tokens) read as zeros
   // dz is written for whole token tiles; x rows past the last one read as zeros
   LCE_DEV const void* p_end() const {
     return reinterpret_cast<const E*>(a.dz) + (rows + kTile - 1) / kTile * kTile * a.vs;
@@ -132,67 +151,65 @@ template <class T, bool SPLIT> struct DwProblem {
   LCE_DEV void epilogue(int item, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq, seg;
     decode(item, tp, tq, seg);
-    if (SPLIT) {
-      dw_partial_epilogue(a, acc, tp, tq, seg);
-    } else {
-      dw_epilogue<T>(a, acc, tp, tq);
-    }
+    float* part = seg >= 0 ? a.dw_part + (int64_t)(item - plan.full) * kTile * kTile : nullptr;
+    dw_epilogue<T>(a, part, acc, tp, tq);
   }
 };
 
-template <class T, bool SPLIT>
+template <class T>
 __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DwProblem<T, SPLIT> prob(a);
-  Pipe3<T, E, false, E, false, DwProblem<T, SPLIT>> pipe(prob);
-  pipe.run(a.vs, prob.ldx, SPLIT ? a.dw_kseg : prob.ktiles(), lds);
+  DwProblem<T> prob(a);
+  Pipe3<T, E, false, E, false, DwProblem<T>> pipe(prob);
+  pipe.run(a.vs, prob.ldx, prob.plan.kt, lds);
 }
 
-// Split mode, second step: dW[:, slab] = coef * sum over segments, in segment order.
+// Second step for the tail tiles: kTailParts workgroups share tail tile b (16 rows of h each) -- they sum
+// its segments in order, scale, and store dW[:, slab] in the output dtype.
+constexpr int kTailParts = 16;
 template <class T>
-__global__ __launch_bounds__(256) void dw_reduce_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(256) void dw_tail_kernel(const BwdArgs a) {
   typedef typename elem_of<T>::type E;
-  const int64_t quads_per_row = a.vs / 4;
-  const int64_t total = a.H * quads_per_row;
+  const DwPlan plan = dw_plan(a, packed_rows(a.n_rows, a.N));
+  const int b = (int)blockIdx.x / kTailParts, piece = (int)blockIdx.x % kTailParts;
+  if (b >= plan.tail_tiles) return;
+  int tp, tq;
+  tile_coords(plan.full + b, plan.tiles, (int)(a.vs / kTile), (int)(a.Hp / kTile), 4, tp, tq);
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t h = i / quads_per_row, vl = (i - h * quads_per_row) * 4;
-    const int64_t v = a.v0 + vl;
-    if (v >= a.V) continue;  // a quad that V cuts through is written whole, into the stride padding of its row
-    const int64_t o = h * a.vs + vl;
-    f32x4_t acc = *reinterpret_cast<const f32x4_t*>(a.dw_part + o);
-    for (int s = 1; s < a.dw_split; ++s) acc += *reinterpret_cast<const f32x4_t*>(a.dw_part + (int64_t)s * a.Hp * a.vs + o);
+  const float* part = a.dw_part + (int64_t)b * plan.nseg * kTile * kTile;
+  constexpr int kQuads = kTile * kTile / 4 / kTailParts;
+  for (int i = piece * kQuads + threadIdx.x; i < (piece + 1) * kQuads; i += 256) {
+    const int row = i / (kTile / 4), vl = (i - row * (kTile / 4)) * 4;
+    const int64_t h = (int64_t)tq * kTile + row, v = a.v0 + (int64_t)tp * kTile + vl;
+    if (h >= a.H || v >= a.V) continue;  // a quad that V cuts through is written whole, into the stride padding of its row
+    f32x4_t acc = *reinterpret_cast<const f32x4_t*>(part + row * kTile + vl);
+#pragma unroll 4
+    for (int s = 1; s < plan.nseg; ++s)
+      acc += *reinterpret_cast<const f32x4_t*>(part + (int64_t)s * kTile * kTile + row * kTile + vl);
     if (a.dw_dtype == DT_F32) {
       *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + h * a.lddw + v) = acc * coef;
     } else {
-      u32x2_t b;
-      b[0] = pack2<T>(acc[0] * coef, acc[1] * coef);
-      b[1] = pack2<T>(acc[2] * coef, acc[3] * coef);
-      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + v) = b;
+      u32x2_t o;
+      o[0] = pack2<T>(acc[0] * coef, acc[1] * coef);
+      o[1] = pack2<T>(acc[2] * coef, acc[3] * coef);
+      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + v) = o;
     }
   }
 }
 
-template <class T, bool SPLIT> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dw_persistent_kernel<T, SPLIT>;
+template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dw_persistent_kernel<T>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
-  const int64_t items = (a.vs / kTile) * (a.Hp / kTile) * (SPLIT ? a.dw_split : 1);
-  const int grid = (int)(items < a.num_cus ? items : a.num_cus);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);
-  return hipGetLastError();
-}
-
-template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  if (a.dw_split <= 1) return launch_tiles<T, false>(a, s);
-  hipError_t e = launch_tiles<T, true>(a, s);
+  hipLaunchKernelGGL(kern, dim3(a.dw_grid), dim3(kThreads), kMainloopLds, s, a);
+  e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const int64_t quads = a.H * (a.vs / 4);
-  int64_t blocks = (quads + 255) / 256;
-  if (blocks > 2048) blocks = 2048;
-  hipLaunchKernelGGL(dw_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, a);
+  if (dw_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // this launch cannot have a split tail
+  // at most dw_grid / 2 tail tiles can be split (two segments each)
+  const unsigned tail_most = (unsigned)(a.dw_grid / 2 > 0 ? a.dw_grid / 2 : 1);
+  hipLaunchKernelGGL(dw_tail_kernel<T>, dim3(tail_most * kTailParts), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 

@@ -94,19 +94,20 @@ LCE_DEV DxPlan dx_plan(const BwdArgs& a, int tiles) {
   const int G = a.dx_grid, kt = (int)(a.vs / kBK);
   p.tiles = tiles;
   p.full = tiles / G * G;
-  const int r = tiles - p.full, cap = G < kDxTailBlocks ? G : kDxTailBlocks;
+  const int r = tiles - p.full, cap = G < kTailBlocks ? G : kTailBlocks;
   int s = 1;
   if (r > 0)
-    while (r * s * 2 <= cap && kt % (s * 4) == 0 && kt / (s * 2) >= 16) s *= 2;
+    while (r * s * 2 <= cap && kt / (s * 2) >= 16) s *= 2;
   if (s == 1) {
     p.full = tiles;
     p.tail_tiles = 0;
     p.nseg = 1;
     p.kseg = kt;
   } else {
+    // an even number of K tiles per segment; a last segment that runs past the slab is masked (K mask)
     p.tail_tiles = r;
-    p.nseg = s;
-    p.kseg = kt / s;  // even: kt is a multiple of 2 s
+    p.kseg = ((kt + s - 1) / s + 1) & ~1;
+    p.nseg = (kt + p.kseg - 1) / p.kseg;
   }
   return p;
 }
@@ -193,15 +194,10 @@ __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
     const int row = i / (kTile / 4), hl = (i - row * (kTile / 4)) * 4;
     const int64_t tok = (int64_t)tq * kTile + row, h = (int64_t)tp * kTile + hl;
     if (tok >= rows || h >= a.H) continue;
-    // nseg is a power of two >= 2: two segments per step keep two loads in flight, the sum stays in segment order
     f32x4_t v = *reinterpret_cast<const f32x4_t*>(part + row * kTile + hl);
-    v += *reinterpret_cast<const f32x4_t*>(part + (int64_t)kTile * kTile + row * kTile + hl);
-    for (int s = 2; s < plan.nseg; s += 2) {
-      const f32x4_t u0 = *reinterpret_cast<const f32x4_t*>(part + (int64_t)s * kTile * kTile + row * kTile + hl);
-      const f32x4_t u1 = *reinterpret_cast<const f32x4_t*>(part + (int64_t)(s + 1) * kTile * kTile + row * kTile + hl);
-      v += u0;
-      v += u1;
-    }
+#pragma unroll 4
+    for (int s = 1; s < plan.nseg; ++s)
+      v += *reinterpret_cast<const f32x4_t*>(part + (int64_t)s * kTile * kTile + row * kTile + hl);
     const int64_t o = tok * a.Hp + h;
     if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + o);
     if (!a.last) {
@@ -227,8 +223,9 @@ template <class T, bool KMASK> hipError_t launch_tiles(const BwdArgs& a, hipStre
 }
 
 template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  // the K mask is only needed when the K tiles run past the columns that exist (segments divide the K tiles evenly)
-  hipError_t e = a.vw == a.vs ? launch_tiles<T, false>(a, s) : launch_tiles<T, true>(a, s);
+  // the K mask is only needed when the K tiles of a work item can run past the columns that exist
+  const bool exact_k = a.vw == a.vs && dx_segments_exact(a.vs);
+  hipError_t e = exact_k ? launch_tiles<T, false>(a, s) : launch_tiles<T, true>(a, s);
   if (e != hipSuccess) return e;
   if (dx_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // no shape of this launch can have a split tail
   // at most dx_grid / 2 tail tiles can be split (two segments each)

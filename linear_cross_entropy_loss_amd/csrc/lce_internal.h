@@ -85,15 +85,15 @@ struct BwdArgs {
   // floats, and a small kernel adds them in a fixed order.  dx_grid = workgroups of the tile kernel.
   int dx_grid;
   float* dx_part;
-  // The same for dW with few output tiles (small vocabulary slab x hidden size): K = tokens is cut into
-  // dw_split segments of dw_kseg K tiles; partial sums in dw_part [dw_split][Hp][vs] (fp32).
-  int dw_split, dw_kseg;
+  // The same for dW (K = tokens): dw_part holds dw_tail_blocks() blocks, dw_grid = workgroups of the tile kernel.
+  int dw_grid;
   float* dw_part;
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
-  // Packed rows (tokens with an ignored label dropped).  *n_rows (device) rows are worked on.  When
-  // *n_rows != N they are the rows of xc (row stride ldxc), dx goes to dxc (row stride lddxc, moved to
-  // its place afterwards), and in either case `y` and `lse` hold the labels / lse of the packed rows.
+  // Packed rows (tokens with an ignored label dropped; n_rows == null: the call works on all rows).
+  // *n_rows (device) rows are worked on.  When *n_rows != N they are the rows of xc (row stride ldxc), dx
+  // goes to dxc (row stride lddxc, moved to its place afterwards), and in either case `y` and `lse` hold
+  // the labels / lse of the packed rows.
   const int64_t* n_rows;
   const void* xc;
   int64_t ldxc;
@@ -115,6 +115,7 @@ hipError_t launch_convert_w_slab(const float* src, int64_t ld, int64_t H, int64_
 // into range: a call restricted to some phases on a workspace whose packing pre-pass did not run must
 // give wrong numbers, not wild addresses.
 __device__ __forceinline__ int64_t packed_rows(const int64_t* n_rows, int64_t N) {
+  if (n_rows == nullptr) return N;  // this call works on all rows
   const int64_t r = n_rows[0];
   return r < 0 ? 0 : (r > N ? N : r);
 }
@@ -144,32 +145,30 @@ hipError_t launch_scatter_rows(const void* dxc, int64_t lddxc_bytes, const int* 
                                int64_t N, const int64_t* y, int64_t ignore_index, void* dx, int64_t lddx_bytes,
                                int64_t row_bytes, int num_cus, hipStream_t s);
 
-// Split of a contraction with few output tiles along K (host side, shared by planning and launch):
-// with `tiles` output tiles on a device assumed to run 256 workgroups, up to 256/tiles segments of
-// at least 16 K tiles each (a power of two, so that segments map onto XCDs evenly).
-inline void k_split_plan(int64_t tiles, int64_t ktiles, int* split, int* kseg) {
-  int s = 1;
-  while (tiles * s * 2 <= 256 && ktiles / (s * 2) >= 16) s *= 2;
-  int64_t seg = (ktiles + s - 1) / s;
-  seg = (seg + 1) & ~(int64_t)1;  // an even number of K tiles, as the pipelined loop requires
-  if (seg < 4) seg = 4;
-  *kseg = (int)seg;
-  *split = (int)((ktiles + seg - 1) / seg);
-}
 // dx of one slab: at most (Np/256) x (Hp/256) tiles, K = vs columns.  Upper bound on the 256 x 256 fp32
 // blocks of partial sums that the device-side plan of the dx kernel can ask for (0: it never splits).
-constexpr int kDxTailBlocks = 256;
+constexpr int kTailBlocks = 256;
+// most segments per tile: a power of two that leaves at least 16 K tiles per segment
+inline int64_t max_k_segments(int64_t kt) {
+  int64_t s = 1;
+  while (kt / (s * 2) >= 16 && s * 2 <= kTailBlocks) s *= 2;
+  return s;
+}
 inline int64_t dx_tail_blocks(int64_t Np, int64_t Hp, int64_t vs) {
-  const int64_t kt = vs / 64;
-  int64_t s = 1;  // most segments per tile: a power of two with at least 16 K tiles each, an even number
-  while (kt % (s * 4) == 0 && kt / (s * 2) >= 16) s *= 2;
+  const int64_t s = max_k_segments(vs / 64);
   if (s == 1) return 0;
   const int64_t most = (Np / 256) * (Hp / 256) * s;
-  return most < kDxTailBlocks ? most : kDxTailBlocks;
+  return most < kTailBlocks ? most : kTailBlocks;
 }
-// dW of one slab: (vs/256) x (Hp/256) tiles, K = Np tokens
-inline void dw_split_plan(int64_t Np, int64_t Hp, int64_t vs, int* split, int* kseg) {
-  k_split_plan((vs / 256) * (Hp / 256), Np / 64, split, kseg);
+// true if every split the dx kernel may choose cuts the K tiles of a slab into equal, even segments
+inline bool dx_segments_exact(int64_t vs) { return (vs / 64) % (2 * max_k_segments(vs / 64)) == 0; }
+// dW of one slab: (vs/256) x (Hp/256) tiles, K = at most Np tokens.  The same bound for the dW kernel, whose
+// segments need not divide the K tiles evenly.
+inline int64_t dw_tail_blocks(int64_t Np, int64_t Hp, int64_t vs) {
+  const int64_t s = max_k_segments(Np / 64);
+  if (s == 1) return 0;
+  const int64_t most = (vs / 256) * (Hp / 256) * s;
+  return most < kTailBlocks ? most : kTailBlocks;
 }
 
 }  // namespace lce

@@ -29,6 +29,12 @@ from . import _lib
 fwd_configs: list = []
 bwd_configs: list = []
 
+# Whether tokens whose label is ignore_index are packed away on the device before the tile kernels run:
+# _lib.PACK_AUTO (the library decides by problem size: the pre-pass costs about 0.07 ms per step, which
+# a small problem does not earn back), _lib.PACK_ALWAYS or _lib.PACK_NEVER.  Results do not depend on it
+# beyond the summation order of dW and of the loss.
+PACK_ROWS = _lib.PACK_AUTO
+
 
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
@@ -88,7 +94,7 @@ def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_ch
             raise ValueError("labels must have one entry per input row")
         prob = _lib.make_problem(
             N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-            ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring,
+            ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring, 0, PACK_ROWS,
         )
         lib = _lib.load()
         _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")
@@ -119,7 +125,7 @@ def _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regulari
             prob = _lib.make_problem(
                 N, H, V, x.stride(0), w.stride(0), dx.stride(0) if need_dx else H + (-H) % 8,
                 dw.stride(0) if need_dw else V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-                ignore_index, logit_scale, z_regularization, N_chunk_size, False,
+                ignore_index, logit_scale, z_regularization, N_chunk_size, False, 0, PACK_ROWS,
             )
             lib = _lib.load()
             _, bwd_bytes = _lib.workspace_bytes(prob)

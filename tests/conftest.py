@@ -31,3 +31,24 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_generate_tests(metafunc):
+    # GPU tests run twice: with the tokens of ignored labels packed away before the tile kernels, and
+    # without (by default the library chooses by problem size, which would leave small test shapes unpacked)
+    if metafunc.definition.get_closest_marker("gpu") is not None and "pack_mode" in metafunc.fixturenames:
+        metafunc.parametrize("pack_mode", ["pack", "nopack"], indirect=True)
+
+
+@pytest.fixture(autouse=True)
+def pack_mode(request):
+    mode = getattr(request, "param", None)
+    if mode is None:
+        yield None
+        return
+    from linear_cross_entropy_loss_amd import _lib, ops
+
+    old = ops.PACK_ROWS
+    ops.PACK_ROWS = _lib.PACK_ALWAYS if mode == "pack" else _lib.PACK_NEVER
+    yield mode
+    ops.PACK_ROWS = old

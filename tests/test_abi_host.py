@@ -49,7 +49,7 @@ def test_struct_layout_matches_header():
     fields = re.findall(r"^\s*(int64_t|int32_t|float)\s+(\w+);", body, flags=re.M)
     ctype = {"int64_t": ctypes.c_int64, "int32_t": ctypes.c_int32, "float": ctypes.c_float}
     assert [(n, ctype[t]) for t, n in fields] == list(_lib.LceProblem._fields_)
-    assert ctypes.sizeof(_lib.LceProblem) == 7 * 8 + 4 * 4 + 8 + 2 * 4 + 8 + 2 * 4
+    assert ctypes.sizeof(_lib.LceProblem) == 7 * 8 + 4 * 4 + 8 + 2 * 4 + 8 + 4 * 4
 
 
 def test_shape_contract(lib):
@@ -81,6 +81,7 @@ def test_shape_contract(lib):
     assert lib.lce_check_problem(ctypes.byref(_prob(ldx=big))) == _lib.LCE_EINVAL_ARG
     assert lib.lce_check_problem(ctypes.byref(_prob(lddx=big))) == _lib.LCE_EINVAL_ARG
     assert lib.lce_check_problem(ctypes.byref(_prob(N=1 << 30, V=1 << 20, ldw=1 << 20, lddw=1 << 20))) == _lib.LCE_EINVAL_SHAPE
+    assert lib.lce_check_problem(ctypes.byref(_prob(pack_rows=3))) == _lib.LCE_EINVAL_ARG
     assert lib.lce_check_problem(None) == _lib.LCE_EINVAL_ARG
 
 
@@ -128,13 +129,14 @@ def test_budget_is_a_target_not_a_refusal():
 
     N, H, nc = 16384, 2048, 4096
     for V in (256, 4096, 8192):     # one slab fits the widened bound: no running dx at all
-        p = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc)
+        p = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc, pack_rows=_lib.PACK_ALWAYS)
         assert _lib.backward_plan(p) == (1, V)
         _, bwd = _lib.workspace_bytes(p)
         # dz for all tokens within the widened bound; on top: the packed rows and at most 64 MiB each of
         # K-split partial sums of dW (few dW tiles) and of dx (room for a split last round of tiles)
         assert nc * V * 4 < N * V * 2 <= nc * V * 4 + N * H * 4 and 0 <= bwd - N * V * 2 - _pack_bytes(N, H) <= 128 << 20
-    p = _prob(N=65536, H=256, V=4096, ldx=256, ldw=4096, lddx=256, lddw=4096, n_chunk=64)   # nothing fits
+    p = _prob(N=65536, H=256, V=4096, ldx=256, ldw=4096, lddx=256, lddw=4096, n_chunk=64,
+              pack_rows=_lib.PACK_ALWAYS)   # nothing fits
     assert _lib.backward_plan(p) == (16, 256)
     _, bwd = _lib.workspace_bytes(p)
     # dz + fp32 running dx (256 dx tiles: no K split) + the split-K partials of the single dW tile
@@ -146,35 +148,28 @@ def test_backward_plan_is_consistent_with_workspace():
 
     pad = lambda v, m: -(-v // m) * m
 
-    def k_split(tiles, ktiles):
-        # a contraction with few output tiles is split along K: up to 256/tiles segments of >= 16 K tiles
-        # (a power of two), an even number of K tiles each
-        s = 1
-        while tiles * s * 2 <= 256 and ktiles // (s * 2) >= 16:
-            s *= 2
-        seg = max(4, (-(-ktiles // s) + 1) & ~1)
-        return -(-ktiles // seg)
-
     def dx_part_bytes(Np, Hp, vs, last_vs):
         # dx: the tiles of a last, mostly idle round of workgroups are cut along K on the device; room for the
         # most 256 x 256 fp32 blocks that can ask for: (tiles x most segments per tile), capped at 256
         def blocks(w):
             kt, s = w // 64, 1
-            while kt % (s * 4) == 0 and kt // (s * 2) >= 16:
+            while kt // (s * 2) >= 16 and s * 2 <= 256:
                 s *= 2
             return 0 if s == 1 else min(256, (Np // 256) * (Hp // 256) * s)
         return max(blocks(vs), blocks(last_vs)) * 256 * 256 * 4
 
     def dw_part_bytes(Np, Hp, vs, last_vs):
-        need = 0
-        for w in (vs, last_vs):
-            split = k_split((w // 256) * (Hp // 256), Np // 64)
-            need = max(need, split * Hp * w * 4 if split > 1 else 0)
-        return need
+        # the same for dW, whose K runs over the tokens and whose segments need not divide the K tiles evenly
+        def blocks(w):
+            kt, s = Np // 64, 1
+            while kt // (s * 2) >= 16 and s * 2 <= 256:
+                s *= 2
+            return 0 if s == 1 else min(256, (w // 256) * (Hp // 256) * s)
+        return max(blocks(vs), blocks(last_vs)) * 256 * 256 * 4
 
     for N, H, V, nc in ((16384, 2048, 131072, 4096), (16384, 2048, 131072, 8192), (65536, 8192, 262144, 8192),
                         (512, 256, 4096, 512), (1000, 520, 50264, 512), (300, 104, 1008, 64), (16384, 768, 50264, 4096)):
-        p = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc)
+        p = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc, pack_rows=_lib.PACK_ALWAYS)
         slabs, width = _lib.backward_plan(p)
         # slabs of `width` columns (a multiple of 256) cover the vocabulary; the last one may be narrower
         assert width % 256 == 0 and (slabs - 1) * width < V <= slabs * width
@@ -185,6 +180,13 @@ def test_backward_plan_is_consistent_with_workspace():
         assert part <= 64 << 20 and partw <= 64 << 20
         assert bwd == _pack_bytes(N, H) + Np * width * 2 + (Np * Hp * 4 if slabs > 1 else 0) + part + partw
         assert Np * width * 2 <= max(1 << 30, Np * 256 * 2)   # dz stage capped at 1 GiB
+        # without the packing of ignored tokens: the same minus its buffers, if the split stays the same;
+        # by default the library packs from 8*N*H*V = 2^41 FLOPs on
+        q = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc, pack_rows=_lib.PACK_NEVER)
+        if _lib.backward_plan(q) == (slabs, width):
+            assert _lib.workspace_bytes(q)[1] == bwd - _pack_bytes(N, H)
+        auto = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=nc)
+        assert _lib.workspace_bytes(auto) == _lib.workspace_bytes(p if 8 * N * H * V >= 2 ** 41 else q)
 
 
 def test_fp32_weight_adds_one_16_bit_slab_copy_to_the_scratch():

@@ -38,7 +38,10 @@ def test_ignored_rows_are_never_read_so_nan_in_them_is_harmless():
     """Tokens with an ignored label are dropped before the tile kernels, so even NaN / Inf in their rows of
     x leaves loss, dx and dW bit-identical (the reference's x^T dz would give NaN * 0 = NaN, ops.py:424).
     With monitoring on, logit_max and logit_norm are taken over all rows (ops.py:15, 17) and do see them."""
+    from linear_cross_entropy_loss_amd import _lib, ops
+
     print("NaN in ignored rows", flush=True)
+    ops.PACK_ROWS = _lib.PACK_ALWAYS  # (the fixture restores it)
     x, y, w = make_inputs(1500, 264, 5000, torch.bfloat16, seed=31, ignore_frac=0.4, device="cuda")
     out_a, dx_a, dw_a = _fb(x, y, w, z_reg=1e-3, n_chunk=64)
     xg = x.clone()
@@ -59,7 +62,10 @@ def test_results_do_not_depend_on_where_the_ignored_tokens_sit(keep_every):
     batch must give the loss, dW and dx rows of the dense batch made of those tokens alone."""
     from oracle import lce_forward_backward_fp64
 
+    from linear_cross_entropy_loss_amd import _lib, ops
+
     print(f"packed rows keep_every={keep_every}", flush=True)
+    ops.PACK_ROWS = _lib.PACK_ALWAYS  # (the fixture restores it)
     N, H, V = 3000, 136, 3003
     x, y, w = make_inputs(N, H, V, torch.float16, seed=40 + keep_every, ignore_frac=0.0, device="cuda")
     keep = torch.zeros(N, dtype=torch.bool, device="cuda")
@@ -85,7 +91,10 @@ def test_valid_count_is_exact_and_nonnegative_ignore_index_is_honoured():
     x, y, w = make_inputs(N, H, V, torch.float16, seed=22, ignore_frac=0.0, device="cuda")
     y[::3] = 7  # ignore_index = 7 is a legal column: those rows are ignored, never matched
     lib = _lib.load()
-    p = _lib.make_problem(N, H, V, H, V, H, V, x.dtype, w.dtype, x.dtype, w.dtype, 7, 1.0, 0.0, 512, False)
+    from linear_cross_entropy_loss_amd import ops
+
+    p = _lib.make_problem(N, H, V, H, V, H, V, x.dtype, w.dtype, x.dtype, w.dtype, 7, 1.0, 0.0, 512, False, 0,
+                          ops.PACK_ROWS)
     fwd_b, _ = _lib.workspace_bytes(p)
     ws = torch.empty(fwd_b, dtype=torch.uint8, device="cuda")
     lse = torch.empty(N, device="cuda")
@@ -101,10 +110,13 @@ def test_valid_count_is_exact_and_nonnegative_ignore_index_is_honoured():
 
     ref = lce_forward_fp64(x.cpu().double(), y.cpu(), w.cpu().double(), 7, 0.0, 1.0)
     assert abs(out5[0].item() - ref.loss.item()) <= 1e-3 * abs(ref.loss.item())
-    # rows with the ignored label are not computed at all (monitoring off): their lse is 0
     keep = (y != 7).cpu()
     assert torch.allclose(lse.cpu().double()[keep], ref.lse[keep], rtol=2e-4, atol=2e-4)
-    assert bool((lse.cpu()[~keep] == 0).all())
+    if ops.PACK_ROWS == _lib.PACK_ALWAYS:
+        # rows with the ignored label are not computed at all (monitoring off): their lse is 0
+        assert bool((lse.cpu()[~keep] == 0).all())
+    else:
+        assert torch.allclose(lse.cpu().double(), ref.lse, rtol=2e-4, atol=2e-4)
     _, dx, _ = _fb(x, y, w, ignore_index=7)
     assert (dx[y == 7] == 0).all()
 
