@@ -90,7 +90,7 @@ typedef struct lce_problem {
  * gradient (ops.py:213, 314, 422).  With packing the kept rows are gathered to
  * the front on the device and the tile kernels run on them only, so time
  * scales with the number of labelled tokens; the pre-pass costs a few small
- * launches (about 0.07 ms per forward + backward), which a small problem does
+ * launches (about 0.04 ms per forward + backward), which a small problem does
  * not earn back.  LCE_PACK_AUTO packs when 8*N*H*V >= 2^41 FLOPs; results are
  * the same either way up to the summation order of dW and the loss, and lse of
  * an ignored row (see lce_forward).  Use the same value in lce_workspace_bytes,

@@ -30,7 +30,7 @@ fwd_configs: list = []
 bwd_configs: list = []
 
 # Whether tokens whose label is ignore_index are packed away on the device before the tile kernels run:
-# _lib.PACK_AUTO (the library decides by problem size: the pre-pass costs about 0.07 ms per step, which
+# _lib.PACK_AUTO (the library decides by problem size: the pre-pass costs about 0.04 ms per step, which
 # a small problem does not earn back), _lib.PACK_ALWAYS or _lib.PACK_NEVER.  Results do not depend on it
 # beyond the summation order of dW and of the loss.
 PACK_ROWS = _lib.PACK_AUTO
