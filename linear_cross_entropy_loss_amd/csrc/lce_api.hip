@@ -123,7 +123,8 @@ FwdPlan plan_fwd(const lce_problem* p) {
 struct BwdPlan {
   int64_t slabs, vs;
   PackPlan pack;
-  size_t lse_c, dxc;  // lse of the packed rows; packed dx before it is moved to its place
+  size_t lse_c, dxc;  // lse of the packed rows; packed dx before it is moved to its place (only for a dx of >= 2 GiB)
+  bool stage_dx;
   int64_t lddxc;
   size_t dz, dx_acc, dx_part, dw_part, w16, total;
 };
@@ -165,7 +166,11 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   b->lse_c = b->pack.end;
   b->dxc = b->lse_c + align_up((size_t)p->N * 4);
   size_t fixed = 0;  // (fp32 activations need the packed copy of x even when rows are not packed)
-  if (pack) fixed = b->dxc + align_up((size_t)p->N * (size_t)b->lddxc * (p->dx_dtype == LCE_F32 ? 4 : 2));
+  // The dx kernels store packed rows straight to their tokens' places through 32-bit offsets into dx; a dx
+  // that large offsets cannot span is staged packed and moved afterwards.
+  const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
+  b->stage_dx = pack && (size_t)p->N * (size_t)p->lddx * dxes >= ((size_t)1 << 31);
+  if (pack) fixed = b->dxc + (b->stage_dx ? align_up((size_t)p->N * (size_t)b->lddxc * dxes) : 0);
   else if (p->x_dtype == LCE_F32) fixed = b->pack.end;
   for (int pass = 0; pass < 2; ++pass) {
     const size_t budget = strict + (pass ? (size_t)p->N * (size_t)p->H * 4 : 0);
@@ -389,7 +394,8 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.ldxc = k.ldxc;
   if (pack) {
     a.n_rows = (const int64_t*)(base + k.n_rows);
-    a.dxc = base + b.dxc;
+    a.perm = (const int*)(base + k.perm);
+    a.dxc = b.stage_dx ? base + b.dxc : nullptr;
     a.lddxc = b.lddxc;
     a.y = (const int64_t*)(base + k.yc);
     a.lse = (const float*)(base + b.lse_c);
@@ -448,7 +454,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     }
   }
   if (pack && dx && (ph & LCE_PHASE_BWD_DX)) {
-    // packed dx rows go to their tokens, dropped tokens get exact zeros (nothing to do if none was dropped)
+    // dropped tokens get exact zeros, staged packed rows go to their tokens (nothing to do if none was dropped)
     hipError_t e = lce::launch_scatter_rows(a.dxc, b.lddxc * dxes, (const int*)(base + k.perm), a.n_rows, p->N, y,
                                             p->ignore_index, dx, p->lddx * dxes, p->H * dxes, a.num_cus, s);
     if (e != hipSuccess) return hip_fail(e, "scatter_rows");

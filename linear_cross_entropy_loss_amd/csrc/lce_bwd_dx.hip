@@ -17,12 +17,13 @@ namespace {
 // out-of-range offset (a quad that H cuts through is written whole: the row
 // stride is a multiple of 4, so it stays inside its row).  No branches: a branch
 // around accumulator reads makes the compiler read all of them up front.
-// `out` / `ldo` / `rows`: dx itself, or the packed copy when tokens were dropped (see BwdArgs).
+// `out` / `ldo` / `rows`: dx itself, or the packed copy when tokens were dropped (see BwdArgs).  `perm` != null
+// (packed rows, dx smaller than 2 GiB): the rows go straight to their tokens' places in dx instead.
 // `part` != null: this is a K segment of a tail tile; its raw fp32 sum goes to that 256 x 256 block and
 // nothing else happens.  Both uses run through the same statements (a different fp32 destination and
 // row stride), because two separate code paths behind a branch would each read the accumulator.
 template <class T>
-LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo, float* part,
+LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo, const int* perm, float* part,
                          f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   typedef typename elem_of<T>::type E;
   const int64_t h0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
@@ -32,10 +33,12 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo,
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
   const int es = a.dx_dtype == DT_F32 ? 4 : 2;
   // descriptor over the rows of this tile: base = first row, range = bytes to the end of dx
-  const char* tile_base = reinterpret_cast<const char*>(out) + t0 * ldo * es;
+  // (scattered rows: base = dx, all of it in range; rows that do not exist get an out-of-range offset below)
+  const char* tile_base = reinterpret_cast<const char*>(out) + (perm != nullptr ? 0 : t0 * ldo * es);
   // whole dwords: with 16-bit data and an odd H the last row ends one element into its stride padding
   const int64_t hcols = es == 2 ? (a.H + 1) & ~(int64_t)1 : a.H;
-  const int64_t left = (reinterpret_cast<const char*>(out) + ((rows - 1) * ldo + hcols) * es) - tile_base;
+  const int64_t last_row = perm != nullptr ? a.N : rows;
+  const int64_t left = (reinterpret_cast<const char*>(out) + ((last_row - 1) * ldo + hcols) * es) - tile_base;
   const unsigned range = left <= 0 ? 0u : (left > 0x7fffffff ? 0x7fffffffu : (unsigned)left);
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(tile_base), 0, (int)range, 0x00020000);
   const bool tail = part != nullptr;
@@ -47,7 +50,8 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo,
   for (int qb = 0; qb < kNB; ++qb) {
     const int row = wq * kWaveTile + qb * kBlk + (lane & 31);  // row inside the tile
     const int64_t tok = t0 + row;
-    const unsigned row_off = (unsigned)(row * ldo * es);
+    unsigned row_off = (unsigned)(row * ldo * es);
+    if (perm != nullptr) row_off = tok < rows ? (unsigned)(packed_token(perm, tok, a.N) * ldo * es) : 0x80000000u;
 #pragma unroll
     for (int pb = 0; pb < kNB; ++pb)
 #pragma unroll
@@ -61,7 +65,7 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo,
         if (to_f32) {
           *reinterpret_cast<f32x4_t*>(f32dst + tok * f32ld + h) = v;
         } else {
-          const unsigned off = h < a.H ? row_off + (unsigned)(h * es) : 0x80000000u;
+          const unsigned off = (h < a.H && row_off != 0x80000000u) ? row_off + (unsigned)(h * es) : 0x80000000u;
           if (a.dx_dtype == DT_F32) {
             const f32x4_t o = v * coef;
             u32x4_t bits;
@@ -156,9 +160,10 @@ template <class T, bool KMASK> struct DxProblem {
   LCE_DEV void epilogue(int item, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq, seg;
     decode(item, tp, tq, seg);
-    const bool packed = rows != a.N;
+    const bool packed = rows != a.N, copy = packed && a.dxc != nullptr;
     float* part = seg >= 0 ? a.dx_part + (int64_t)(item - plan.full) * kTile * kTile : nullptr;
-    dx_epilogue<T>(a, rows, packed ? a.dxc : a.dx, packed ? a.lddxc : a.lddx, part, acc, tp, tq);
+    dx_epilogue<T>(a, rows, copy ? a.dxc : a.dx, copy ? a.lddxc : a.lddx, packed && !copy ? a.perm : nullptr, part, acc,
+                   tp, tq);
   }
 };
 
@@ -184,9 +189,10 @@ __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
   if (b >= plan.tail_tiles) return;
   int tp, tq;
   tile_coords(plan.full + b, plan.tiles, tiles_p, tiles_q, 8, tp, tq);
-  const bool packed = rows != a.N;
-  void* out = packed ? a.dxc : a.dx;
-  const int64_t ldo = packed ? a.lddxc : a.lddx;
+  const bool packed = rows != a.N, copy = packed && a.dxc != nullptr;
+  void* out = copy ? a.dxc : a.dx;
+  const int64_t ldo = copy ? a.lddxc : a.lddx;
+  const int* perm = packed && !copy ? a.perm : nullptr;
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
   const float* part = a.dx_part + (int64_t)b * plan.nseg * kTile * kTile;
   constexpr int kQuads = kTile * kTile / 4 / kTailParts;  // quads of this workgroup: 16 rows of the tile
@@ -202,13 +208,16 @@ __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
     if (!a.first) v += *reinterpret_cast<const f32x4_t*>(a.dx_acc + o);
     if (!a.last) {
       *reinterpret_cast<f32x4_t*>(a.dx_acc + o) = v;
-    } else if (a.dx_dtype == DT_F32) {
-      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + tok * ldo + h) = v * coef;
     } else {
-      u32x2_t b;
-      b[0] = pack2<T>(v[0] * coef, v[1] * coef);
-      b[1] = pack2<T>(v[2] * coef, v[3] * coef);
-      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(out) + tok * ldo + h) = b;
+      const int64_t dst_row = perm != nullptr ? packed_token(perm, tok, a.N) : tok;
+      if (a.dx_dtype == DT_F32) {
+        *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + dst_row * ldo + h) = v * coef;
+      } else {
+        u32x2_t b;
+        b[0] = pack2<T>(v[0] * coef, v[1] * coef);
+        b[1] = pack2<T>(v[2] * coef, v[3] * coef);
+        *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(out) + dst_row * ldo + h) = b;
+      }
     }
   }
 }

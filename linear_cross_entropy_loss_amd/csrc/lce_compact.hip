@@ -8,7 +8,7 @@
 //
 //   compact_labels  perm[j] = original index of the j-th kept token, yc[j] its label, n_rows = how many
 //   gather_rows     xc[j] = x[perm[j]], lse_c[j] = lse[perm[j]]
-//   scatter_rows    dx[perm[j]] = dxc[j]; rows of dropped tokens = 0
+//   scatter_rows    rows of dropped tokens of dx = 0 (and dx[perm[j]] = dxc[j] where dx was staged packed)
 //
 // When no token is dropped (n_rows == N) the row copies are skipped and the
 // tile kernels read x and write dx in place.
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(const char* dxc, int6
   const int64_t rows = packed_rows(n_rows, N);
   if (rows == N) return;  // nothing was dropped: the tile kernel wrote dx itself
   for (int64_t i = blockIdx.x; i < N; i += gridDim.x) {
-    if (i < rows) {
+    if (dxc != nullptr && i < rows) {
       const u32x2_t* s = reinterpret_cast<const u32x2_t*>(dxc + i * lddxc_bytes);
       u32x2_t* d = reinterpret_cast<u32x2_t*>(dx + packed_token(perm, i, N) * lddx_bytes);
       for (int c = threadIdx.x; c < chunks; c += 256) d[c] = s[c];

@@ -91,10 +91,12 @@ struct BwdArgs {
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
   // Packed rows (tokens with an ignored label dropped; n_rows == null: the call works on all rows).
-  // *n_rows (device) rows are worked on.  When *n_rows != N they are the rows of xc (row stride ldxc), dx
-  // goes to dxc (row stride lddxc, moved to its place afterwards), and in either case `y` and `lse` hold
-  // the labels / lse of the packed rows.
+  // *n_rows (device) rows are worked on.  When *n_rows != N they are the rows of xc (row stride ldxc) and
+  // row j of dx belongs to token perm[j]: the dx kernels store it there themselves, or -- dxc != null, a dx
+  // of 2 GiB or more -- into dxc (row stride lddxc), from where it is moved afterwards.  In either case `y`
+  // and `lse` hold the labels / lse of the packed rows.
   const int64_t* n_rows;
+  const int* perm;
   const void* xc;
   int64_t ldxc;
   void* dxc;
@@ -139,8 +141,8 @@ hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, const int* perm,
 hipError_t launch_gather_rows_f32(const float* x, int64_t ldx, int64_t H, const int* perm, const int64_t* n_rows,
                                   int64_t N, void* xc, int64_t ldxc, const float* lse, float* lse_c, int num_cus,
                                   hipStream_t s);
-// dx[perm[j]] = dxc[j] for j < *n_rows and dx[i] = 0 for every token i with y[i] == ignore_index, in 8-byte
-// pieces covering row_bytes; nothing when *n_rows == N.
+// dx[perm[j]] = dxc[j] for j < *n_rows (skipped when dxc is null) and dx[i] = 0 for every token i with
+// y[i] == ignore_index, in 8-byte pieces covering row_bytes; nothing when *n_rows == N.
 hipError_t launch_scatter_rows(const void* dxc, int64_t lddxc_bytes, const int* perm, const int64_t* n_rows,
                                int64_t N, const int64_t* y, int64_t ignore_index, void* dx, int64_t lddx_bytes,
                                int64_t row_bytes, int num_cus, hipStream_t s);

@@ -112,12 +112,15 @@ def test_backward_scratch_within_n_chunk_bound(N, H, V, n_chunk):
 
 def _pack_bytes(N, H, es_x=2, es_dx=2, backward=True):
     """Scratch of the packed rows (tokens with an ignored label dropped): segment counts, the row count, the
-    row -> token map, packed labels and the packed copy of x; for the backward also the packed lse and dx."""
+    row -> token map, packed labels and the packed copy of x; for the backward also the packed lse and -- only
+    for a dx of 2 GiB or more, which 32-bit store offsets cannot span -- a packed staging copy of dx."""
     al = lambda v: -(-v // 256) * 256
     pad = lambda v, m: -(-v // m) * m
     b = al(-(-N // 2048) * 4) + 256 + al(4 * N) + al(8 * N) + al(N * pad(H, 16 // es_x) * es_x)
     if backward:
-        b += al(4 * N) + al(N * pad(H, 8) * es_dx)
+        b += al(4 * N)
+        if N * H * es_dx >= 1 << 31:   # (the tests use lddx = H)
+            b += al(N * pad(H, 8) * es_dx)
     return b
 
 

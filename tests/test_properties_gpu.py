@@ -83,6 +83,34 @@ def test_results_do_not_depend_on_where_the_ignored_tokens_sit(keep_every):
     assert max(rel_errors(dx, ref.dx)) <= 2e-2 and max(rel_errors(dw, ref.dw)) <= 2e-2
 
 
+def test_dx_of_2_gib_is_staged_packed_and_moved(pack_mode):
+    """Packed dx rows normally go straight to their tokens through 32-bit store offsets; a dx of 2 GiB or
+    more is staged packed and moved by a copy kernel.  Same rows through the same kernels either way."""
+    from linear_cross_entropy_loss_amd import _lib, ops
+
+    if pack_mode != "pack":
+        pytest.skip("one run is enough")
+    print("staged dx", flush=True)
+    N, H, V = 131072, 8192, 512
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(N, H, device="cuda", dtype=torch.bfloat16, generator=g)
+    w = (torch.randn(H, V, device="cuda", generator=g) / math.sqrt(H)).to(torch.bfloat16)
+    y = torch.randint(0, V, (N,), device="cuda", generator=g)
+    y[torch.rand(N, device="cuda", generator=g) < 0.3] = -1
+    res = {}
+    for mode in (_lib.PACK_ALWAYS, _lib.PACK_NEVER):
+        ops.PACK_ROWS = mode
+        out, dx, dw = _fb(x, y, w, n_chunk=65536)
+        res[mode] = (out[0].item(), dx, dw)
+        del out
+    a, b = res[_lib.PACK_ALWAYS], res[_lib.PACK_NEVER]
+    assert abs(a[0] - b[0]) <= 1e-6 * abs(b[0])
+    assert torch.equal(a[1], b[1])          # dx rows do not depend on which other rows share their tile
+    assert (a[1][y == -1] == 0).all()
+    e_max, e_l2 = rel_errors(a[2], b[2])         # dW: another summation order over the tokens, then bf16 rounding
+    assert e_max <= 1e-2 and e_l2 <= 1e-3
+
+
 def test_valid_count_is_exact_and_nonnegative_ignore_index_is_honoured():
     from linear_cross_entropy_loss_amd import _lib
 
