@@ -1,10 +1,12 @@
 // Backward, step 3: dW[h][v] = coef * sum_token x[token][h] * dz[token][v] for
 // the columns of one vocabulary slab (the contraction of
 // linear_cross_entropy/ops.py:424).  K = token, so both operands are read
-// through the LDS transpose path.  Each workgroup owns its dW tile over ALL
-// tokens: the fp32 accumulator never leaves registers, no cross-workgroup
-// reduction exists, and the result is written once in the output dtype after
-// scaling by grad_out * logit_scale / n_valid (ops.py:443-447, 810).
+// through the LDS transpose path.  A workgroup owns its dW tile over ALL tokens
+// (the rows that are left after tokens with an ignored label were packed away):
+// the fp32 accumulator never leaves registers and the result is written once
+// in the output dtype after scaling by grad_out * logit_scale / n_valid
+// (ops.py:443-447, 810).  Only the tiles of a mostly idle last round of
+// workgroups are cut along K instead and summed by a second kernel (DwPlan).
 #include "lce_gemm3.h"
 #include "lce_internal.h"
 

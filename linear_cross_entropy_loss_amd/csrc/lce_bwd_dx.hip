@@ -3,6 +3,9 @@
 // operands are K-contiguous (K = v).  The running sum over slabs is kept in
 // fp32; the factor grad_out * logit_scale / n_valid is applied once, after the
 // last slab, as the reference does after its accumulation (ops.py:332, 810).
+// The token rows are those left after tokens with an ignored label were packed
+// away; the tiles of a mostly idle last round of workgroups are cut along K
+// and summed by a second kernel (DxPlan).
 #include "lce_gemm3.h"
 #include "lce_internal.h"
 
