@@ -219,7 +219,7 @@ int current_num_cus(int* out) {
 
 extern "C" {
 
-int lce_version(void) { return 100; }
+int lce_version(void) { return 200; }  // 0.2.0: lce_problem gained pack_rows
 
 const char* lce_strerror(int status) {
   switch (status) {
