@@ -100,8 +100,9 @@ def time_phases(cfg, x, y, w, torch, reps=5):
     fwd(0)
     bwd(0)
     torch.cuda.synchronize()
-    # tokens with an ignored label are dropped before the tile kernels: FLOPs are counted on the others only
-    rows = int(nv.item())
+    # tokens with an ignored label are dropped before the tile kernels (from 8*N*H*V = 2^41 FLOPs on, the
+    # library's default rule): FLOPs are counted on the others only
+    rows = int(nv.item()) if 8.0 * N * H * V >= 2.0 ** 41 else N
     # launches per call: the backward runs once per vocabulary slab
     slabs, _ = _lib.backward_plan(prob(0))
     out = {}
@@ -248,7 +249,7 @@ def main():
     out_bytes = x.numel() * x.element_size() + w.numel() * w.element_size()
     # Tokens whose label is ignored are dropped before the tile kernels (their rows of the four GEMMs are
     # not computed), so the rate counts the computed rows only; with monitoring on the forward keeps all rows.
-    rows = int((y != -1).sum().item())
+    rows = int((y != -1).sum().item()) if 8.0 * N * H * V >= 2.0 ** 41 else N
     flops = (2.0 * (N if cfg["monitoring"] else rows) + 6.0 * rows) * H * V
     tflops = flops / ms / 1e9
     peak = PEAK_TFLOPS[cfg["dtype"]]
