@@ -209,6 +209,8 @@ template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s)
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (dw_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // this launch cannot have a split tail
+  // (the tile count does not depend on the rows: no second kernel when the last round is not split)
+  if (!has_split_tail((a.vs / kTile) * (a.Hp / kTile), a.dw_grid)) return hipSuccess;
   // at most dw_grid / 2 tail tiles can be split (two segments each)
   const unsigned tail_most = (unsigned)(a.dw_grid / 2 > 0 ? a.dw_grid / 2 : 1);
   hipLaunchKernelGGL(dw_tail_kernel<T>, dim3(tail_most * kTailParts), dim3(256), 0, s, a);

@@ -240,6 +240,8 @@ template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s)
   hipError_t e = exact_k ? launch_tiles<T, false>(a, s) : launch_tiles<T, true>(a, s);
   if (e != hipSuccess) return e;
   if (dx_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // no shape of this launch can have a split tail
+  // without packed rows the tile count is known here: no second kernel when its last round is not split
+  if (a.n_rows == nullptr && !has_split_tail((a.Np / kTile) * (a.Hp / kTile), a.dx_grid)) return hipSuccess;
   // at most dx_grid / 2 tail tiles can be split (two segments each)
   const unsigned tail_most = (unsigned)(a.dx_grid / 2 > 0 ? a.dx_grid / 2 : 1);
   hipLaunchKernelGGL(dx_tail_kernel<T>, dim3(tail_most * kTailParts), dim3(256), 0, s, a);

@@ -162,6 +162,11 @@ inline int64_t dx_tail_blocks(int64_t Np, int64_t Hp, int64_t vs) {
   const int64_t most = (Np / 256) * (Hp / 256) * s;
   return most < kTailBlocks ? most : kTailBlocks;
 }
+// Whether T output tiles on G workgroups end in a last round that the kernels cut along K (at most half full).
+inline bool has_split_tail(int64_t T, int64_t G) {
+  const int64_t r = T % G, cap = G < kTailBlocks ? G : kTailBlocks;
+  return r > 0 && r * 2 <= cap;
+}
 // true if every split the dx kernel may choose cuts the K tiles of a slab into equal, even segments
 inline bool dx_segments_exact(int64_t vs) { return (vs / 64) % (2 * max_k_segments(vs / 64)) == 0; }
 // dW of one slab: (vs/256) x (Hp/256) tiles, K = at most Np tokens.  The same bound for the dW kernel, whose
