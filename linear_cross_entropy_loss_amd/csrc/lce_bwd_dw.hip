@@ -134,7 +134,7 @@ template <class T> struct DwProblem {
       tile = plan.full + j / plan.nseg;
       seg = j % plan.nseg;
     }
-    tile_coords(tile, plan.tiles, tiles_p, tiles_q, 4, tp, tq);
+    tile_coords(tile, plan.tiles, tiles_p, tiles_q, 8, tp, tq);
   }
   LCE_DEV int item_ktiles(int item) const { return item < plan.full ? plan.kt : plan.kseg; }
   LCE_DEV void origins(int item, const void*& p, const void*& q) const {
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(256) void dw_tail_kernel(const BwdArgs a) {
   const int b = (int)blockIdx.x / kTailParts, piece = (int)blockIdx.x % kTailParts;
   if (b >= plan.tail_tiles) return;
   int tp, tq;
-  tile_coords(plan.full + b, plan.tiles, (int)(a.vs / kTile), (int)(a.Hp / kTile), 4, tp, tq);
+  tile_coords(plan.full + b, plan.tiles, (int)(a.vs / kTile), (int)(a.Hp / kTile), 8, tp, tq);
   const float coef = a.grad_out[0] * a.scale / (float)a.n_valid[0];
   const float* part = a.dw_part + (int64_t)b * plan.nseg * kTile * kTile;
   constexpr int kQuads = kTile * kTile / 4 / kTailParts;
