@@ -55,7 +55,8 @@ typedef enum lce_status {
   LCE_EINVAL_DTYPE = -2, /* unsupported dtype combination                            */
   LCE_EINVAL_ARG = -3,   /* null pointer, bad stride, bad scalar                     */
   LCE_EWORKSPACE = -4,   /* workspace missing or smaller than lce_workspace_bytes    */
-  LCE_EHIP = -5          /* a HIP launch failed; see lce_last_hip_error              */
+  LCE_EHIP = -5,         /* a HIP launch failed; see lce_last_hip_error              */
+  LCE_ESTATIC = -6       /* lce_forward_static: problem needs more than LCE_STATIC_SCRATCH_BYTES */
 } lce_status;
 
 /*
@@ -167,6 +168,29 @@ int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width)
 int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_t* y,
                 float* lse, float* out5, int64_t* n_valid,
                 void* ws, size_t ws_bytes, void* stream);
+
+/*
+ * Forward without a workspace argument, for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference (every buffer there
+ * is a torch allocation, ops.py:693-703).  Same inputs, outputs and results
+ * (bit for bit) as lce_forward; the scratch is a fixed array of
+ * LCE_STATIC_SCRATCH_BYTES in device memory that every GPU the library runs on
+ * holds until the process ends.  The call allocates and frees nothing.
+ *
+ *   - A problem whose lce_workspace_bytes forward size exceeds
+ *     LCE_STATIC_SCRATCH_BYTES is refused with LCE_ESTATIC (e.g. N = 4096 rows
+ *     at V = 131072, H = 2048 fits; N = 16384 does not): use lce_forward.
+ *   - All calls on one GPU share that GPU's array: calls that overlap in time
+ *     on one GPU (two streams, two threads) race.  Calls on one stream, or
+ *     otherwise ordered, are fine; nothing is carried from one call to the next.
+ *   - The first call on a device looks the array's address up
+ *     (hipGetSymbolAddress, which may load the code object): make one call
+ *     outside any graph capture before capturing.
+ */
+#define LCE_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int lce_forward_static(const lce_problem* p, const void* x, const void* w, const int64_t* y,
+                       float* lse, float* out5, int64_t* n_valid, void* stream);
 
 /*
  * Backward.  Replaces linear_xent_bwd_dispatcher and its dx / dA programs

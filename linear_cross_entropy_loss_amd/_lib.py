@@ -13,7 +13,8 @@ LCE_BF16, LCE_F16, LCE_F32 = 0, 1, 2
 LCE_OK = 0
 PHASE_FWD_TILES, PHASE_FWD_REDUCE, PHASE_BWD_DZ, PHASE_BWD_DX, PHASE_BWD_DW, PHASE_PACK = 1, 2, 4, 8, 16, 32
 PACK_AUTO, PACK_ALWAYS, PACK_NEVER = 0, 1, 2
-LCE_EINVAL_SHAPE, LCE_EINVAL_DTYPE, LCE_EINVAL_ARG, LCE_EWORKSPACE, LCE_EHIP = -1, -2, -3, -4, -5
+LCE_EINVAL_SHAPE, LCE_EINVAL_DTYPE, LCE_EINVAL_ARG, LCE_EWORKSPACE, LCE_EHIP, LCE_ESTATIC = -1, -2, -3, -4, -5, -6
+STATIC_SCRATCH_BYTES = 64 << 20
 
 EXPORTS = (
     "lce_version",
@@ -23,6 +24,7 @@ EXPORTS = (
     "lce_workspace_bytes",
     "lce_backward_plan",
     "lce_forward",
+    "lce_forward_static",
     "lce_backward",
 )
 
@@ -86,6 +88,8 @@ def load():
     lib.lce_backward_plan.argtypes = [P, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]
     lib.lce_forward.restype = ctypes.c_int
     lib.lce_forward.argtypes = [P, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+    lib.lce_forward_static.restype = ctypes.c_int
+    lib.lce_forward_static.argtypes = [P, vp, vp, vp, vp, vp, vp, vp]
     lib.lce_backward.restype = ctypes.c_int
     lib.lce_backward.argtypes = [P, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
     _lib = lib

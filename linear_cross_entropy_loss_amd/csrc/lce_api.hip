@@ -4,6 +4,7 @@
 // (linear_cross_entropy/ops.py:681-802) -- minus every allocation, which is the
 // caller's -- and what its backward does (ops.py:804-810).
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdio.h>
 #include <string.h>
 
@@ -205,6 +206,30 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
 
 bool misaligned(const void* p) { return ((uintptr_t)p & 15) != 0; }
 
+// Scratch of lce_forward_static: a fixed array in device memory, one copy per GPU the library runs on,
+// held until the process ends.  On the host `scratch` is only a handle for hipGetSymbolAddress; the
+// device address is looked up once per device and kept in g_scratch_ptr.
+constexpr size_t kStaticScratchBytes = LCE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return LCE_EINVAL_ARG;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread finds the same address
+  }
+  *out = ptr;
+  return LCE_OK;
+}
+
 // Compute units of the current device (grid size of the persistent kernels).
 int current_num_cus(int* out) {
   int dev = 0, n = 0;
@@ -215,60 +240,9 @@ int current_num_cus(int* out) {
   return LCE_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-int lce_version(void) { return 200; }  // 0.2.0: lce_problem gained pack_rows
-
-const char* lce_strerror(int status) {
-  switch (status) {
-    case LCE_OK: return "ok";
-    case LCE_EINVAL_SHAPE:
-      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N, V <= 2^30, H <= 2^20; "
-             "ceil(N/256) * ceil(V/256) <= 2^28)";
-    case LCE_EINVAL_DTYPE:
-      return "unsupported dtype combination (x: bf16/f16/f32; w: x dtype or f32; grads: same dtype or f32)";
-    case LCE_EINVAL_ARG:
-      return "invalid argument (null or misaligned pointer; row strides must be >= the row length and multiples of 8 "
-             "elements for 16-bit data, 4 for fp32, and at most 8 MiB for x, a 16-bit w and dx; logit_scale <= 0 or "
-             "z_reg < 0)";
-    case LCE_EWORKSPACE: return "workspace missing or too small for this problem and N_chunk_size";
-    case LCE_EHIP: return "HIP error";
-    default: return "unknown status";
-  }
-}
-
-const char* lce_last_hip_error(void) { return g_hip_error; }
-
-int lce_check_problem(const lce_problem* p) { return check(p, true); }
-
-int lce_workspace_bytes(const lce_problem* p, size_t* fwd_bytes, size_t* bwd_bytes) {
-  int rc = check(p, false);
-  if (rc != LCE_OK) return rc;
-  if (fwd_bytes) *fwd_bytes = plan_fwd(p).total;
-  if (bwd_bytes) {
-    BwdPlan b;
-    rc = plan_bwd(p, &b);
-    if (rc != LCE_OK) return rc;
-    *bwd_bytes = b.total;
-  }
-  return LCE_OK;
-}
-
-int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width) {
-  int rc = check(p, false);
-  if (rc != LCE_OK) return rc;
-  BwdPlan b;
-  rc = plan_bwd(p, &b);
-  if (rc != LCE_OK) return rc;
-  if (slabs) *slabs = b.slabs;
-  if (slab_width) *slab_width = b.vs;
-  return LCE_OK;
-}
-
-int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_t* y, float* lse,
-                float* out5, int64_t* n_valid, void* ws, size_t ws_bytes, void* stream) {
+// Body of lce_forward; `ws` is the caller's workspace or the library's static scratch.
+int forward_impl(const lce_problem* p, const void* x, const void* w, const int64_t* y, float* lse, float* out5,
+                 int64_t* n_valid, void* ws, size_t ws_bytes, void* stream) {
   int rc = check(p, false);
   if (rc != LCE_OK) return rc;
   if (!x || !w || !y || !lse || !out5 || !n_valid) return LCE_EINVAL_ARG;
@@ -351,6 +325,79 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
     if (e != hipSuccess) return hip_fail(e, "fwd_reduce");
   }
   return LCE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lce_version(void) { return 200; }  // 0.2.0: lce_problem gained pack_rows
+
+const char* lce_strerror(int status) {
+  switch (status) {
+    case LCE_OK: return "ok";
+    case LCE_EINVAL_SHAPE:
+      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N, V <= 2^30, H <= 2^20; "
+             "ceil(N/256) * ceil(V/256) <= 2^28)";
+    case LCE_EINVAL_DTYPE:
+      return "unsupported dtype combination (x: bf16/f16/f32; w: x dtype or f32; grads: same dtype or f32)";
+    case LCE_EINVAL_ARG:
+      return "invalid argument (null or misaligned pointer; row strides must be >= the row length and multiples of 8 "
+             "elements for 16-bit data, 4 for fp32, and at most 8 MiB for x, a 16-bit w and dx; logit_scale <= 0 or "
+             "z_reg < 0)";
+    case LCE_EWORKSPACE: return "workspace missing or too small for this problem and N_chunk_size";
+    case LCE_EHIP: return "HIP error";
+    case LCE_ESTATIC:
+      return "problem needs more forward scratch than the library's static buffer (LCE_STATIC_SCRATCH_BYTES = 64 MiB); "
+             "call lce_forward with a workspace instead";
+    default: return "unknown status";
+  }
+}
+
+const char* lce_last_hip_error(void) { return g_hip_error; }
+
+int lce_check_problem(const lce_problem* p) { return check(p, true); }
+
+int lce_workspace_bytes(const lce_problem* p, size_t* fwd_bytes, size_t* bwd_bytes) {
+  int rc = check(p, false);
+  if (rc != LCE_OK) return rc;
+  if (fwd_bytes) *fwd_bytes = plan_fwd(p).total;
+  if (bwd_bytes) {
+    BwdPlan b;
+    rc = plan_bwd(p, &b);
+    if (rc != LCE_OK) return rc;
+    *bwd_bytes = b.total;
+  }
+  return LCE_OK;
+}
+
+int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width) {
+  int rc = check(p, false);
+  if (rc != LCE_OK) return rc;
+  BwdPlan b;
+  rc = plan_bwd(p, &b);
+  if (rc != LCE_OK) return rc;
+  if (slabs) *slabs = b.slabs;
+  if (slab_width) *slab_width = b.vs;
+  return LCE_OK;
+}
+
+int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_t* y, float* lse,
+                float* out5, int64_t* n_valid, void* ws, size_t ws_bytes, void* stream) {
+  return forward_impl(p, x, w, y, lse, out5, n_valid, ws, ws_bytes, stream);
+}
+
+int lce_forward_static(const lce_problem* p, const void* x, const void* w, const int64_t* y, float* lse,
+                       float* out5, int64_t* n_valid, void* stream) {
+  int rc = check(p, false);
+  if (rc != LCE_OK) return rc;
+  if (plan_fwd(p).total > kStaticScratchBytes) return LCE_ESTATIC;  // before any device call
+  void* ptr = nullptr;
+  rc = static_scratch(&ptr);
+  if (rc != LCE_OK) return rc;
+  // Nothing in the forward scratch has to start at zero: every cell a kernel reads was written by an
+  // earlier kernel of the same call, so the contents the previous call left behind are never looked at.
+  return forward_impl(p, x, w, y, lse, out5, n_valid, ptr, kStaticScratchBytes, stream);
 }
 
 int lce_backward(const lce_problem* p, const void* x, const void* w, const int64_t* y,
