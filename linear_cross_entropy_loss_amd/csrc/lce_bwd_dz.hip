@@ -2,6 +2,7 @@
 // MFMA main loop as the forward (so the logits are bit-identical to the ones
 // the saved lse was built from) and turn it, in registers, into
 //     dz = softmax * (1 + 2*z_reg*lse) - onehot(y),   0 for ignored tokens
+// (times 2^dz_shift, a power of two that keeps small probabilities in fp16's normal range)
 // (linear_cross_entropy/ops.py:309-314 and 415-422), rounded once to the
 // 16-bit compute type exactly where the reference casts dz before its dot
 // products (ops.py:314, 422).  The tile is transposed through LDS and written
@@ -73,7 +74,8 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
     const int64_t rel = yy - slice_v0;
     const bool valid = yy != a.ignore_index;
     const float l = exists ? a.lse[tok] : 0.f;
-    nlse[qb] = valid ? -l * kLog2e : -INFINITY;
+    // (the power-of-two factor of the staged dz rides along in the exponent)
+    nlse[qb] = valid ? fmaf(-l, kLog2e, (float)dz_shift<T>::value) : -INFINITY;
     gain[qb] = 1.f + 2.f * a.z_reg * l;
     // target column inside this wave's slice, only in the lane half that holds it
     ykey[qb] = (valid && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == half) ? (int)rel : -1;
@@ -140,7 +142,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
             if (want == pp * 16 + r) zt = acc[2 * ph + pp][qb][r];
         float p = __builtin_amdgcn_exp2f(fmaf(zt, c1, nlse[qb]));
         if (ZREG) p *= gain[qb];
-        *reinterpret_cast<unsigned short*>(lrow + (((yl >> 3) ^ sw) << 4) + (yl & 7) * 2) = to_bits<T>(p - 1.f);
+        *reinterpret_cast<unsigned short*>(lrow + (((yl >> 3) ^ sw) << 4) + (yl & 7) * 2) = to_bits<T>(p - dz_scale<T>());
       }
       // keep the register footprint small: an operand tile is in flight across this function
       __builtin_amdgcn_sched_barrier(0);

@@ -10,6 +10,8 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    config.addinivalue_line("markers", "pack_auto: run once, with the library's own choice of packing ignored tokens "
+                                       "(full-size cases, where that choice is to pack)")
 
 
 def pytest_sessionstart(session):
@@ -36,6 +38,8 @@ def pytest_collection_modifyitems(config, items):
 def pytest_generate_tests(metafunc):
     # GPU tests run twice: with the tokens of ignored labels packed away before the tile kernels, and
     # without (by default the library chooses by problem size, which would leave small test shapes unpacked)
+    if metafunc.definition.get_closest_marker("pack_auto") is not None:
+        return
     if metafunc.definition.get_closest_marker("gpu") is not None and "pack_mode" in metafunc.fixturenames:
         metafunc.parametrize("pack_mode", ["pack", "nopack"], indirect=True)
 
