@@ -55,10 +55,14 @@ int check(const lce_problem* p, bool backward) {
 
 // Buffers of the packing pre-pass (tokens with an ignored label dropped), relative to `base`.
 struct PackPlan {
-  size_t cnt, n_rows, perm, yc, xc, end;
+  size_t cnt, n_rows, perm, yc, xc, xk, end;
   int64_t ldxc;  // row stride of the packed copy of x, elements: rows of whole 16-byte pieces
-  size_t xes;    // element size of the packed copy: that of x, or 2 for fp32 activations (stored rounded to bf16)
+  int64_t ldxk;  // fp32 activations, backward: row stride of the copy stacked along the tokens (lce_compact.hip)
+  size_t xes;    // element size of the packed copy: that of x, or 2 for fp32 activations (stored as bf16 pairs)
 };
+
+// fp32 activations (and with them an fp32 weight) are computed as bf16 pairs, hi + lo (lce_gemm.h).
+bool splits(const lce_problem* p) { return p->x_dtype == LCE_F32; }
 
 // Whether the tokens with an ignored label are packed away before the tile kernels run (lce.h).
 bool packs_rows(const lce_problem* p) {
@@ -67,17 +71,20 @@ bool packs_rows(const lce_problem* p) {
   return 8.0 * (double)p->N * (double)p->H * (double)p->V >= 2199023255552.0;  // 2^41
 }
 
-PackPlan plan_pack(const lce_problem* p, size_t base) {
+PackPlan plan_pack(const lce_problem* p, size_t base, bool backward) {
   PackPlan k;
   const size_t N = (size_t)p->N, es = 2;
   k.xes = es;
-  k.ldxc = lce::pad_to(p->H, (int64_t)(16 / es));
+  k.ldxc = lce::pad_to(splits(p) ? 3 * p->H : p->H, (int64_t)(16 / es));
+  k.ldxk = lce::pad_to(p->H, (int64_t)(16 / es));
   size_t o = base;
   k.cnt = o; o += align_up((size_t)lce::compact_segments(p->N) * 4);
   k.n_rows = o; o += 256;
   k.perm = o; o += align_up(N * 4);
   k.yc = o; o += align_up(N * 8);
   k.xc = o; o += align_up(N * (size_t)k.ldxc * es);
+  k.xk = o;
+  if (splits(p) && backward) o += align_up(3 * (size_t)lce::padded_tokens(p->N) * (size_t)k.ldxk * es);
   k.end = o;
   return k;
 }
@@ -108,13 +115,14 @@ FwdPlan plan_fwd(const lce_problem* p) {
   f.vs = (int64_t)Vp;
   if (p->w_dtype == LCE_F32) {
     // slab copies of at most 256 MiB (at least one tile column)
-    int64_t cols = ((int64_t)256 << 20) / (p->H * 2) / 256 * 256;
+    const int64_t hw = splits(p) ? 3 * p->H : p->H;  // rows of the copy
+    int64_t cols = ((int64_t)256 << 20) / (hw * 2) / 256 * 256;
     if (cols < 256) cols = 256;
     if (cols < f.vs) f.vs = cols;
-    o += align_up((size_t)p->H * (size_t)f.vs * 2);
+    o += align_up((size_t)hw * (size_t)f.vs * 2);
   }
   if ((!p->monitoring && packs_rows(p)) || p->x_dtype == LCE_F32) {
-    f.pack = plan_pack(p, o);
+    f.pack = plan_pack(p, o, false);
     o = f.pack.end;
   }
   f.total = o;
@@ -162,7 +170,8 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   const int64_t cols = Vp / 256;
   // buffers of the packed rows come first and count towards the bound
   const bool pack = packs_rows(p);
-  b->pack = plan_pack(p, 0);
+  b->pack = plan_pack(p, 0, true);
+  const bool split = splits(p);
   b->lddxc = lce::pad_to(p->H, 8);
   b->lse_c = b->pack.end;
   b->dxc = b->lse_c + align_up((size_t)p->N * 4);
@@ -179,12 +188,13 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
       const int64_t vs = (cols + s - 1) / s * 256;
       if (s > 1 && (cols + s - 2) / (s - 1) * 256 == vs) continue;  // same width as with one slab fewer
       const int64_t slabs = (Vp + vs - 1) / vs;
-      const size_t dz = align_up(Np * (size_t)vs * 2);
-      const size_t acc = slabs > 1 ? align_up(Np * Hp * 4) : 0;
+      // (bf16 pairs: three blocks of dz, and dx is summed over three passes per slab, so it always needs the running sum)
+      const size_t dz = align_up(Np * (size_t)vs * 2 * (split ? 3 : 1));
+      const size_t acc = slabs > 1 || split ? align_up(Np * Hp * 4) : 0;
       const int64_t last_vs = Vp - (slabs - 1) * vs;  // padded width of the last slab
-      const size_t dxp = dx_part_bytes(Np, Hp, vs, last_vs), dwp = dw_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
+      const size_t dxp = dx_part_bytes(Np, Hp, vs, last_vs), dwp = dw_part_bytes(split ? 3 * Np : Np, Hp, vs, last_vs);  // at most 64 MiB each
       const size_t part = dxp + dwp;
-      const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2) : 0;  // 16-bit copy of the slab of W
+      const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2 * (split ? 3 : 1)) : 0;  // 16-bit copy of the slab of W
       // the widened bound of the second pass is for the staging proper; the split-K partial sums
       // (at most 64 MiB each for dx and dW) and the packed rows come on top of it there
       const size_t counted = dz + acc + w16 + (pass == 0 ? fixed + part : 0);
@@ -290,16 +300,17 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
                                        (int*)(base + k.perm), (int64_t*)(base + k.yc), s);
         if (e != hipSuccess) return hip_fail(e, "compact_labels");
       }
-      e = x32 ? lce::launch_gather_rows_f32((const float*)x, p->ldx, p->H, a.perm, a.n_rows, p->N, base + k.xc, k.ldxc,
-                                            nullptr, nullptr, a.num_cus, s)
+      e = x32 ? lce::launch_gather_rows_split((const float*)x, p->ldx, p->H, a.perm, a.n_rows, p->N, base + k.xc,
+                                              k.ldxc, nullptr, 0, nullptr, nullptr, a.num_cus, s)
               : lce::launch_gather_rows(x, p->ldx * 2, a.perm, a.n_rows, p->N, base + k.xc, k.ldxc * 2, nullptr, nullptr,
                                         a.num_cus, s);
       if (e != hipSuccess) return hip_fail(e, "gather_rows");
     }
-    if (x32) {  // the tile kernels read the bf16 copy, whether or not rows were dropped
+    if (x32) {  // the tile kernels read the copy in bf16 pairs ([hi | hi | lo], K = 3 H), whether or not rows were dropped
       a.x = a.xc;
       a.ldx = a.ldxc;
       a.x_dtype = lce::DT_BF16;
+      a.H = 3 * p->H;
     }
   }
   if (ph & LCE_PHASE_FWD_TILES) {
@@ -310,7 +321,8 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
       a.vw = p->V - v0 < f.vs ? p->V - v0 : f.vs;
       if (p->w_dtype == LCE_F32) {
         const int64_t ld16 = lce::pad_to(a.vw, 256);
-        e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, v0, a.vw, base + f.w16, ld16, compute_dtype(p), s);
+        e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, v0, a.vw, base + f.w16, ld16, compute_dtype(p),
+                                       splits(p), s);
         if (e != hipSuccess) return hip_fail(e, "convert_w");
         a.w = base + f.w16; a.ldw = ld16; a.w_dtype = compute_dtype(p); a.wv0 = v0; a.Vw = a.vw;
       } else {
@@ -426,7 +438,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.scale = p->logit_scale; a.z_reg = p->z_reg;
   a.dx = dx; a.dw = dw;
   a.dz = base + b.dz;
-  a.dx_acc = b.slabs > 1 ? (float*)(base + b.dx_acc) : nullptr;
+  a.dx_acc = b.slabs > 1 || splits(p) ? (float*)(base + b.dx_acc) : nullptr;
   a.dx_part = (float*)(base + b.dx_part);
   a.dw_part = (float*)(base + b.dw_part);
   rc = current_num_cus(&a.num_cus);
@@ -456,17 +468,19 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
       if (e != hipSuccess) return hip_fail(e, "compact_labels");
     }
     float* lse_c = pack ? (float*)(base + b.lse_c) : nullptr;
-    e = x32 ? lce::launch_gather_rows_f32((const float*)x, p->ldx, p->H, perm, a.n_rows, p->N, base + k.xc, k.ldxc,
-                                          pack ? lse : nullptr, lse_c, a.num_cus, s)
+    e = x32 ? lce::launch_gather_rows_split((const float*)x, p->ldx, p->H, perm, a.n_rows, p->N, base + k.xc, k.ldxc,
+                                            base + k.xk, k.ldxk, pack ? lse : nullptr, lse_c, a.num_cus, s)
             : lce::launch_gather_rows(x, p->ldx * 2, perm, a.n_rows, p->N, base + k.xc, k.ldxc * 2, lse, lse_c,
                                       a.num_cus, s);
     if (e != hipSuccess) return hip_fail(e, "gather_rows");
   }
-  if (x32) {  // fp32 activations reach the tile kernels as the bf16 packed copy, whether or not rows were dropped
+  if (x32) {  // fp32 activations reach the tile kernels as copies in bf16 pairs, whether or not rows were dropped
     a.x = a.xc;
     a.ldx = a.ldxc;
     a.x_dtype = lce::DT_BF16;
   }
+  const bool split = splits(p);
+  const int64_t blk_bytes = a.Np * 2;  // times the slab width: one of the three blocks [hi ; lo ; hi] of a split dz
 
   for (int64_t i = 0; i < b.slabs; ++i) {
     a.v0 = i * b.vs;
@@ -478,7 +492,8 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     if (p->w_dtype == LCE_F32) {
       // dz and dx of this slab read a 16-bit copy of its columns of the fp32 weight
       if ((ph & LCE_PHASE_BWD_DZ) || (dx && (ph & LCE_PHASE_BWD_DX))) {
-        e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, a.v0, a.vw, base + b.w16, a.vs, compute_dtype(p), s);
+        e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, a.v0, a.vw, base + b.w16, a.vs, compute_dtype(p),
+                                       split, s);
         if (e != hipSuccess) return hip_fail(e, "convert_w");
       }
       a.w = base + b.w16; a.ldw = a.vs; a.w_dtype = compute_dtype(p); a.wv0 = a.v0; a.Vw = a.vw;
@@ -487,16 +502,56 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     }
     a.first = i == 0;
     a.last = i == b.slabs - 1;
+    if (!split) {
+      if (ph & LCE_PHASE_BWD_DZ) {
+        e = lce::launch_bwd_dz(a, s);
+        if (e != hipSuccess) return hip_fail(e, "bwd_dz");
+      }
+      if (dx && (ph & LCE_PHASE_BWD_DX)) {
+        e = lce::launch_bwd_dx(a, s);
+        if (e != hipSuccess) return hip_fail(e, "bwd_dx");
+      }
+      if (dw && (ph & LCE_PHASE_BWD_DW)) {
+        e = lce::launch_bwd_dw(a, s);
+        if (e != hipSuccess) return hip_fail(e, "bwd_dw");
+      }
+      continue;
+    }
+    // fp32 tensors as bf16 pairs (lce_gemm.h): x = [hi | hi | lo] against W = [hi ; lo ; hi] along a K axis of
+    // 3 H for the logits; dz comes back as three blocks [hi ; lo ; hi] of Np rows.
+    char* dz0 = (char*)a.dz;
+    const int64_t blk = blk_bytes * a.vs;
     if (ph & LCE_PHASE_BWD_DZ) {
-      e = lce::launch_bwd_dz(a, s);
+      lce::BwdArgs z = a;
+      z.H = 3 * p->H;
+      z.split = 1;
+      e = lce::launch_bwd_dz(z, s);
       if (e != hipSuccess) return hip_fail(e, "bwd_dz");
     }
     if (dx && (ph & LCE_PHASE_BWD_DX)) {
-      e = lce::launch_bwd_dx(a, s);
-      if (e != hipSuccess) return hip_fail(e, "bwd_dx");
+      // dx += dz_hi W_hi^T + dz_lo W_hi^T + dz_hi W_lo^T: three passes over the running fp32 sum
+      const char* w_hi = (const char*)a.w;
+      const char* w_lo = w_hi + p->H * a.ldw * 2;
+      for (int pass = 0; pass < 3; ++pass) {
+        lce::BwdArgs d = a;
+        d.dz = dz0 + (pass == 1 ? blk : 0);
+        d.w = pass == 2 ? w_lo : w_hi;
+        d.first = a.first && pass == 0;
+        d.last = a.last && pass == 2;
+        e = lce::launch_bwd_dx(d, s);
+        if (e != hipSuccess) return hip_fail(e, "bwd_dx");
+      }
     }
     if (dw && (ph & LCE_PHASE_BWD_DW)) {
-      e = lce::launch_bwd_dw(a, s);
+      // dW = x_hi^T dz_hi + x_hi^T dz_lo + x_lo^T dz_hi: one contraction over 3 Np token rows, the copy of x
+      // stacked [hi ; hi ; lo] against the three blocks of dz (rows past the last kept token are zeros in both)
+      lce::BwdArgs g = a;
+      g.x = base + k.xk;
+      g.ldx = k.ldxk;
+      g.n_rows = nullptr;
+      g.N = 3 * a.Np;
+      g.Np = 3 * a.Np;
+      e = lce::launch_bwd_dw(g, s);
       if (e != hipSuccess) return hip_fail(e, "bwd_dw");
     }
   }

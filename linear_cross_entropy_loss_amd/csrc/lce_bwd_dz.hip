@@ -45,7 +45,11 @@ static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must
 // but at most one is inside or outside as a whole, uniformly over the wave; the
 // one run that V cuts through is handled element by element.  Columns outside
 // are written as exact zeros.
-template <class T, bool ZREG, bool VTAIL>
+//
+// SPLIT (fp32 tensors carried as bf16 pairs, lce_gemm.h): dz is staged as hi = bf16(dz) and lo = bf16(dz - hi)
+// in three blocks of Np rows, [hi ; lo ; hi].  The staging sequence simply runs twice, once per part (this
+// path serves accuracy, not speed).
+template <class T, bool ZREG, bool VTAIL, bool SPLIT>
 LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
   typedef typename elem_of<T>::type E;
   const int64_t v0 = a.v0 + (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
@@ -81,6 +85,9 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
     ykey[qb] = (valid && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == half) ? (int)rel : -1;
   }
 
+  const int64_t blk = a.Np * a.vs;  // SPLIT: elements between the three blocks of the stage
+#pragma unroll
+  for (int part = 0; part < (SPLIT ? 2 : 1); ++part)
 #pragma unroll
   for (int ph = 0; ph < 2; ++ph) {
 #pragma unroll
@@ -114,6 +121,10 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
               for (int i = 4 * h2; i < 4 * h2 + 4; ++i) d[i] = 0.f;
             }
           }
+          if (SPLIT && part == 1) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d[i] = bf16_lo(d[i]);
+          }
           const unsigned x0 = pack2<T>(d[0], d[1]), x1 = pack2<T>(d[2], d[3]);
           const unsigned y0 = pack2<T>(d[4], d[5]), y1 = pack2<T>(d[6], d[7]);
           // lanes 0..31 keep their quad g and receive the partner's quad g; lanes
@@ -142,7 +153,9 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
             if (want == pp * 16 + r) zt = acc[2 * ph + pp][qb][r];
         float p = __builtin_amdgcn_exp2f(fmaf(zt, c1, nlse[qb]));
         if (ZREG) p *= gain[qb];
-        *reinterpret_cast<unsigned short*>(lrow + (((yl >> 3) ^ sw) << 4) + (yl & 7) * 2) = to_bits<T>(p - dz_scale<T>());
+        float tv = p - dz_scale<T>();
+        if (SPLIT && part == 1) tv = bf16_lo(tv);
+        *reinterpret_cast<unsigned short*>(lrow + (((yl >> 3) ^ sw) << 4) + (yl & 7) * 2) = to_bits<T>(tv);
       }
       // keep the register footprint small: an operand tile is in flight across this function
       __builtin_amdgcn_sched_barrier(0);
@@ -156,7 +169,9 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * (kPassCols * 2) + ((chunk ^ (row & 7) ^ ((row >> 3) & 1)) << 4));
       // streaming store: dz (1 GiB per slab) is read back from HBM by the next kernels anyway, and a
       // normal store would evict the W / x tiles the following main loop is about to reuse from L2
-      __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.vs + ph * kPassCols + chunk * 8));
+      E* dst = out + (int64_t)row * a.vs + ph * kPassCols + chunk * 8 + (SPLIT && part == 1 ? blk : 0);
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(dst));
+      if (SPLIT && part == 0) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(dst + 2 * blk));
       if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most 4 rows in registers at a time
     }
   }
@@ -169,7 +184,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
 // The launch covers `tiles_p` tile columns of the slab starting at column tile
 // `tp0`: all the full ones, or (VTAIL) those from the one straddling the end
 // of the vocabulary to the end of the padded slab.
-template <class T, bool ZREG, bool VTAIL, bool KMASK> struct DzProblem {
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT> struct DzProblem {
   typedef typename elem_of<T>::type E;
   static constexpr bool kKMask = KMASK;
   static constexpr bool kVarK = false;
@@ -184,7 +199,9 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK> struct DzProblem {
     const bool packed = rows != a.N;
     x = reinterpret_cast<const E*>(packed ? a.xc : a.x);
     ldx = packed ? a.ldxc : a.ldx;
-    tiles_q = (int)((rows + kTile - 1) / kTile);
+    // SPLIT: the dW contraction runs through all Np rows of each of the three blocks of the stage, so every
+    // token tile is written (rows past the last kept token as zeros), not only those that hold kept tokens
+    tiles_q = SPLIT ? (int)(a.Np / kTile) : (int)((rows + kTile - 1) / kTile);
   }
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void coords(int tile, int& tp, int& tq) const {
@@ -203,22 +220,22 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK> struct DzProblem {
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
     coords(tile, tp, tq);
-    dz_epilogue_impl<T, ZREG, VTAIL>(a, rows, acc, tp, tq, scratch);
+    dz_epilogue_impl<T, ZREG, VTAIL, SPLIT>(a, rows, acc, tp, tq, scratch);
   }
 };
 
-template <class T, bool ZREG, bool VTAIL, bool KMASK>
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DzProblem<T, ZREG, VTAIL, KMASK> prob(a);
-  Pipe3<T, E, false, E, true, DzProblem<T, ZREG, VTAIL, KMASK>> pipe(prob);
+  DzProblem<T, ZREG, VTAIL, KMASK, SPLIT> prob(a);
+  Pipe3<T, E, false, E, true, DzProblem<T, ZREG, VTAIL, KMASK, SPLIT>> pipe(prob);
   pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
-template <class T, bool ZREG, bool VTAIL, bool KMASK>
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT>
 hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = bwd_dz_persistent_kernel<T, ZREG, VTAIL, KMASK>;
+  auto kern = bwd_dz_persistent_kernel<T, ZREG, VTAIL, KMASK, SPLIT>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e != hipSuccess) return e;
@@ -228,29 +245,30 @@ hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
 }
 
 // All full tile columns of the slab, then the column that straddles the end of the vocabulary.
-template <class T, bool ZREG> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
+template <class T, bool ZREG, bool SPLIT> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
   const int64_t tq = a.Np / kTile, full = a.vw / kTile, tail = a.vs / kTile - full;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = exact_k ? launch_one<T, ZREG, false, false>(a, full * tq, s)
-                           : launch_one<T, ZREG, false, true>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, ZREG, false, false, SPLIT>(a, full * tq, s)
+                           : launch_one<T, ZREG, false, true, SPLIT>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (tail > 0) return launch_one<T, ZREG, true, true>(a, tail * tq, s);
+  if (tail > 0) return launch_one<T, ZREG, true, true, SPLIT>(a, tail * tq, s);
   return hipSuccess;
 }
 
-template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  return a.z_reg != 0.f ? launch_persistent_z<T, true>(a, s)
-                        : launch_persistent_z<T, false>(a, s);
+template <class T, bool SPLIT> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  return a.z_reg != 0.f ? launch_persistent_z<T, true, SPLIT>(a, s)
+                        : launch_persistent_z<T, false, SPLIT>(a, s);
 }
 
 }  // namespace
 
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
-  // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as the bf16 packed copy)
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16)
+    return a.split ? launch_persistent<BF16, true>(a, s) : launch_persistent<BF16, false>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, false>(a, s);
+  // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as bf16 pairs with split set)
   return hipErrorInvalidValue;
 }
 

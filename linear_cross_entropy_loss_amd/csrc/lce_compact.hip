@@ -7,7 +7,7 @@
 // and multiplies them away.)
 //
 //   compact_labels  perm[j] = original index of the j-th kept token, yc[j] its label, n_rows = how many
-//   gather_rows     xc[j] = x[perm[j]], lse_c[j] = lse[perm[j]]
+//   gather_rows     xc[j] = x[perm[j]], lse_c[j] = lse[perm[j]]  (fp32 activations: as bf16 pairs, see gather_rows_split_kernel)
 //   scatter_rows    rows of dropped tokens of dx = 0 (and dx[perm[j]] = dxc[j] where dx was staged packed)
 //
 // When no token is dropped (n_rows == N) the row copies are skipped and the
@@ -111,32 +111,49 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const char* x, int64_t
   }
 }
 
-// fp32 activations: the packed copy is made in the 16-bit compute type (round to nearest even), so the tile
-// kernels only ever read 16-bit operands.  The copy is made even when no token is dropped, and `perm` /
-// `n_rows` may be null (all rows, in place order).  One thread converts 8 consecutive elements.
-template <class T>
-__global__ __launch_bounds__(256) void gather_rows_f32_kernel(const float* x, int64_t ldx, int64_t H, const int* perm,
-                                                              const int64_t* n_rows, int64_t N, unsigned short* xc,
-                                                              int64_t ldxc, const float* lse, float* lse_c) {
+// fp32 activations reach the tile kernels as bf16 pairs, x = hi + lo (lce_gemm.h), in two copies that are made
+// even when no token is dropped (`perm` / `n_rows` may be null: all rows, in their order):
+//   xc  [rows][3 H]       row j = [hi | hi | lo] of x[perm[j]]: the K axis of the logit contraction, three
+//                         times as long, against a weight copy laid out [hi ; lo ; hi]
+//   xk  [3][Np][H]        hi, hi, lo again, stacked along the TOKEN axis, which is the K axis of
+//                         dW = x^T dz (against dz staged as [hi ; lo ; hi]); rows from `rows` to Np of each
+//                         block are zeros, since K runs through them.  Null in the forward.
+// One workgroup per packed row (grid-stride); elements go out as single 16-bit stores, consecutive lanes to
+// consecutive addresses (H need not be a multiple of anything, so the three parts of a row of xc do not
+// start on 16-byte boundaries).
+__global__ __launch_bounds__(256) void gather_rows_split_kernel(const float* x, int64_t ldx, int64_t H, const int* perm,
+                                                                const int64_t* n_rows, int64_t N, int64_t Np,
+                                                                unsigned short* xc, int64_t ldxc, unsigned short* xk,
+                                                                int64_t ldxk, const float* lse, float* lse_c) {
   const int64_t rows = n_rows != nullptr ? packed_rows(n_rows, N) : N;
-  const int chunks = (int)(ldxc / 8);
-  for (int64_t j = blockIdx.x; j < rows; j += gridDim.x) {
+  const int64_t jend = xk != nullptr ? Np : rows;
+  for (int64_t j = blockIdx.x; j < jend; j += gridDim.x) {
+    if (j >= rows) {  // K padding of the dW contraction
+      for (int64_t k = threadIdx.x; k < ldxk; k += 256)
+        xk[j * ldxk + k] = xk[(Np + j) * ldxk + k] = xk[(2 * Np + j) * ldxk + k] = 0;
+      continue;
+    }
     const int64_t src = perm != nullptr ? packed_token(perm, j, N) : j;
     if (lse != nullptr && threadIdx.x == 0) lse_c[j] = lse[src];
     const float* s = x + src * ldx;
-    for (int c = threadIdx.x; c < chunks; c += 256) {
-      // the row stride is a multiple of 4: a quad that starts inside the row may be read whole
-      f32x4_t lo, hi;
-      for (int e = 0; e < 4; ++e) lo[e] = hi[e] = 0.f;
-      if (8 * c < H) lo = *reinterpret_cast<const f32x4_t*>(s + 8 * c);
-      if (8 * c + 4 < H) hi = *reinterpret_cast<const f32x4_t*>(s + 8 * c + 4);
-      u32x4_t o;
-      o[0] = pack2<T>(lo[0], lo[1]);
-      o[1] = pack2<T>(lo[2], lo[3]);
-      o[2] = pack2<T>(hi[0], hi[1]);
-      o[3] = pack2<T>(hi[2], hi[3]);
-      *reinterpret_cast<u32x4_t*>(xc + j * ldxc + 8 * c) = o;
+    unsigned short* c = xc + j * ldxc;
+    for (int64_t k = threadIdx.x; k < H; k += 256) {
+      const float v = s[k];
+      const unsigned short hi = to_bits<BF16>(v), lo = to_bits<BF16>(bf16_lo(v));
+      c[k] = hi;
+      c[H + k] = hi;
+      c[2 * H + k] = lo;
+      if (xk != nullptr) {
+        xk[j * ldxk + k] = hi;
+        xk[(Np + j) * ldxk + k] = hi;
+        xk[(2 * Np + j) * ldxk + k] = lo;
+      }
     }
+    // stride padding is read by the tile kernels and must be finite
+    for (int64_t k = 3 * H + threadIdx.x; k < ldxc; k += 256) c[k] = 0;
+    if (xk != nullptr)
+      for (int64_t k = H + threadIdx.x; k < ldxk; k += 256)
+        xk[j * ldxk + k] = xk[(Np + j) * ldxk + k] = xk[(2 * Np + j) * ldxk + k] = 0;
   }
 }
 
@@ -183,11 +200,13 @@ hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_ind
   return hipGetLastError();
 }
 
-hipError_t launch_gather_rows_f32(const float* x, int64_t ldx, int64_t H, const int* perm, const int64_t* n_rows,
-                                  int64_t N, void* xc, int64_t ldxc, const float* lse, float* lse_c, int num_cus,
-                                  hipStream_t s) {
-  hipLaunchKernelGGL(gather_rows_f32_kernel<BF16>, dim3(row_grid(N, num_cus)), dim3(256), 0, s, x, ldx, H, perm, n_rows,
-                     N, reinterpret_cast<unsigned short*>(xc), ldxc, lse, lse_c);
+hipError_t launch_gather_rows_split(const float* x, int64_t ldx, int64_t H, const int* perm, const int64_t* n_rows,
+                                    int64_t N, void* xc, int64_t ldxc, void* xk, int64_t ldxk, const float* lse,
+                                    float* lse_c, int num_cus, hipStream_t s) {
+  const int64_t Np = padded_tokens(N);
+  hipLaunchKernelGGL(gather_rows_split_kernel, dim3(row_grid(Np, num_cus)), dim3(256), 0, s, x, ldx, H, perm, n_rows, N,
+                     Np, reinterpret_cast<unsigned short*>(xc), ldxc, reinterpret_cast<unsigned short*>(xk), ldxk, lse,
+                     lse_c);
   return hipGetLastError();
 }
 

@@ -13,7 +13,9 @@ namespace lce {
 namespace {
 
 // One thread converts 8 consecutive columns of one row (two 16-byte loads, one 16-byte store).
-template <class T>
+// SPLIT (fp32 activations as well as weight): the copy has 3 H rows -- bf16(w), then bf16(w - bf16(w)),
+// then bf16(w) again -- the [hi | lo | hi] operand of the three-term product described in lce_gemm.h.
+template <class T, bool SPLIT>
 __global__ __launch_bounds__(256) void convert_w_slab_kernel(const float* src, int64_t ld, int64_t H, int64_t v0,
                                                                int64_t vw, unsigned short* dst, int64_t dst_ld) {
   const int64_t runs_per_row = dst_ld / 8;
@@ -37,22 +39,30 @@ __global__ __launch_bounds__(256) void convert_w_slab_kernel(const float* src, i
 #pragma unroll
     for (int j = 0; j < 4; ++j) o[j] = pack2<T>(v[2 * j], v[2 * j + 1]);
     *reinterpret_cast<u32x4_t*>(dst + h * dst_ld + c) = o;
+    if (SPLIT) {
+      *reinterpret_cast<u32x4_t*>(dst + (2 * H + h) * dst_ld + c) = o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = pack2<T>(bf16_lo(v[2 * j]), bf16_lo(v[2 * j + 1]));
+      *reinterpret_cast<u32x4_t*>(dst + (H + h) * dst_ld + c) = o;
+    }
   }
 }
 
 }  // namespace
 
 hipError_t launch_convert_w_slab(const float* src, int64_t ld, int64_t H, int64_t v0, int64_t vw, void* dst,
-                                 int64_t dst_ld, int compute_dtype, hipStream_t s) {
+                                 int64_t dst_ld, int compute_dtype, bool split, hipStream_t s) {
   const int64_t total = H * (dst_ld / 8);
   int64_t blocks = (total + 255) / 256;
   if (blocks > 8192) blocks = 8192;
   if (blocks < 1) return hipSuccess;
   unsigned short* d = reinterpret_cast<unsigned short*>(dst);
-  if (compute_dtype == DT_F16) {
-    hipLaunchKernelGGL(convert_w_slab_kernel<F16>, dim3((unsigned)blocks), dim3(256), 0, s, src, ld, H, v0, vw, d, dst_ld);
+  if (split) {
+    hipLaunchKernelGGL((convert_w_slab_kernel<BF16, true>), dim3((unsigned)blocks), dim3(256), 0, s, src, ld, H, v0, vw, d, dst_ld);
+  } else if (compute_dtype == DT_F16) {
+    hipLaunchKernelGGL((convert_w_slab_kernel<F16, false>), dim3((unsigned)blocks), dim3(256), 0, s, src, ld, H, v0, vw, d, dst_ld);
   } else {
-    hipLaunchKernelGGL(convert_w_slab_kernel<BF16>, dim3((unsigned)blocks), dim3(256), 0, s, src, ld, H, v0, vw, d, dst_ld);
+    hipLaunchKernelGGL((convert_w_slab_kernel<BF16, false>), dim3((unsigned)blocks), dim3(256), 0, s, src, ld, H, v0, vw, d, dst_ld);
   }
   return hipGetLastError();
 }

@@ -82,6 +82,15 @@ template <> struct dz_shift<F16> { static constexpr int value = 10; };
 template <class T> constexpr float dz_scale() { return (float)(1 << dz_shift<T>::value); }
 template <class T> constexpr float dz_unscale() { return 1.f / (float)(1 << dz_shift<T>::value); }
 
+// fp32 operands are carried as two bf16 numbers, v = hi + lo with hi = bf16(v) and lo = bf16(v - hi): 16
+// bits of mantissa instead of 8.  A product a*b is then taken as a_hi*b_hi + a_hi*b_lo + a_lo*b_hi (the
+// a_lo*b_lo term is of relative order 2^-18 and dropped), which the kernels get by running along a K axis
+// that is three times as long, over copies of the operands laid out as [hi | hi | lo] and [hi | lo | hi].
+LCE_DEV float bf16_hi(float v) {
+  return __builtin_bit_cast(float, (unsigned)to_bits<BF16>(v) << 16);
+}
+LCE_DEV float bf16_lo(float v) { return v - bf16_hi(v); }  // exact in fp32; rounded to bf16 when stored
+
 // threadIdx.x behind an optimisation barrier.  Epilogues that run inside a
 // persistent tile loop derive their per-lane indices from this, so that the
 // compiler recomputes them per tile instead of hoisting them out of the loop

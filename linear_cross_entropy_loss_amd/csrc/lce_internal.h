@@ -90,6 +90,10 @@ struct BwdArgs {
   float* dw_part;
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
+  // fp32 tensors carried as bf16 pairs (lce_gemm.h): dz is staged as three blocks of Np rows,
+  // [hi ; lo ; hi], `dz` pointing at the first; only bwd_dz looks at this flag (the dx and dW launches get
+  // plain 16-bit problems over these blocks).
+  int split;
   // Packed rows (tokens with an ignored label dropped; n_rows == null: the call works on all rows).
   // *n_rows (device) rows are worked on.  When *n_rows != N they are the rows of xc (row stride ldxc) and
   // row j of dx belongs to token perm[j]: the dx kernels store it there themselves, or -- dxc != null, a dx
@@ -109,9 +113,9 @@ hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
 // dst[h][c] = 16-bit rounding of src[h * ld + v0 + c] for c < vw, 0 for vw <= c < dst_ld; h < H.
-// compute_dtype: DT_BF16 or DT_F16.
+// compute_dtype: DT_BF16 or DT_F16.  split: dst has 3 H rows, [bf16 hi ; bf16 lo ; bf16 hi] of the fp32 values.
 hipError_t launch_convert_w_slab(const float* src, int64_t ld, int64_t H, int64_t v0, int64_t vw, void* dst,
-                                 int64_t dst_ld, int compute_dtype, hipStream_t s);
+                                 int64_t dst_ld, int compute_dtype, bool split, hipStream_t s);
 
 // Row count / row -> token map of the packed rows as the kernels read them from device memory, forced
 // into range: a call restricted to some phases on a workspace whose packing pre-pass did not run must
@@ -136,11 +140,13 @@ hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_ind
 hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, const int* perm, const int64_t* n_rows, int64_t N,
                               void* xc, int64_t ldxc_bytes, const float* lse, float* lse_c, int num_cus,
                               hipStream_t s);
-// The same for fp32 activations: xc is written in bf16 (the compute type of fp32 inputs), always, also when
-// no token is dropped; perm / n_rows may be null (all N rows in their order).  ldx, ldxc in elements.
-hipError_t launch_gather_rows_f32(const float* x, int64_t ldx, int64_t H, const int* perm, const int64_t* n_rows,
-                                  int64_t N, void* xc, int64_t ldxc, const float* lse, float* lse_c, int num_cus,
-                                  hipStream_t s);
+// fp32 activations: xc[j] = [hi | hi | lo] of x[perm[j]] as bf16 (3 H elements per row, row stride ldxc), and
+// -- xk not null -- the same three parts stacked along the tokens, xk[b * Np + j] (row stride ldxk, rows from
+// *n_rows to Np of each block zeroed).  Always made, also when no token is dropped; perm / n_rows may be null
+// (all N rows in their order).  Strides in elements.
+hipError_t launch_gather_rows_split(const float* x, int64_t ldx, int64_t H, const int* perm, const int64_t* n_rows,
+                                    int64_t N, void* xc, int64_t ldxc, void* xk, int64_t ldxk, const float* lse,
+                                    float* lse_c, int num_cus, hipStream_t s);
 // dx[perm[j]] = dxc[j] for j < *n_rows (skipped when dxc is null) and dx[i] = 0 for every token i with
 // y[i] == ignore_index, in 8-byte pieces covering row_bytes; nothing when *n_rows == N.
 hipError_t launch_scatter_rows(const void* dxc, int64_t lddxc_bytes, const int* perm, const int64_t* n_rows,

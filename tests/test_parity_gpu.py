@@ -2,7 +2,9 @@
 
 Tolerances (the ones the operator is specified to): loss within 1e-3 relative; dx and dW within 2e-2 both
 as max_abs(diff)/max_abs(ref) and as an L2 ratio, for 16-bit compute; valid-token count and ignore_index
-masking bit-exact.
+masking bit-exact.  fp32 tensors are computed as bf16 pairs (16 bits of mantissa, better than the tf32
+products the reference's tl.dot uses for fp32 tensors, ops.py:195) and are held to 1e-5 on the loss and
+1e-3 on the gradients.
 """
 import pytest
 import torch
@@ -13,6 +15,11 @@ pytestmark = pytest.mark.gpu
 
 LOSS_RTOL = 1e-3
 GRAD_TOL = 2e-2
+
+
+def _tols(dtype):
+    """(loss, gradient) tolerance for tensors of `dtype`."""
+    return (1e-5, 1e-3) if dtype == torch.float32 else (LOSS_RTOL, GRAD_TOL)
 
 
 def _run(x, y, w, ignore_index, z_reg, scale, n_chunk, monitoring, grad_output=1.0):
@@ -52,10 +59,11 @@ def test_forward_backward_matches_oracle(N, H, V, dtype, w_dtype, ign, z_reg, sc
     out, dx, dw = _run(x, y, w, -1, z_reg, scale, n_chunk, mon, grad_output=1.7)
     ref = _oracle(x, y, w, -1, z_reg, scale, grad_output=1.7)
     loss = out[0].item()
-    assert abs(loss - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item()), (loss, ref.loss.item())
-    assert abs(out[1].item() - ref.z_reg.item()) <= LOSS_RTOL * abs(ref.z_reg.item())
+    loss_tol, grad_tol = _tols(dtype)
+    assert abs(loss - ref.loss.item()) <= loss_tol * abs(ref.loss.item()), (loss, ref.loss.item())
+    assert abs(out[1].item() - ref.z_reg.item()) <= loss_tol * abs(ref.z_reg.item())
     if mon:
-        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item()) + 1e-3
+        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-3 * abs(ref.logit_max.item())
         assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item())
         assert abs(out[4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item())
     else:
@@ -64,7 +72,7 @@ def test_forward_backward_matches_oracle(N, H, V, dtype, w_dtype, ign, z_reg, sc
     for name, got, want in (("dx", dx, ref.dx), ("dw", dw, ref.dw)):
         emax, el2 = rel_errors(got, want)
         print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
-        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
+        assert emax <= grad_tol and el2 <= grad_tol, (name, emax, el2)
     # bit-exact masking
     ignored = (y == -1)
     if ignored.any():
@@ -98,9 +106,10 @@ def test_mid_size_matches_fp64_oracle_evaluated_on_gpu(N, H, V, dtype, w_dtype, 
     out[0].backward()
     torch.cuda.synchronize()
     ref = lce_forward_backward_fp64(x, y, w, -1, z_reg, scale, chunk=512)
-    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item())
+    loss_tol, grad_tol = _tols(dtype)
+    assert abs(out[0].item() - ref.loss.item()) <= loss_tol * abs(ref.loss.item())
     if mon:
-        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item()) + 1e-3
+        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-3 * abs(ref.logit_max.item())
         assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item())
         assert abs(out[4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item())
     for name, got, want in (("dx", xd.grad, ref.dx), ("dw", wd.grad, ref.dw)):
@@ -108,7 +117,7 @@ def test_mid_size_matches_fp64_oracle_evaluated_on_gpu(N, H, V, dtype, w_dtype, 
         emax = (d.abs().max() / want.abs().max()).item()
         el2 = (d.norm() / want.norm()).item()
         print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
-        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
+        assert emax <= grad_tol and el2 <= grad_tol, (name, emax, el2)
     assert (xd.grad[y == -1] == 0).all()
 
 
@@ -141,17 +150,18 @@ def test_arbitrary_shapes_match_oracle(N, H, V, dtype, w_dtype, ign, z_reg, scal
     y[0] = V - 1  # a target in the last valid column
     out, dx, dw = _run(x, y, w, -1, z_reg, scale, n_chunk, mon, grad_output=0.9)
     ref = _oracle(x, y, w, -1, z_reg, scale, grad_output=0.9)
-    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item()), (out[0].item(), ref.loss.item())
-    assert abs(out[1].item() - ref.z_reg.item()) <= LOSS_RTOL * abs(ref.z_reg.item())
+    loss_tol, grad_tol = _tols(dtype)
+    assert abs(out[0].item() - ref.loss.item()) <= loss_tol * abs(ref.loss.item()), (out[0].item(), ref.loss.item())
+    assert abs(out[1].item() - ref.z_reg.item()) <= loss_tol * abs(ref.z_reg.item())
     if mon:
-        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item()) + 1e-3
+        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-3 * abs(ref.logit_max.item())
         assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item()) + 1e-4
         assert abs(out[4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item())
     assert dx.shape == x.shape and dw.shape == w.shape and dx.dtype == x.dtype and dw.dtype == w.dtype
     for name, got, want in (("dx", dx, ref.dx), ("dw", dw, ref.dw)):
         emax, el2 = rel_errors(got, want)
         print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
-        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
+        assert emax <= grad_tol and el2 <= grad_tol, (name, emax, el2)
     ignored = (y == -1)
     if ignored.any():
         assert (dx.cpu()[ignored] == 0).all()
@@ -227,12 +237,13 @@ def test_randomized_shapes_and_options_match_oracle():
             y[0] = 0
         out, dx, dw = _run(x, y, w, -1, zreg, scale, nc, mon, grad_output=1.3)
         ref = _oracle(x, y, w, -1, zreg, scale, grad_output=1.3)
-        assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item()), it
+        loss_tol, grad_tol = _tols(dt)
+        assert abs(out[0].item() - ref.loss.item()) <= loss_tol * abs(ref.loss.item()), it
         if mon:
-            assert abs(out[2].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item()) + 1e-3, it
+            assert abs(out[2].item() - ref.logit_max.item()) <= 1e-3 * abs(ref.logit_max.item()) + 1e-5, it
             assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item()) + 1e-4, it
             assert abs(out[4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item()), it
         for got, want in ((dx, ref.dx), (dw, ref.dw)):
             emax, el2 = rel_errors(got, want)
-            assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (it, emax, el2)
+            assert emax <= grad_tol and el2 <= grad_tol, (it, emax, el2)
         assert (dx.cpu()[y == -1] == 0).all(), it

@@ -223,7 +223,7 @@ def test_module_api_3d_input_monitoring_and_no_grad():
     assert torch.equal(loss2, loss.detach())
     assert set(m.latest_metrics) == {"logit_norm", "logit_max", "logit_entropy", "z_value"}
     ref = lce_forward_fp64(x.detach().cpu().double(), y.cpu(), m.weight.detach().cpu().double(), -1, 1e-4, 0.5)
-    assert abs(m.latest_metrics["logit_max"].item() - ref.logit_max.item()) <= 1e-2 * abs(ref.logit_max.item())
+    assert abs(m.latest_metrics["logit_max"].item() - ref.logit_max.item()) <= 1e-3 * abs(ref.logit_max.item())
     assert abs(m.latest_metrics["logit_entropy"].item() - ref.logit_entropy.item()) <= 2e-3 * ref.logit_entropy.item()
     assert abs(m.latest_metrics["logit_norm"].item() - ref.logit_norm.item()) <= 2e-3 * ref.logit_norm.item()
     assert abs(m.latest_metrics["z_value"].item() - ref.z_reg.item()) <= 1e-3 * ref.z_reg.item()
