@@ -107,6 +107,15 @@ struct BwdArgs {
   int64_t lddxc;
 };
 
+// Factor applied to dx and dW after their fp32 accumulation: grad_out * logit_scale / n_valid
+// (linear_cross_entropy/ops.py:332, 443-447, 810), times the power of two that undoes the scaling of the staged
+// dz (`unscale`).  With no valid label at all every dz is zero and the factor is taken as 0, so both
+// gradients are exact zeros (what F.cross_entropy's backward gives for such a batch; the loss itself is NaN).
+__device__ __forceinline__ float final_factor_of(const BwdArgs& a, float unscale) {
+  const int64_t n = a.n_valid[0];
+  return n > 0 ? a.grad_out[0] * a.scale / (float)n * unscale : 0.f;
+}
+
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s);
 hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s);

@@ -16,6 +16,7 @@ may run any number of times and forward-only use pays no gradient cost.
 """
 from __future__ import annotations
 
+import contextvars
 import ctypes
 import math
 
@@ -32,8 +33,16 @@ bwd_configs: list = []
 # Whether tokens whose label is ignore_index are packed away on the device before the tile kernels run:
 # _lib.PACK_AUTO (the library decides by problem size: the pre-pass costs about 0.04 ms per step, which
 # a small problem does not earn back), _lib.PACK_ALWAYS or _lib.PACK_NEVER.  Results do not depend on it
-# beyond the summation order of dW and of the loss.
-PACK_ROWS = _lib.PACK_AUTO
+# beyond the summation order of dW and of the loss.  A context variable: `pack_rows.set(mode)` affects the
+# calling thread / task only (reset with the token it returns); the value seen by a forward call is carried
+# to its backward, which autograd may run on another thread.
+pack_rows: contextvars.ContextVar = contextvars.ContextVar("lce_pack_rows", default=_lib.PACK_AUTO)
+
+
+@torch.compiler.assume_constant_result
+def _pack_mode() -> int:
+    """Current value of `pack_rows`; while torch.compile traces, the value at trace time is baked into the graph."""
+    return int(pack_rows.get())
 
 
 def _ptr(t):
@@ -67,6 +76,15 @@ def _empty_rows(rows, cols, dtype, device):
     return torch.empty((rows, -(-cols // m) * m), dtype=dtype, device=device)[:, :cols]
 
 
+def _autocast_x(x, At):
+    """Under autocast the activations take the 16-bit type the weight already has, or -- fp32 master weight,
+    which is not copied -- the autocast dtype.  (The reference casts x and the whole weight to fp16, ops.py:665.)"""
+    if not torch.is_autocast_enabled("cuda"):
+        return x
+    target = At.dtype if At.dtype in (torch.float16, torch.bfloat16) else torch.get_autocast_dtype("cuda")
+    return x if x.dtype == target else x.to(target)
+
+
 def _check_inputs(x, y, At):
     if not (x.is_cuda and y.is_cuda and At.is_cuda):
         raise RuntimeError(
@@ -79,9 +97,17 @@ def _check_inputs(x, y, At):
         raise ValueError("weight must be 2-D with shape (in_features, out_features)")
 
 
-def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring):
+def _check_dtypes(x, At):
+    if x.dtype != At.dtype and not (At.dtype == torch.float32 and x.dtype in (torch.float16, torch.bfloat16)):
+        raise ValueError(
+            f"input is {x.dtype} but the weight is {At.dtype}: they must share a dtype, or the weight may be a "
+            "float32 master weight under 16-bit activations (under torch.autocast the input is cast for you)")
+
+
+def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack):
     """Runs lce_forward.  Returns (out5, lse, n_valid) and the (x, y, w) views the kernels read."""
     _check_inputs(x_in, y, At)
+    _check_dtypes(x_in, At)
     with torch.cuda.device(x_in.device):
         x = _aligned_rows(x_in.reshape(-1, x_in.shape[-1]))
         y1 = y.reshape(-1).contiguous()
@@ -94,7 +120,7 @@ def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_ch
             raise ValueError("labels must have one entry per input row")
         prob = _lib.make_problem(
             N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-            ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring, 0, PACK_ROWS,
+            ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring, 0, pack,
         )
         lib = _lib.load()
         _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")
@@ -113,7 +139,7 @@ def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_ch
 
 
 def _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,
-                   N_chunk_size, need_dx, need_dw):
+                   N_chunk_size, need_dx, need_dw, pack):
     """Runs lce_backward on what _forward_impl returned.  dx is (N, H), dw is (H, V); None when not needed."""
     N, H = x.shape
     V = w.shape[1]
@@ -125,7 +151,7 @@ def _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regulari
             prob = _lib.make_problem(
                 N, H, V, x.stride(0), w.stride(0), dx.stride(0) if need_dx else H + (-H) % 8,
                 dw.stride(0) if need_dw else V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-                ignore_index, logit_scale, z_regularization, N_chunk_size, False, 0, PACK_ROWS,
+                ignore_index, logit_scale, z_regularization, N_chunk_size, False, 0, pack,
             )
             lib = _lib.load()
             _, bwd_bytes = _lib.workspace_bytes(prob)
@@ -159,14 +185,15 @@ class LinearXentImplementation(torch.autograd.Function):
         N_chunk_size: int = 4096,
         monitoring: bool = True,
     ):
-        # Under autocast the activations take the autocast dtype; a float32 weight is NOT copied:
-        # the library rounds the fp32 master weight one vocabulary slab at a time, inside its workspace.
-        if torch.is_autocast_enabled("cuda") and x_in.dtype == torch.float32:
-            x_in = x_in.to(torch.get_autocast_dtype("cuda"))
+        # Under autocast the activations take the weight's 16-bit type or the autocast dtype; a float32 weight
+        # is NOT copied: the library rounds the fp32 master weight one vocabulary slab at a time, inside its
+        # workspace.
+        x_in = _autocast_x(x_in, At)
+        pack = _pack_mode()
         out5, lse, n_valid, x, y1, w = _forward_impl(
-            x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring)
+            x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack)
         ctx.save_for_backward(x, y1, w, lse, n_valid)
-        ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size)
+        ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size, pack)
         ctx.x_shape = x_in.shape
         loss, z_reg, logit_max, logit_ent, logit_norm = out5.unbind(0)
         ctx.mark_non_differentiable(z_reg, logit_max, logit_ent, logit_norm)
@@ -176,9 +203,9 @@ class LinearXentImplementation(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output, void0=None, void1=None, void2=None, void3=None):
         x, y1, w, lse, n_valid = ctx.saved_tensors
-        ignore_index, z_regularization, logit_scale, N_chunk_size = ctx.lce_cfg
+        ignore_index, z_regularization, logit_scale, N_chunk_size, pack = ctx.lce_cfg
         dx, dw = _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,
-                                N_chunk_size, ctx.needs_input_grad[0], ctx.needs_input_grad[2])
+                                N_chunk_size, ctx.needs_input_grad[0], ctx.needs_input_grad[2], pack)
         if dx is not None:
             dx = dx.view(ctx.x_shape)
         return dx, None, dw, None, None, None, None, None
@@ -193,14 +220,15 @@ class LinearXentImplementation(torch.autograd.Function):
 # ---------------------------------------------------------------------------------------------------------
 @torch.library.custom_op("lce_amd::forward", mutates_args=(), device_types="cuda")
 def _op_forward(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, ignore_index: int, z_regularization: float,
-                logit_scale: float, N_chunk_size: int, monitoring: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                logit_scale: float, N_chunk_size: int, monitoring: bool,
+                pack_rows_mode: int = 0) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     out5, lse, n_valid, _, _, _ = _forward_impl(x, y, At, ignore_index, z_regularization, logit_scale,
-                                                N_chunk_size, monitoring)
+                                                N_chunk_size, monitoring, pack_rows_mode)
     return out5, lse, n_valid
 
 
 @_op_forward.register_fake
-def _(x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring):
+def _(x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack_rows_mode=0):
     n = x.numel() // x.shape[-1]
     return (x.new_empty((5,), dtype=torch.float32), x.new_empty((n,), dtype=torch.float32),
             x.new_empty((1,), dtype=torch.int64))
@@ -209,41 +237,44 @@ def _(x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monit
 @torch.library.custom_op("lce_amd::backward", mutates_args=(), device_types="cuda")
 def _op_backward(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, lse: torch.Tensor, n_valid: torch.Tensor,
                  grad_loss: torch.Tensor, ignore_index: int, z_regularization: float, logit_scale: float,
-                 N_chunk_size: int, need_dx: bool, need_dw: bool) -> tuple[torch.Tensor, torch.Tensor]:
+                 N_chunk_size: int, need_dx: bool, need_dw: bool,
+                 pack_rows_mode: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
     x2 = _aligned_rows(x.reshape(-1, x.shape[-1]))
     dx, dw = _backward_impl(x2, y.reshape(-1).contiguous(), _aligned_rows(At), lse, n_valid, grad_loss,
-                            ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw)
+                            ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw,
+                            pack_rows_mode)
     dx = dx.view(x.shape) if dx is not None else x.new_empty((0,))
     dw = dw if dw is not None else At.new_empty((0,))
     return dx, dw
 
 
 @_op_backward.register_fake
-def _(x, y, At, lse, n_valid, grad_loss, ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw):
+def _(x, y, At, lse, n_valid, grad_loss, ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw,
+      pack_rows_mode=0):
     return (torch.empty_like(x, memory_format=torch.contiguous_format) if need_dx else x.new_empty((0,)),
             torch.empty_like(At, memory_format=torch.contiguous_format) if need_dw else At.new_empty((0,)))
 
 
 def _op_setup_context(ctx, inputs, output):
-    x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, _ = inputs
+    x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, _, pack = inputs
     _, lse, n_valid = output
     ctx.save_for_backward(x, y, At, lse, n_valid)
-    ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size)
+    ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size, pack)
 
 
 def _op_autograd(ctx, grad_out5, grad_lse, grad_n_valid):
     # Only the loss (entry 0 of the 5 scalars) is differentiable; the monitoring values are treated as
     # constants, as the reference marks them non-differentiable (ops.py:798-800).
     x, y, At, lse, n_valid = ctx.saved_tensors
-    ignore_index, z_regularization, logit_scale, N_chunk_size = ctx.lce_cfg
+    ignore_index, z_regularization, logit_scale, N_chunk_size, pack = ctx.lce_cfg
     need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[2]
     dx = dw = None
     if need_dx or need_dw:
         gx, gw = _op_backward(x, y, At, lse, n_valid, grad_out5[0:1].to(torch.float32), ignore_index,
-                              z_regularization, logit_scale, N_chunk_size, need_dx, need_dw)
+                              z_regularization, logit_scale, N_chunk_size, need_dx, need_dw, pack)
         dx = gx if need_dx else None
         dw = gw if need_dw else None
-    return dx, None, dw, None, None, None, None, None
+    return dx, None, dw, None, None, None, None, None, None
 
 
 _op_forward.register_autograd(_op_autograd, setup_context=_op_setup_context)
@@ -264,8 +295,10 @@ def linear_cross_entropy(
     While ``torch.compile`` / ``torch.export`` trace, the call goes through the registered operator
     ``torch.ops.lce_amd.forward``, so it can sit inside a compiled region; in eager mode it goes through
     ``LinearXentImplementation`` (same device calls, bit-identical results, about 80 us less dispatch
-    overhead per forward+backward).  Under autocast an fp32 ``x`` takes the autocast dtype; an fp32
-    weight is read as is (no 16-bit copy) and gets an fp32 gradient.
+    overhead per forward+backward).  Under autocast ``x`` takes the weight's 16-bit dtype, or the autocast
+    dtype when the weight is fp32; an fp32 weight is read as is (no 16-bit copy) and gets an fp32 gradient.
+    fp32 ``x`` with an fp32 weight (no autocast) is computed as bf16 pairs, accurate to about 1e-5 of the
+    largest gradient entry, at three times the matrix work of 16-bit tensors.
     """
     _check_inputs(x, y, At)
     if not torch.compiler.is_compiling():
@@ -273,10 +306,9 @@ def linear_cross_entropy(
             x, y, At, int(ignore_index), float(z_regularization), float(logit_scale), int(N_chunk_size),
             bool(monitoring))
         return loss, z_reg, logit_max, logit_ent, logit_norm
-    if torch.is_autocast_enabled("cuda") and x.dtype == torch.float32:
-        x = x.to(torch.get_autocast_dtype("cuda"))
+    x = _autocast_x(x, At)
     out5, _, _ = _op_forward(x, y, At, int(ignore_index), float(z_regularization), float(logit_scale),
-                             int(N_chunk_size), bool(monitoring))
+                             int(N_chunk_size), bool(monitoring), _pack_mode())
     loss, z_reg, logit_max, logit_ent, logit_norm = out5.unbind(0)
     return loss, z_reg.detach(), logit_max.detach(), logit_ent.detach(), logit_norm.detach()
 
@@ -295,8 +327,12 @@ class LinearCrossEntropyLoss(torch.nn.Linear):
         ignore_index: label value that is skipped. Default -100.
         logit_scale: positive factor applied to the logits before the loss. Default 1.0.
         z_regularization: weight of the ``mean(logsumexp(z)^2)`` penalty. Default 0.0.
-        N_chunk_size: bounds the scratch memory of a call to ``N_chunk_size * out_features * 4`` bytes
-            (the number of rows of ``x`` is free). Default 4096.
+        N_chunk_size: target for the scratch memory of the backward, ``N_chunk_size * out_features * 4`` bytes
+            (what the reference spends on one chunk of logits); the backward works through the vocabulary in
+            as many slabs as that takes.  The number of rows of ``x`` is free, but two terms grow with it: the
+            forward's per-token partial sums (``out_features / 32`` bytes per token, four times that with
+            monitoring) and the backward's fp32 running sum of ``dx`` and packed copy of ``x``
+            (``6 * in_features`` bytes per token).  Default 4096.
         init_method: optional callable applied to the weight instead of the default truncated normal.
 
     Set ``module.monitoring = True`` to also collect ``logit_norm``, ``logit_max``, ``logit_entropy`` and

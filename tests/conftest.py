@@ -52,7 +52,6 @@ def pack_mode(request):
         return
     from linear_cross_entropy_loss_amd import _lib, ops
 
-    old = ops.PACK_ROWS
-    ops.PACK_ROWS = _lib.PACK_ALWAYS if mode == "pack" else _lib.PACK_NEVER
+    token = ops.pack_rows.set(_lib.PACK_ALWAYS if mode == "pack" else _lib.PACK_NEVER)
     yield mode
-    ops.PACK_ROWS = old
+    ops.pack_rows.reset(token)  # (also undoes whatever the test itself set in between)

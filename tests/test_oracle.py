@@ -168,3 +168,24 @@ def test_all_ignored_gives_nan_like_cross_entropy():
     r = lce_forward_fp64(x, y, w, -1, 0.0, 1.0)
     assert r.n_valid == 0 and math.isnan(r.loss.item())
     assert math.isnan(F.cross_entropy(x @ w, y, ignore_index=-1).item())
+
+
+@pytest.mark.parametrize("zreg,scale,ignore_index", [(0.0, 1.0, -1), (1e-2, 0.5, -1), (0.3, 2.0, 5)])
+def test_eager_fp32_step_is_the_same_function_in_single_precision(zreg, scale, ignore_index):
+    """The CPU baseline (eager fp32 matmul + F.cross_entropy through autograd) against the fp64 closed forms:
+    same loss and gradients up to fp32 rounding, with z-regularisation and ignored labels present."""
+    from oracle import eager_fp32_step
+
+    x, y, w = _rand(48, 24, 40, seed=17, ignore_frac=0.3, ignore_index=ignore_index)
+    ref = lce_forward_backward_fp64(x, y, w, ignore_index, zreg, scale)
+    loss, dx, dw = eager_fp32_step(x, y, w, ignore_index, zreg, scale)
+    assert loss.dtype == torch.float32 and dx.dtype == torch.float32 and dw.dtype == torch.float32
+    assert abs(loss.item() - ref.loss.item()) <= 1e-5 * abs(ref.loss.item())
+    assert torch.allclose(dx.double(), ref.dx, rtol=1e-4, atol=1e-6 * ref.dx.abs().max().item())
+    assert torch.allclose(dw.double(), ref.dw, rtol=1e-4, atol=1e-6 * ref.dw.abs().max().item())
+    assert (dx[y == ignore_index] == 0).all()
+    # a dropped z-reg term or a wrong sign would not survive this: the two differ visibly when zreg changes
+    if zreg > 0:
+        loss0, dx0, _ = eager_fp32_step(x, y, w, ignore_index, 0.0, scale)
+        assert abs(loss0.item() - loss.item()) > 1e-3 * abs(loss.item())
+        assert (dx0 - dx).abs().max() > 1e-3 * dx.abs().max()
