@@ -134,6 +134,8 @@ struct BwdPlan {
   PackPlan pack;
   size_t lse_c, dxc;  // lse of the packed rows; packed dx before it is moved to its place (only for a dx of >= 2 GiB)
   bool stage_dx;
+  bool pack_on;   // tokens with an ignored label are packed away in this backward
+  bool parts_on;  // tail tiles of dx / dW may be split along K (partial-sum blocks exist)
   int64_t lddxc;
   size_t dz, dx_acc, dx_part, dw_part, w16, total;
 };
@@ -156,34 +158,39 @@ size_t dw_part_bytes(size_t Np, size_t Hp, int64_t vs, int64_t last_vs) {
 // N_chunk_size does not translate into a larger footprint.
 //
 // The bound is n_chunk * V * 4 bytes, what the reference spends on its logits
-// chunk (ops.py:700).  Shapes with a small vocabulary and many tokens cannot
-// meet it (the fp32 running dx alone is larger, and a split into very narrow
-// slabs leaves the GPU idle); for those the bound is widened by N * H * 4 bytes,
-// the fp32 x_grad buffer the reference allocates next to its logits chunk
-// (ops.py:693) and this library does not -- and by the split-K partial sums.  If even that fails, the narrowest
-// split is used: the bound is a target, the operator never refuses a shape.
+// chunk (ops.py:700).  Everything counts towards it: the dz stage, the fp32 running dx, the packed rows and
+// the partial sums of split tail tiles.  When that leaves only narrow slabs (under 8192 columns: few dW
+// tiles per launch), the two optional items are given up first if that buys wider slabs -- `lean`: tokens
+// with an ignored label are then not packed away in the backward and tail tiles are not split.
+// Shapes with a small vocabulary and many tokens cannot meet the bound at all (the fp32 running dx alone is
+// larger, and a split into very narrow slabs leaves the GPU idle); for those the bound is widened by
+// N * H * 4 bytes, the fp32 x_grad buffer the reference allocates next to its logits chunk (ops.py:693) and
+// this library does not -- and by the split-K partial sums.  If even that fails, the narrowest split is used:
+// the bound is a target, the operator never refuses a shape.
 int plan_bwd(const lce_problem* p, BwdPlan* b) {
   const size_t strict = (size_t)p->n_chunk * (size_t)p->V * 4;
   const size_t dz_cap = (size_t)1 << 30;
   const size_t Np = (size_t)lce::padded_tokens(p->N), Hp = (size_t)lce::padded_hidden(p->H);
   const int64_t Vp = lce::padded_vocab(p->V);
   const int64_t cols = Vp / 256;
-  // buffers of the packed rows come first and count towards the bound
-  const bool pack = packs_rows(p);
-  b->pack = plan_pack(p, 0, true);
   const bool split = splits(p);
+  const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
+  b->pack = plan_pack(p, 0, true);
   b->lddxc = lce::pad_to(p->H, 8);
   b->lse_c = b->pack.end;
   b->dxc = b->lse_c + align_up((size_t)p->N * 4);
-  size_t fixed = 0;  // (fp32 activations need the packed copy of x even when rows are not packed)
-  // The dx kernels store packed rows straight to their tokens' places through 32-bit offsets into dx; a dx
-  // that large offsets cannot span is staged packed and moved afterwards.
-  const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
-  b->stage_dx = pack && (size_t)p->N * (size_t)p->lddx * dxes >= ((size_t)1 << 31);
-  if (pack) fixed = b->dxc + (b->stage_dx ? align_up((size_t)p->N * (size_t)b->lddxc * dxes) : 0);
-  else if (p->x_dtype == LCE_F32) fixed = b->pack.end;
-  for (int pass = 0; pass < 2; ++pass) {
-    const size_t budget = strict + (pass ? (size_t)p->N * (size_t)p->H * 4 : 0);
+
+  // mode 0: everything; mode 1: lean (at the strict bound only); mode 2: everything, widened bound
+  auto fits = [&](int mode, BwdPlan* out) -> bool {
+    const bool lean = mode == 1;
+    const bool pack = packs_rows(p) && !(lean && p->pack_rows == LCE_PACK_AUTO);
+    // The dx kernels store packed rows straight to their tokens' places through 32-bit offsets into dx; a dx
+    // that large offsets cannot span is staged packed and moved afterwards.
+    const bool stage_dx = pack && (size_t)p->N * (size_t)p->lddx * dxes >= ((size_t)1 << 31);
+    size_t fixed = 0;  // buffers of the packed rows come first (fp32 activations need the copies of x even when rows are not packed)
+    if (pack) fixed = b->dxc + (stage_dx ? align_up((size_t)p->N * (size_t)b->lddxc * dxes) : 0);
+    else if (split) fixed = b->pack.end;
+    const size_t budget = strict + (mode == 2 ? (size_t)p->N * (size_t)p->H * 4 : 0);
     for (int64_t s = 1; s <= cols; ++s) {
       const int64_t vs = (cols + s - 1) / s * 256;
       if (s > 1 && (cols + s - 2) / (s - 1) * 256 == vs) continue;  // same width as with one slab fewer
@@ -192,25 +199,39 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
       const size_t dz = align_up(Np * (size_t)vs * 2 * (split ? 3 : 1));
       const size_t acc = slabs > 1 || split ? align_up(Np * Hp * 4) : 0;
       const int64_t last_vs = Vp - (slabs - 1) * vs;  // padded width of the last slab
-      const size_t dxp = dx_part_bytes(Np, Hp, vs, last_vs), dwp = dw_part_bytes(split ? 3 * Np : Np, Hp, vs, last_vs);  // at most 64 MiB each
+      const size_t dxp = lean ? 0 : dx_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
+      const size_t dwp = lean ? 0 : dw_part_bytes(split ? 3 * Np : Np, Hp, vs, last_vs);
       const size_t part = dxp + dwp;
       const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2 * (split ? 3 : 1)) : 0;  // 16-bit copy of the slab of W
-      // the widened bound of the second pass is for the staging proper; the split-K partial sums
-      // (at most 64 MiB each for dx and dW) and the packed rows come on top of it there
-      const size_t counted = dz + acc + w16 + (pass == 0 ? fixed + part : 0);
-      if ((counted <= budget && (dz <= dz_cap || vs == 256)) || (pass == 1 && vs == 256)) {
-        b->slabs = slabs;
-        b->vs = vs;
-        b->dz = fixed;
-        b->dx_acc = fixed + dz;
-        b->dx_part = fixed + dz + acc;
-        b->dw_part = fixed + dz + acc + dxp;
-        b->w16 = fixed + dz + acc + part;
-        b->total = fixed + dz + acc + part + w16;
-        return LCE_OK;
+      // the widened bound is for the staging proper; the split-K partial sums (at most 64 MiB each for dx
+      // and dW) and the packed rows come on top of it there
+      // (reserve: what the caller holds besides the workspace between forward and backward -- lse and a few scalars)
+      const size_t reserve = align_up((size_t)p->N * 4) + 4096;
+      const size_t counted = dz + acc + w16 + (mode != 2 ? fixed + part + reserve : 0);
+      if ((counted <= budget && (dz <= dz_cap || vs == 256)) || (mode == 2 && vs == 256)) {
+        out->slabs = slabs;
+        out->vs = vs;
+        out->pack_on = pack;
+        out->parts_on = !lean;
+        out->stage_dx = stage_dx;
+        out->dz = fixed;
+        out->dx_acc = fixed + dz;
+        out->dx_part = fixed + dz + acc;
+        out->dw_part = fixed + dz + acc + dxp;
+        out->w16 = fixed + dz + acc + part;
+        out->total = fixed + dz + acc + part + w16;
+        return true;
       }
     }
-  }
+    return false;
+  };
+  BwdPlan full = *b, lean = *b;
+  const bool ok_full = fits(0, &full);
+  if (ok_full && (full.vs >= 8192 || full.slabs == 1)) { *b = full; return LCE_OK; }
+  const bool ok_lean = fits(1, &lean);
+  if (ok_lean && (!ok_full || lean.vs > full.vs)) { *b = lean; return LCE_OK; }
+  if (ok_full) { *b = full; return LCE_OK; }
+  if (fits(2, b)) return LCE_OK;
   return LCE_EWORKSPACE;
 }
 
@@ -439,15 +460,15 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.dx = dx; a.dw = dw;
   a.dz = base + b.dz;
   a.dx_acc = b.slabs > 1 || splits(p) ? (float*)(base + b.dx_acc) : nullptr;
-  a.dx_part = (float*)(base + b.dx_part);
-  a.dw_part = (float*)(base + b.dw_part);
+  a.dx_part = b.parts_on ? (float*)(base + b.dx_part) : nullptr;
+  a.dw_part = b.parts_on ? (float*)(base + b.dw_part) : nullptr;
   rc = current_num_cus(&a.num_cus);
   if (rc != LCE_OK) return rc;
   const int ph = p->phases ? p->phases : ~0;
 
   // Tokens with an ignored label have dz == 0: the kernels run on the other rows only, packed to the front.
   const PackPlan& k = b.pack;
-  const bool pack = packs_rows(p), x32 = p->x_dtype == LCE_F32;
+  const bool pack = b.pack_on, x32 = p->x_dtype == LCE_F32;
   const int64_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
   a.xc = base + k.xc;
   a.ldxc = k.ldxc;

@@ -92,7 +92,7 @@ LCE_DEV DwPlan dw_plan(const BwdArgs& a, int64_t rows) {
   p.full = p.tiles / G * G;
   const int r = p.tiles - p.full, cap = G < kTailBlocks ? G : kTailBlocks;
   int s = 1;
-  if (r > 0)
+  if (r > 0 && a.dw_part != nullptr)  // (no blocks for partial sums: nothing is split)
     while (r * s * 2 <= cap && p.kt / (s * 2) >= 16) s *= 2;
   if (s == 1) {
     p.full = p.tiles;
@@ -208,7 +208,7 @@ template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s)
   hipLaunchKernelGGL(kern, dim3(a.dw_grid), dim3(kThreads), kMainloopLds, s, a);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  if (dw_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // this launch cannot have a split tail
+  if (a.dw_part == nullptr || dw_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // this launch cannot have a split tail
   // (the tile count does not depend on the rows: no second kernel when the last round is not split)
   if (!has_split_tail((a.vs / kTile) * (a.Hp / kTile), a.dw_grid)) return hipSuccess;
   // at most dw_grid / 2 tail tiles can be split (two segments each)

@@ -103,7 +103,7 @@ LCE_DEV DxPlan dx_plan(const BwdArgs& a, int tiles) {
   p.full = tiles / G * G;
   const int r = tiles - p.full, cap = G < kTailBlocks ? G : kTailBlocks;
   int s = 1;
-  if (r > 0)
+  if (r > 0 && a.dx_part != nullptr)  // (no blocks for partial sums: nothing is split)
     while (r * s * 2 <= cap && kt / (s * 2) >= 16) s *= 2;
   if (s == 1) {
     p.full = tiles;
@@ -239,7 +239,7 @@ template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s)
   const bool exact_k = a.vw == a.vs && dx_segments_exact(a.vs);
   hipError_t e = exact_k ? launch_tiles<T, false>(a, s) : launch_tiles<T, true>(a, s);
   if (e != hipSuccess) return e;
-  if (dx_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // no shape of this launch can have a split tail
+  if (a.dx_part == nullptr || dx_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // no shape of this launch can have a split tail
   // without packed rows the tile count is known here: no second kernel when its last round is not split
   if (a.n_rows == nullptr && !has_split_tail((a.Np / kTile) * (a.Hp / kTile), a.dx_grid)) return hipSuccess;
   // at most dx_grid / 2 tail tiles can be split (two segments each)

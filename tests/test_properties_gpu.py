@@ -202,7 +202,10 @@ def test_n_chunk_size_only_changes_scratch_not_results():
         assert torch.equal(got[0][0], ref[0][0])
         # dx is summed over vocabulary slabs in fp32, so a different slab count may move the last bit
         assert rel_errors(got[1], ref[1])[0] < 1e-2
-        assert torch.equal(got[2], ref[2])  # dW never depends on the slab split
+        # dW: a tile's sum over the tokens is cut into segments when its slab has few tiles, and a tight bound
+        # can switch that (and the packing of ignored tokens) off: the order of an fp32 sum, one bf16 rounding
+        emax, el2 = rel_errors(got[2], ref[2])
+        assert emax < 1e-2 and el2 < 2e-3
 
 
 def test_module_api_3d_input_monitoring_and_no_grad():
@@ -596,14 +599,14 @@ def test_autocast_follows_a_16_bit_weight_and_mismatched_dtypes_are_named():
 
 
 def test_function_and_registered_operator_agree_bitwise():
-    from linear_cross_entropy_loss_amd import LinearXentImplementation, linear_cross_entropy
+    from linear_cross_entropy_loss_amd import LinearXentImplementation, linear_cross_entropy, ops
 
     print("Function vs operator", flush=True)
     x, y, w = make_inputs(777, 264, 10008, torch.float16, seed=10, ignore_frac=0.1, device="cuda")
     res = []
 
     def via_operator(x, y, w, *cfg):  # what linear_cross_entropy calls while torch.compile traces
-        return torch.ops.lce_amd.forward(x, y, w, *cfg)[0].unbind(0)
+        return torch.ops.lce_amd.forward(x, y, w, *cfg, ops.pack_rows.get())[0].unbind(0)
 
     for fn in (LinearXentImplementation.apply, linear_cross_entropy, via_operator):
         xi = x.clone().requires_grad_(True)
