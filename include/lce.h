@@ -83,7 +83,7 @@ typedef struct lce_problem {
   int32_t monitoring;   /* 0/1: also produce max / entropy / norm (ops.py:678) */
   int32_t phases;       /* 0 = everything; otherwise a mask of LCE_PHASE_* (profiling aid) */
   int32_t pack_rows;    /* LCE_PACK_AUTO | LCE_PACK_ALWAYS | LCE_PACK_NEVER: see below        */
-  int32_t reserved;     /* 0                                                                  */
+  int32_t max_workgroups; /* profiling aid: cap on the persistent workgroups of the tile kernels (0 = one per compute unit) */
 } lce_problem;
 
 /*

@@ -53,7 +53,7 @@ class LceProblem(ctypes.Structure):
         ("monitoring", ctypes.c_int32),
         ("phases", ctypes.c_int32),
         ("pack_rows", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("max_workgroups", ctypes.c_int32),
     ]
 
 
@@ -120,13 +120,14 @@ def raise_for_status(rc: int, what: str) -> None:
 
 
 def make_problem(N, H, V, ldx, ldw, lddx, lddw, x_dtype, w_dtype, dx_dtype, dw_dtype, ignore_index,
-                 logit_scale, z_reg, n_chunk, monitoring, phases=0, pack_rows=0) -> LceProblem:
+                 logit_scale, z_reg, n_chunk, monitoring, phases=0, pack_rows=0, max_workgroups=0) -> LceProblem:
     return LceProblem(
         N=N, H=H, V=V, ldx=ldx, ldw=ldw, lddx=lddx, lddw=lddw,
         x_dtype=dtype_code(x_dtype), w_dtype=dtype_code(w_dtype),
         dx_dtype=dtype_code(dx_dtype), dw_dtype=dtype_code(dw_dtype),
         ignore_index=int(ignore_index), logit_scale=float(logit_scale), z_reg=float(z_reg),
         n_chunk=int(n_chunk), monitoring=1 if monitoring else 0, phases=int(phases), pack_rows=int(pack_rows),
+        max_workgroups=int(max_workgroups),
     )
 
 

@@ -16,6 +16,10 @@ LIB_NAME = "liblce_gfx950.so"
 LIB_PATH = PKG_DIR / LIB_NAME
 
 SOURCES = ["lce_api.hip", "lce_fwd.hip", "lce_bwd_dz.hip", "lce_bwd_dx.hip", "lce_bwd_dw.hip", "lce_convert.hip", "lce_compact.hip"]
+# Measurement probes (`bench.py --probe`): a library of their own, so that the operator's library holds the operator only.
+PROBE_LIB_NAME = "liblce_probe_gfx950.so"
+PROBE_LIB_PATH = PKG_DIR / PROBE_LIB_NAME
+PROBE_SOURCES = ["lce_probe.hip"]
 
 # Packed-fp32 VALU forms are disabled for all device code.
 HIPCC_FLAGS = [
@@ -38,6 +42,8 @@ def _hipcc() -> str:
 def _compile(src: str, objdir: Path) -> Path:
     obj = objdir / (src + ".o")
     extra = os.environ.get("LCE_EXTRA_HIPCC_FLAGS", "").split()
+    if src in PROBE_SOURCES:
+        extra = extra + ["-munsafe-fp-atomics"]  # the flush probe measures hardware fp32 atomic adds
     cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -51,17 +57,18 @@ def build(force: bool = True, verbose: bool = False) -> Path:
         return LIB_PATH
     objdir = PKG_DIR / "build"
     objdir.mkdir(exist_ok=True)
-    jobs = min(len(SOURCES), int(os.environ.get("MAX_JOBS", "8")))
+    jobs = min(len(SOURCES) + len(PROBE_SOURCES), int(os.environ.get("MAX_JOBS", "8")))
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, objdir), SOURCES))
-    tmp = LIB_PATH.with_suffix(".so.tmp")
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"link failed:\n{r.stderr}")
-    os.replace(tmp, LIB_PATH)
-    if verbose:
-        print(f"built {LIB_PATH}")
+        all_objs = list(ex.map(lambda s: _compile(s, objdir), SOURCES + PROBE_SOURCES))
+    for path, objs in ((LIB_PATH, all_objs[:len(SOURCES)]), (PROBE_LIB_PATH, all_objs[len(SOURCES):])):
+        tmp = path.with_suffix(".so.tmp")
+        cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"link failed:\n{r.stderr}")
+        os.replace(tmp, path)
+        if verbose:
+            print(f"built {path}")
     return LIB_PATH
 
 

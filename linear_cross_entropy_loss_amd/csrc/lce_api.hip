@@ -34,6 +34,7 @@ int check(const lce_problem* p, bool backward) {
   if (!ok) return LCE_EINVAL_DTYPE;
   if (!(p->logit_scale > 0.f) || !(p->z_reg >= 0.f)) return LCE_EINVAL_ARG;
   if (p->pack_rows != LCE_PACK_AUTO && p->pack_rows != LCE_PACK_ALWAYS && p->pack_rows != LCE_PACK_NEVER) return LCE_EINVAL_ARG;
+  if (p->max_workgroups < 0) return LCE_EINVAL_ARG;
   const int64_t xa = xd == LCE_F32 ? 4 : 8, wa = wd == LCE_F32 ? 4 : 8;  // 16-byte rows
   if (p->ldx < p->H || p->ldx % xa || p->ldw < p->V || p->ldw % wa) return LCE_EINVAL_ARG;
   // The kernels address a 256-row tile of x, of a 16-bit W and of dx with 32-bit byte offsets: 256 rows must
@@ -261,13 +262,14 @@ int static_scratch(void** out) {
   return LCE_OK;
 }
 
-// Compute units of the current device (grid size of the persistent kernels).
-int current_num_cus(int* out) {
+// Compute units of the current device (grid size of the persistent kernels), capped by `cap` when that is positive.
+int current_num_cus(int* out, int cap) {
   int dev = 0, n = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e == hipSuccess) e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
   if (e != hipSuccess) return hip_fail(e, "device query");
   *out = n > 0 ? n : 1;
+  if (cap > 0 && cap < *out) *out = cap;
   return LCE_OK;
 }
 
@@ -298,7 +300,7 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
   a.part_sq = (float*)(base + f.part_sq);
   a.tgt = (float*)(base + f.tgt);
   a.blk = (float*)(base + f.blk);
-  rc = current_num_cus(&a.num_cus);
+  rc = current_num_cus(&a.num_cus, p->max_workgroups);
   if (rc != LCE_OK) return rc;
 
   const int ph = p->phases ? p->phases : ~0;
@@ -462,7 +464,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.dx_acc = b.slabs > 1 || splits(p) ? (float*)(base + b.dx_acc) : nullptr;
   a.dx_part = b.parts_on ? (float*)(base + b.dx_part) : nullptr;
   a.dw_part = b.parts_on ? (float*)(base + b.dw_part) : nullptr;
-  rc = current_num_cus(&a.num_cus);
+  rc = current_num_cus(&a.num_cus, p->max_workgroups);
   if (rc != LCE_OK) return rc;
   const int ph = p->phases ? p->phases : ~0;
 

@@ -1,0 +1,122 @@
+// Measurement probes (liblce_probe_gfx950.so; not part of the operator, loaded only by `bench.py --probe`).
+//
+//   lce_probe_mfma    what the matrix pipes of this part sustain with no data movement at all: every wave
+//                     keeps 4 A and 4 B fragments in registers and issues v_mfma_f32_32x32x16_bf16 over a
+//                     4 x 4 grid of accumulator blocks (the 128 x 128 wave tile of the operator's kernels),
+//                     on constant or on random operands.  The ceiling the tile kernels are measured against.
+//   lce_probe_flush   what adding 256 x 256 fp32 blocks of partial sums into a matrix in memory costs, with
+//                     atomics or as plain read-modify-write: the traffic a backward that fed dz straight into
+//                     the dx and dW contractions would generate once per dz tile (its H-wide accumulators do
+//                     not fit a compute unit, so each dz tile's contribution would have to be flushed).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+__device__ __forceinline__ unsigned hash32(unsigned x) {
+  x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+  return x;
+}
+
+// A bf16 with random sign and mantissa and an exponent in [2^-2, 2^1): every operand bit toggles from one
+// fragment to the next, as with real activations and weights.
+__device__ __forceinline__ short random_bf16(unsigned seed) {
+  const unsigned h = hash32(seed);
+  const unsigned exp = 125u + (h >> 8 & 3u);
+  return (short)((h & 0x8000u) | (exp << 7) | (h & 0x7fu));
+}
+
+// pattern 0: all operands 1.0 (no bit toggles between consecutive instructions); 1: random operands, a different
+// (A, B) fragment pair in each of the 16 MFMAs of a step -- what the operator's kernels issue between LDS reads.
+__global__ __launch_bounds__(256) void mfma_loop_kernel(int pattern, int iters, float* out) {
+  s16x8_t a[4], b[4];
+  const unsigned tid = blockIdx.x * 256u + threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      a[i][e] = pattern == 0 ? (short)0x3f80 : random_bf16(tid * 64u + i * 8u + e);
+      b[i][e] = pattern == 0 ? (short)0x3f80 : random_bf16(tid * 64u + 32u + i * 8u + e);
+    }
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[i]),
+                                                            __builtin_bit_cast(bf16x8_t, b[j]), acc[i][j], 0, 0, 0);
+    asm volatile("" ::: "memory");
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s += acc[i][j][r];
+  out[tid] = s;
+}
+
+// Each workgroup adds `tiles` blocks of 256 x 256 floats into dst[rows][ld]: it walks down the row tiles of
+// column tile b / 4, then of the next one, so that (as in a tile order that shares operand bands between
+// neighbouring workgroups) four workgroups add into the same block at about the same time -- the pattern
+// of four token tiles of one vocabulary tile flushing their contributions to dW.
+template <bool ATOMIC>
+__global__ __launch_bounds__(256) void flush_kernel(float* dst, int64_t rows, int64_t ld, int tiles) {
+  const int col_tiles = (int)(ld / 256), row_tiles = (int)(rows / 256);
+  const int lane_col = (threadIdx.x & 63) * 4, row0 = threadIdx.x >> 6;
+  for (int k = 0; k < tiles; ++k) {
+    const int ct = ((int)blockIdx.x / 4 + k / row_tiles) % col_tiles, rt = k % row_tiles;
+    float* base = dst + (int64_t)rt * 256 * ld + (int64_t)ct * 256;
+    for (int r = row0; r < 256; r += 4) {
+      float* p = base + (int64_t)r * ld + lane_col;
+      if (ATOMIC) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) atomicAdd(p + e, 1.0f);
+      } else {
+        f32x4_t v = *reinterpret_cast<f32x4_t*>(p);
+        v += 1.0f;
+        *reinterpret_cast<f32x4_t*>(p) = v;
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+// Launches `wgs` workgroups of 4 waves, each wave issuing iters * 16 MFMAs (32 x 32 x 16, bf16).
+// out: wgs * 256 floats.  FLOPs = wgs * 4 * iters * 16 * 32768.
+int lce_probe_mfma(int pattern, int wgs, int iters, float* out, void* stream) {
+  if (pattern < 0 || pattern > 1 || wgs <= 0 || iters <= 0 || !out) return -3;
+  hipLaunchKernelGGL(mfma_loop_kernel, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, pattern, iters, out);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+// Launches `wgs` workgroups, each adding `tiles` blocks of 256 x 256 floats into dst[rows][ld] (rows and ld
+// multiples of 256).  atomic != 0: one fp32 atomic add per element; else 16-byte loads and stores.
+// Payload = wgs * tiles * 256 KiB.
+int lce_probe_flush(int atomic, float* dst, int64_t rows, int64_t ld, int tiles, int wgs, void* stream) {
+  if (!dst || rows < 256 || ld < 256 || rows % 256 || ld % 256 || tiles <= 0 || wgs <= 0) return -3;
+  if (atomic) {
+    hipLaunchKernelGGL(flush_kernel<true>, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, dst, rows, ld, tiles);
+  } else {
+    hipLaunchKernelGGL(flush_kernel<false>, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, dst, rows, ld, tiles);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+}  // extern "C"
