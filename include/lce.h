@@ -148,10 +148,11 @@ int lce_check_problem(const lce_problem* p);
 
 /*
  * Scratch sizes in bytes for lce_forward and lce_backward on problem `p`.
- * The forward size does not depend on n_chunk: V/32 bytes of partial sums per
- * token (four times that with monitoring), plus a 16-bit copy of at most
- * 256 MiB of an fp32 weight, plus -- when tokens are packed or x is fp32 -- a
- * packed copy of x.
+ * The forward works through the tokens in chunks of max(n_chunk, 16384) rows
+ * (65536 under an fp32 weight): V/32 bytes of partial sums per token of one
+ * chunk (four times that with monitoring), plus a 16-bit copy of at most
+ * 256 MiB of an fp32 weight, plus 12 bytes per token, plus -- when tokens are
+ * packed or x is fp32 -- a packed copy of x.
  * The backward size stays within n_chunk * V * 4 bytes -- the memory bound the
  * reference documents for N_chunk_size (ops.py:677, 700, 860) -- whenever the
  * narrowest split (256-column slabs plus an fp32 running dx) fits in it; for

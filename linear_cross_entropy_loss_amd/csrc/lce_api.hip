@@ -96,7 +96,19 @@ struct FwdPlan {
   // reach the tile kernels through the packed copy (rounded to bf16 there).
   PackPlan pack;
   int64_t vs;  // columns per forward launch: all of V, or the width of the 16-bit slab copy of an fp32 weight
+  int64_t nc;  // token rows per forward launch (a multiple of 256): the width of the partial-sum buffers
 };
+
+// The forward works through the tokens in chunks, so that its partial sums (V/32 bytes per token of a chunk)
+// do not grow with the number of tokens: chunks of n_chunk rows, but at least 16384 -- shorter chunks only
+// add launches -- and at least 65536 under an fp32 weight, whose 16-bit slab copies are made once per chunk.
+int64_t fwd_chunk_rows(const lce_problem* p) {
+  const int64_t Np = lce::padded_tokens(p->N);
+  int64_t nc = lce::pad_to(p->n_chunk, 256);
+  const int64_t least = p->w_dtype == LCE_F32 ? 65536 : 16384;
+  if (nc < least) nc = least;
+  return nc < Np ? nc : Np;
+}
 
 // 16-bit type the kernels compute in: that of the activations (bf16 for fp32 activations).
 int compute_dtype(const lce_problem* p) { return p->x_dtype == LCE_F16 ? LCE_F16 : LCE_BF16; }
@@ -104,7 +116,8 @@ int compute_dtype(const lce_problem* p) { return p->x_dtype == LCE_F16 ? LCE_F16
 FwdPlan plan_fwd(const lce_problem* p) {
   FwdPlan f;
   const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V);
-  const size_t part = align_up(Vp / lce::kChunkV * Np * 4);
+  f.nc = fwd_chunk_rows(p);
+  const size_t part = align_up(Vp / lce::kChunkV * (size_t)f.nc * 4);
   size_t o = 0;
   f.part_lse = o; o += part;
   f.part_max = o; if (p->monitoring) o += part;
@@ -336,28 +349,38 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
       a.H = 3 * p->H;
     }
   }
-  if (ph & LCE_PHASE_FWD_TILES) {
-    // One launch over the whole vocabulary, or -- fp32 weight -- one per slab, each on a
-    // 16-bit copy of its columns made just before it (same stream, one buffer).
-    for (int64_t v0 = 0; v0 < p->V; v0 += f.vs) {
-      a.v0 = v0;
-      a.vw = p->V - v0 < f.vs ? p->V - v0 : f.vs;
-      if (p->w_dtype == LCE_F32) {
-        const int64_t ld16 = lce::pad_to(a.vw, 256);
-        e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, v0, a.vw, base + f.w16, ld16, compute_dtype(p),
-                                       splits(p), s);
-        if (e != hipSuccess) return hip_fail(e, "convert_w");
-        a.w = base + f.w16; a.ldw = ld16; a.w_dtype = compute_dtype(p); a.wv0 = v0; a.Vw = a.vw;
-      } else {
-        a.wv0 = 0; a.Vw = p->V;
+  // The tokens go through in chunks of f.nc rows (one chunk at the benchmark shapes): tile kernels, then the row
+  // merge of that chunk, on partial-sum buffers that are one chunk wide.
+  a.nc = f.nc;
+  for (a.row0 = 0; a.row0 < a.Np; a.row0 += f.nc) {
+    if (ph & LCE_PHASE_FWD_TILES) {
+      // One launch over the whole vocabulary, or -- fp32 weight -- one per slab, each on a
+      // 16-bit copy of its columns made just before it (same stream, one buffer).
+      for (int64_t v0 = 0; v0 < p->V; v0 += f.vs) {
+        lce::FwdArgs t = a;
+        t.v0 = v0;
+        t.vw = p->V - v0 < f.vs ? p->V - v0 : f.vs;
+        if (p->w_dtype == LCE_F32) {
+          const int64_t ld16 = lce::pad_to(t.vw, 256);
+          e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, v0, t.vw, base + f.w16, ld16, compute_dtype(p),
+                                         splits(p), s);
+          if (e != hipSuccess) return hip_fail(e, "convert_w");
+          t.w = base + f.w16; t.ldw = ld16; t.w_dtype = compute_dtype(p); t.wv0 = v0; t.Vw = t.vw;
+        } else {
+          t.wv0 = 0; t.Vw = p->V;
+        }
+        e = lce::launch_fwd_tiles(t, s);
+        if (e != hipSuccess) return hip_fail(e, "fwd_tiles");
       }
-      e = lce::launch_fwd_tiles(a, s);
-      if (e != hipSuccess) return hip_fail(e, "fwd_tiles");
+    }
+    if (ph & LCE_PHASE_FWD_REDUCE) {
+      e = lce::launch_fwd_rows(a, s);
+      if (e != hipSuccess) return hip_fail(e, "fwd_rows");
     }
   }
   if (ph & LCE_PHASE_FWD_REDUCE) {
-    e = lce::launch_fwd_reduce(a, s);
-    if (e != hipSuccess) return hip_fail(e, "fwd_reduce");
+    e = lce::launch_fwd_final(a, s);
+    if (e != hipSuccess) return hip_fail(e, "fwd_final");
   }
   return LCE_OK;
 }
@@ -366,7 +389,7 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
 
 extern "C" {
 
-int lce_version(void) { return 200; }  // 0.2.0: lce_problem gained pack_rows
+int lce_version(void) { return 300; }  // 0.3.0: lce_forward_static, lce_problem.max_workgroups, fp32 tensors as bf16 pairs
 
 const char* lce_strerror(int status) {
   switch (status) {

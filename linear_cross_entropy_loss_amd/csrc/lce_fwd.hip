@@ -37,7 +37,7 @@ LCE_DEV float fast_log(float v) { return __builtin_amdgcn_logf(v) * kLn2; }
 // the one run that V cuts through is handled element by element.
 template <class T, bool VTAIL>
 LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
-  const int64_t v0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
+  const int64_t v0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;  // t0: inside the chunk of rows of this launch
   const int tid = opaque_tid();
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
@@ -52,8 +52,9 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
   const int64_t slice = slice_v0 / kChunkV;
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-    const int64_t o = slice * a.Np + tok;
+    const int64_t tokl = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);  // row inside the chunk
+    const int64_t tok = a.row0 + tokl;
+    const int64_t o = slice * a.nc + tokl;
     if (VTAIL && vrem == 0) {  // nothing of this slice exists
       if (lane < 32) {
         a.part_lse[o] = -INFINITY;
@@ -169,7 +170,10 @@ template <class T, bool VTAIL, bool KMASK> struct FwdProblem {
     const bool packed = rows != a.N;
     x = reinterpret_cast<const E*>(packed ? a.xc : a.x);
     ldx = packed ? a.ldxc : a.ldx;
-    tiles_q = (int)((rows + kTile - 1) / kTile);
+    // rows of this launch's chunk that exist
+    int64_t here = rows - a.row0;
+    here = here < 0 ? 0 : (here > a.nc ? a.nc : here);
+    tiles_q = (int)((here + kTile - 1) / kTile);
   }
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void coords(int tile, int& tp, int& tq) const {
@@ -180,7 +184,7 @@ template <class T, bool VTAIL, bool KMASK> struct FwdProblem {
     int tp, tq;
     coords(tile, tp, tq);
     p = reinterpret_cast<const E*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
-    q = x + (int64_t)tq * kTile * ldx;
+    q = x + (a.row0 + (int64_t)tq * kTile) * ldx;
   }
   LCE_DEV const void* p_end() const { return matrix_end<E>(a.w, a.H, a.ldw, a.Vw); }
   LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
@@ -207,7 +211,8 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
   __shared__ float sh_pz[4][kMergeRows], sh_sq[4][kMergeRows], sh_mx[4][kMergeRows];
   __shared__ double sh_red[7][kMergeRows];
   const int r = threadIdx.x & 63, g = threadIdx.x >> 6;
-  const int64_t tok = (int64_t)blockIdx.x * kMergeRows + r;  // < Np; rows that do not exist only keep the block sums aligned
+  const int64_t tokl = (int64_t)blockIdx.x * kMergeRows + r;  // row inside the chunk of this launch
+  const int64_t tok = a.row0 + tokl;  // < Np; rows that do not exist only keep the block sums aligned
   const int64_t rows = a.n_rows ? packed_rows(a.n_rows, a.N) : a.N;
   const bool exists = tok < rows;
   // packed rows: lse goes back to the token's own place; tokens that were dropped get 0
@@ -223,7 +228,7 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int c = c0 + 4 * u;
-      l[u] = c < nslices ? a.part_lse[(int64_t)c * a.Np + tok] : -INFINITY;
+      l[u] = c < nslices ? a.part_lse[(int64_t)c * a.nc + tokl] : -INFINITY;
     }
     float mb = l[0];
 #pragma unroll
@@ -259,7 +264,7 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
       for (int u = 0; u < 8; ++u) {
         const int c = c0 + 4 * u;
         const bool in = c < nslices;
-        const int64_t o = (int64_t)(in ? c : 0) * a.Np + tok;
+        const int64_t o = (int64_t)(in ? c : 0) * a.nc + tokl;
         pl[u] = in ? a.part_lse[o] : -INFINITY;
         pp[u] = in ? a.part_pz[o] : 0.f;
         ps[u] = in ? a.part_sq[o] : 0.f;
@@ -304,7 +309,7 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
     const int q = threadIdx.x;
     double acc = sh_red[q][0];
     for (int i = 1; i < kMergeRows; ++i) acc = (q == 4) ? fmax(acc, sh_red[q][i]) : acc + sh_red[q][i];
-    reinterpret_cast<double*>(a.blk)[(int64_t)blockIdx.x * 8 + q] = acc;
+    reinterpret_cast<double*>(a.blk)[(a.row0 / kMergeRows + (int64_t)blockIdx.x) * 8 + q] = acc;
   }
 }
 
@@ -362,7 +367,8 @@ hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
 
 // All full tile columns of the vocabulary, then the column that straddles V.
 template <class T> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
-  const int64_t tq = a.Np / kTile, full = a.vw / kTile;
+  const int64_t left = a.Np - a.row0;  // token tiles of this chunk at most
+  const int64_t tq = (left < a.nc ? left : a.nc) / kTile, full = a.vw / kTile;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
     hipError_t e = exact_k ? launch_one<T, false, false>(a, full * tq, s)
@@ -382,10 +388,13 @@ hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s) {
-  hipLaunchKernelGGL(fwd_rows_kernel, dim3((unsigned)(a.Np / kMergeRows)), dim3(256), 0, s, a);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
+hipError_t launch_fwd_rows(const FwdArgs& a, hipStream_t s) {
+  const int64_t left = a.Np - a.row0;
+  hipLaunchKernelGGL(fwd_rows_kernel, dim3((unsigned)((left < a.nc ? left : a.nc) / kMergeRows)), dim3(256), 0, s, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_fwd_final(const FwdArgs& a, hipStream_t s) {
   hipLaunchKernelGGL(fwd_final_kernel, dim3(1), dim3(256), 0, s, a);
   return hipGetLastError();
 }

@@ -31,6 +31,9 @@ struct FwdArgs {
   const int64_t* y;
   int64_t N, H, V, ldx, ldw;
   int64_t Np, Vp;  // padded_tokens(N), padded_vocab(V)
+  // Token rows [row0, row0 + nc) covered by this launch (both multiples of 256): the forward works through the
+  // rows in chunks of nc, so that the per-slice partials below are nc rows wide however many tokens there are.
+  int64_t row0, nc;
   // Vocabulary columns [v0, v0 + vw) covered by this launch (v0 a multiple of 256), and the
   // window of W that the buffer `w` holds: columns [wv0, wv0 + Vw) of the weight, row stride ldw.
   // (`w` is the caller's matrix, wv0 = 0, Vw = V -- or a 16-bit copy of one slab of an fp32 weight.)
@@ -52,10 +55,10 @@ struct FwdArgs {
   float* lse;        // [N]
   float* out5;       // [5]
   int64_t* n_valid;  // [1]
-  float* part_lse;   // [Vp/128][Np]  per-slice logsumexp (-inf for a slice with no valid column)
-  float* part_max;   // [Vp/128][Np]  per-slice max            (monitoring)
-  float* part_pz;    // [Vp/128][Np]  per-slice sum softmax*z  (monitoring)
-  float* part_sq;    // [Vp/128][Np]  per-slice sum z^2        (monitoring)
+  float* part_lse;   // [Vp/128][nc]  per-slice logsumexp (-inf for a slice with no valid column), rows of the current chunk
+  float* part_max;   // [Vp/128][nc]  per-slice max            (monitoring)
+  float* part_pz;    // [Vp/128][nc]  per-slice sum softmax*z  (monitoring)
+  float* part_sq;    // [Vp/128][nc]  per-slice sum z^2        (monitoring)
   float* tgt;        // [Np]          target logit (written for tokens whose label is a column of W)
   float* blk;        // [Np/64][8]    per-merge-block partial sums
 };
@@ -117,7 +120,9 @@ __device__ __forceinline__ float final_factor_of(const BwdArgs& a, float unscale
 }
 
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s);
-hipError_t launch_fwd_reduce(const FwdArgs& a, hipStream_t s);
+// Row merge of the current chunk (lse, per-block sums), and -- once, after the last chunk -- the final reduction.
+hipError_t launch_fwd_rows(const FwdArgs& a, hipStream_t s);
+hipError_t launch_fwd_final(const FwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);

@@ -205,7 +205,30 @@ def test_fp32_weight_adds_one_16_bit_slab_copy_to_the_scratch():
     f32, b32 = _lib.workspace_bytes(p32)
     slabs, width = _lib.backward_plan(p32)
     assert b32 - b16 == H * width * 2 and b32 <= nc * V * 4
-    assert 0 < f32 - f16 <= 256 << 20
+    # forward: the slab copy (at most 256 MiB), and partial sums for chunks of 65536 tokens instead of 16384
+    # (the copies are made once per chunk of tokens, so chunks are longer under an fp32 weight)
+    assert f32 - f16 == (256 << 20) + (65536 - 16384) * (V // 128) * 4
+
+
+def test_forward_scratch_does_not_grow_with_the_partial_sums_of_all_tokens():
+    """The forward works through the tokens in chunks (of N_chunk_size rows, at least 16384), so its partial sums
+    are one chunk wide however many tokens there are; what still grows with N is 16 bytes per token of packing
+    state, 4 + 1/8 bytes of per-token results and, when tokens are packed, the packed copy of x."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    H, V = 2048, 131072
+    for mon in (False, True):
+        sizes = []
+        for N in (16384, 65536, 1 << 20):
+            p = _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=4096, monitoring=1 if mon else 0,
+                      pack_rows=_lib.PACK_NEVER)
+            sizes.append(_lib.workspace_bytes(p)[0])
+        part = (V // 128) * 16384 * 4 * (4 if mon else 1)
+        for N, f in zip((16384, 65536, 1 << 20), sizes):
+            assert part <= f <= part + N * 8 + 4096, (N, f)
+    # a larger N_chunk_size widens the chunks
+    p = _prob(N=1 << 20, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=65536, pack_rows=_lib.PACK_NEVER)
+    assert _lib.workspace_bytes(p)[0] >= (V // 128) * 65536 * 4
 
 
 def test_null_and_small_workspace_are_rejected_without_touching_the_gpu(lib):

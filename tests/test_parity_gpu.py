@@ -247,3 +247,52 @@ def test_randomized_shapes_and_options_match_oracle():
             emax, el2 = rel_errors(got, want)
             assert emax <= grad_tol and el2 <= grad_tol, (it, emax, el2)
         assert (dx.cpu()[y == -1] == 0).all(), it
+
+
+@pytest.mark.parametrize("mon", [False, True])
+def test_many_tokens_go_through_the_forward_in_chunks(mon):
+    """More tokens than one forward chunk holds (chunks of max(N_chunk_size, 16384) rows: here 16384 + 16384 +
+    7232, the last one not a multiple of the tile size): per-token lse, the loss, the monitoring values and both
+    gradients against the oracle, and lse of every kept token individually."""
+    from linear_cross_entropy_loss_amd import _lib, linear_cross_entropy
+    from oracle import lce_forward_backward_fp64
+
+    N, H, V = 40000, 72, 1000
+    print(f"chunked forward N={N} H={H} V={V} monitoring={mon}", flush=True)
+    x, y, w = make_inputs(N, H, V, torch.bfloat16, seed=77, ignore_frac=0.2, device="cuda")
+    y[N - 1] = V - 1
+    out, dx, dw = _run(x, y, w, -1, 1e-4, 1.0, 512, mon)
+    ref = lce_forward_backward_fp64(x, y, w, -1, 1e-4, 1.0, chunk=4096)
+    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item())
+    assert abs(out[1].item() - ref.z_reg.item()) <= LOSS_RTOL * abs(ref.z_reg.item())
+    if mon:
+        assert abs(out[2].item() - ref.logit_max.item()) <= 1e-3 * abs(ref.logit_max.item())
+        assert abs(out[3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item())
+        assert abs(out[4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item())
+    for got, want in ((dx, ref.dx), (dw, ref.dw)):
+        emax, el2 = rel_errors(got, want)
+        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (emax, el2)
+    assert (dx[y == -1] == 0).all()
+    # lse of every kept token, through the C ABI (the autograd path keeps it to itself)
+    import ctypes
+
+    from linear_cross_entropy_loss_amd import ops
+
+    lib = _lib.load()
+    p = _lib.make_problem(N, H, V, H, V, H, V, x.dtype, w.dtype, x.dtype, w.dtype, -1, 1.0, 1e-4, 512, mon, 0,
+                          ops.pack_rows.get())
+    fwd_b, _ = _lib.workspace_bytes(p)
+    assert fwd_b < (V // 128 + 1) * 16384 * 4 * (4 if mon else 1) + N * (H * 2 + 64)  # partials one chunk wide
+    ws = torch.empty(fwd_b, dtype=torch.uint8, device="cuda")
+    lse = torch.empty(N, device="cuda")
+    out5 = torch.empty(5, device="cuda")
+    nv = torch.empty(1, dtype=torch.int64, device="cuda")
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = lib.lce_forward(ctypes.byref(p), P(x), P(w), P(y), P(lse), P(out5), P(nv), P(ws), fwd_b,
+                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    keep = y != -1
+    assert nv.item() == int(keep.sum().item())
+    assert torch.allclose(lse[keep].double(), ref.lse[keep], rtol=2e-4, atol=2e-4)
+    assert torch.equal(out5[0], out[0])
