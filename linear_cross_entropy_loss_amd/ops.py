@@ -329,10 +329,10 @@ class LinearCrossEntropyLoss(torch.nn.Linear):
         z_regularization: weight of the ``mean(logsumexp(z)^2)`` penalty. Default 0.0.
         N_chunk_size: target for the scratch memory of the backward, ``N_chunk_size * out_features * 4`` bytes
             (what the reference spends on one chunk of logits); the backward works through the vocabulary in
-            as many slabs as that takes.  The number of rows of ``x`` is free, but two terms grow with it: the
-            forward's per-token partial sums (``out_features / 32`` bytes per token, four times that with
-            monitoring) and the backward's fp32 running sum of ``dx`` and packed copy of ``x``
-            (``6 * in_features`` bytes per token).  Default 4096.
+            as many slabs as that takes, and the forward through the tokens in chunks of
+            ``max(N_chunk_size, 16384)`` rows.  The number of rows of ``x`` is free; what grows with it is the
+            backward's fp32 running sum of ``dx`` and the packed copy of ``x`` (``6 * in_features`` bytes per
+            token).  Default 4096.
         init_method: optional callable applied to the weight instead of the default truncated normal.
 
     Set ``module.monitoring = True`` to also collect ``logit_norm``, ``logit_max``, ``logit_entropy`` and
