@@ -29,7 +29,12 @@
  *     the row length is not such a multiple, the elements between the end of a
  *     row and the next multiple ("stride padding") are read, must be finite,
  *     and never influence a result; the same positions of dx / dW rows may be
- *     written.
+ *     written.  Of the LAST row of x and w nothing is read past the 4-byte
+ *     word that holds its last element, so a matrix may end with that row's
+ *     elements (an allocation of (rows - 1) * ld + cols elements, rounded up to
+ *     4 bytes; with an odd row length the other half of that last word counts
+ *     as stride padding and must be finite).  dx and dw are written in pieces of up to 16 bytes and need
+ *     all rows * ld elements.
  *   - Every function returns LCE_OK (0) or a negative lce_status; nothing
  *     throws or aborts.
  */

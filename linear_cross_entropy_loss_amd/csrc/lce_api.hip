@@ -338,7 +338,7 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
       }
       e = x32 ? lce::launch_gather_rows_split((const float*)x, p->ldx, p->H, a.perm, a.n_rows, p->N, base + k.xc,
                                               k.ldxc, nullptr, 0, nullptr, nullptr, a.num_cus, s)
-              : lce::launch_gather_rows(x, p->ldx * 2, a.perm, a.n_rows, p->N, base + k.xc, k.ldxc * 2, nullptr, nullptr,
+              : lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, a.perm, a.n_rows, p->N, base + k.xc, k.ldxc * 2, nullptr, nullptr,
                                         a.num_cus, s);
       if (e != hipSuccess) return hip_fail(e, "gather_rows");
     }
@@ -516,7 +516,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     float* lse_c = pack ? (float*)(base + b.lse_c) : nullptr;
     e = x32 ? lce::launch_gather_rows_split((const float*)x, p->ldx, p->H, perm, a.n_rows, p->N, base + k.xc, k.ldxc,
                                             base + k.xk, k.ldxk, pack ? lse : nullptr, lse_c, a.num_cus, s)
-            : lce::launch_gather_rows(x, p->ldx * 2, perm, a.n_rows, p->N, base + k.xc, k.ldxc * 2, lse, lse_c,
+            : lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, perm, a.n_rows, p->N, base + k.xc, k.ldxc * 2, lse, lse_c,
                                       a.num_cus, s);
     if (e != hipSuccess) return hip_fail(e, "gather_rows");
   }

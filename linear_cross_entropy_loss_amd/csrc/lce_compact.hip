@@ -94,10 +94,12 @@ __global__ __launch_bounds__(256) void pack_kept_kernel(const int64_t* y, int64_
 }
 
 // One workgroup per packed row (grid-stride).  Rows are moved in 16-byte pieces; `chunks` pieces per row.
+// The last row of x may end with its last element (a caller's matrix need not own the stride padding of its
+// last row): of that row only the whole pieces are moved as such, the rest 16 bits at a time, zero-filled.
 __global__ __launch_bounds__(256) void gather_rows_kernel(const char* x, int64_t ldx_bytes, const int* perm,
                                                           const int64_t* n_rows, int64_t N, char* xc,
-                                                          int64_t ldxc_bytes, int chunks, const float* lse,
-                                                          float* lse_c) {
+                                                          int64_t ldxc_bytes, int chunks, int64_t row_bytes,
+                                                          const float* lse, float* lse_c) {
   const int64_t rows = packed_rows(n_rows, N);
   const bool copy_x = rows != N;
   for (int64_t j = blockIdx.x; j < rows; j += gridDim.x) {
@@ -106,7 +108,13 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const char* x, int64_t
     if (copy_x) {
       const u32x4_t* s = reinterpret_cast<const u32x4_t*>(x + src * ldx_bytes);
       u32x4_t* d = reinterpret_cast<u32x4_t*>(xc + j * ldxc_bytes);
-      for (int c = threadIdx.x; c < chunks; c += 256) d[c] = s[c];
+      const int whole = src == N - 1 ? (int)(row_bytes / 16) : chunks;
+      for (int c = threadIdx.x; c < whole; c += 256) d[c] = s[c];
+      if (whole < chunks && threadIdx.x < 8) {  // the piece that the end of the last row cuts through
+        const int64_t b = (int64_t)whole * 16 + threadIdx.x * 2;
+        const unsigned short v = b < row_bytes ? *reinterpret_cast<const unsigned short*>(x + src * ldx_bytes + b) : 0;
+        *reinterpret_cast<unsigned short*>(xc + j * ldxc_bytes + b) = v;
+      }
     }
   }
 }
@@ -210,12 +218,12 @@ hipError_t launch_gather_rows_split(const float* x, int64_t ldx, int64_t H, cons
   return hipGetLastError();
 }
 
-hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, const int* perm, const int64_t* n_rows, int64_t N,
-                              void* xc, int64_t ldxc_bytes, const float* lse, float* lse_c, int num_cus,
-                              hipStream_t s) {
+hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, int64_t row_bytes, const int* perm,
+                              const int64_t* n_rows, int64_t N, void* xc, int64_t ldxc_bytes, const float* lse,
+                              float* lse_c, int num_cus, hipStream_t s) {
   hipLaunchKernelGGL(gather_rows_kernel, dim3(row_grid(N, num_cus)), dim3(256), 0, s,
                      reinterpret_cast<const char*>(x), ldx_bytes, perm, n_rows, N, reinterpret_cast<char*>(xc),
-                     ldxc_bytes, (int)(ldxc_bytes / 16), lse, lse_c);
+                     ldxc_bytes, (int)(ldxc_bytes / 16), row_bytes, lse, lse_c);
   return hipGetLastError();
 }
 

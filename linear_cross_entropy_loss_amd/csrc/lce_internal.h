@@ -150,10 +150,11 @@ int64_t compact_segments(int64_t N);
 hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_index, int* cnt, int64_t* n_rows,
                                  int* perm, int64_t* yc, hipStream_t s);
 // xc[j] = x[perm[j]] for j < *n_rows, in 16-byte pieces of rows ldxc_bytes long (skipped when *n_rows == N);
+// row_bytes = bytes of a row that hold elements (nothing past them is read of the last row of x);
 // lse_c[j] = lse[perm[j]] when lse is not null (always).
-hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, const int* perm, const int64_t* n_rows, int64_t N,
-                              void* xc, int64_t ldxc_bytes, const float* lse, float* lse_c, int num_cus,
-                              hipStream_t s);
+hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, int64_t row_bytes, const int* perm,
+                              const int64_t* n_rows, int64_t N, void* xc, int64_t ldxc_bytes, const float* lse,
+                              float* lse_c, int num_cus, hipStream_t s);
 // fp32 activations: xc[j] = [hi | hi | lo] of x[perm[j]] as bf16 (3 H elements per row, row stride ldxc), and
 // -- xk not null -- the same three parts stacked along the tokens, xk[b * Np + j] (row stride ldxk, rows from
 // *n_rows to Np of each block zeroed).  Always made, also when no token is dropped; perm / n_rows may be null

@@ -190,6 +190,37 @@ def test_strided_inputs_and_garbage_in_the_stride_padding():
         assert torch.equal(a, b)
 
 
+def test_nothing_is_read_past_the_last_row_of_the_inputs():
+    """x and W whose memory ends with the last element of their last row (row length not a multiple of 8, so the
+    row stride has padding): what would be the stride padding of the LAST row lies outside the matrices and holds
+    NaN here.  The results must be those of the dense call, bit for bit, with and without packed rows."""
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    print("last row ends the matrix", flush=True)
+    N, H, V = 600, 100, 1004
+    x, y, w = make_inputs(N, H, V, torch.float16, seed=15, ignore_frac=0.25, device="cuda")
+    y[N - 1] = 3  # the last token is kept, so its row is gathered when rows are packed
+    ldx, ldw = 104, 1008
+    xbuf = torch.zeros(N * ldx, dtype=x.dtype, device="cuda")
+    wbuf = torch.zeros(H * ldw, dtype=w.dtype, device="cuda")
+    xs = xbuf.as_strided((N, H), (ldx, 1))
+    ws = wbuf.as_strided((H, V), (ldw, 1))
+    xs.copy_(x)
+    ws.copy_(w)
+    xbuf[(N - 1) * ldx + H:] = float("nan")
+    wbuf[(H - 1) * ldw + V:] = float("nan")
+    res = []
+    for xi, wi in ((x, w), (xs, ws)):
+        xi = xi.detach().requires_grad_(True)
+        wi = wi.detach().requires_grad_(True)
+        out = linear_cross_entropy(xi, y, wi, -1, 1e-4, 1.0, 256, True)
+        out[0].backward()
+        res.append((torch.stack(out).detach(), xi.grad.clone(), wi.grad.clone()))
+    assert torch.isfinite(res[1][0]).all()
+    for a, b in zip(res[0], res[1]):
+        assert torch.equal(a, b)
+
+
 def test_gpt2_vocabulary_matches_fp64_oracle_evaluated_on_gpu():
     """V = 50257 (not a multiple of 8), H = 768, N = 3000: oracle in fp64 on the GPU."""
     from linear_cross_entropy_loss_amd import linear_cross_entropy
