@@ -219,11 +219,15 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
       for (int b = 0; b < kNB; ++b) pf[buf][b] = pr.read(stage, b, ks);
     }
   }
+  // The accumulator blocks of a row are visited left to right in even rows and right to left in odd ones, so
+  // that consecutive matrix instructions always differ in exactly one operand (measured 0.1-0.3 % faster than
+  // restarting every row on the left, where both operands change at a row change).
   template <bool ZERO> LCE_DEV void mfma_rows(f32x16_t (&acc)[kNB][kNB], int buf, int i0, int i1) {
 #pragma unroll
     for (int i = i0; i < i1; ++i)
 #pragma unroll
-      for (int j = 0; j < kNB; ++j) {
+      for (int jj = 0; jj < kNB; ++jj) {
+        const int j = (i & 1) ? kNB - 1 - jj : jj;
         f32x16_t c;
         if (ZERO) {
 #pragma unroll
