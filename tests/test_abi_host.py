@@ -350,3 +350,21 @@ int main(void) {
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split(None, 5)
     assert int(out[0]) >= 100 and int(out[3]) == 4 and int(out[4]) == 32768
     assert int(out[2]) <= 4096 * 131072 * 4 and "workspace" in out[5]
+
+
+def test_library_imports_no_allocation_or_synchronisation_routine():
+    """The operator's library allocates nothing, frees nothing and never synchronises: its dynamic symbol table
+    imports no HIP routine that could (the whole list is device query, launch, error text and the symbol
+    lookup of the static scratch)."""
+    import subprocess
+
+    from linear_cross_entropy_loss_amd import _lib
+
+    out = subprocess.run(["nm", "-D", "--undefined-only", str(_lib.LIB_PATH)], capture_output=True, text=True, check=True)
+    hip = sorted({line.split()[-1].split("@")[0] for line in out.stdout.splitlines() if " hip" in line})
+    allowed = {"hipDeviceGetAttribute", "hipFuncSetAttribute", "hipGetDevice", "hipGetErrorString", "hipGetLastError",
+               "hipGetSymbolAddress", "hipLaunchKernel", "__hipRegisterFatBinary", "__hipRegisterFunction",
+               "__hipRegisterVar", "__hipUnregisterFatBinary", "__hipPushCallConfiguration", "__hipPopCallConfiguration"}
+    assert set(hip) <= allowed, set(hip) - allowed
+    for banned in ("Malloc", "Free", "Synchronize", "Memcpy", "Memset", "MemPool"):
+        assert not any(banned in name for name in hip), (banned, hip)
