@@ -242,13 +242,14 @@ def test_module_api_3d_input_monitoring_and_no_grad():
     assert x.grad is not None
 
 
-def test_gradient_of_one_input_alone_equals_that_of_the_full_call():
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_gradient_of_one_input_alone_equals_that_of_the_full_call(dtype):
     """dx without dW (frozen weight) and dW without dx (frozen activations) skip the other contraction and,
     with packed rows, the zeroing of dropped dx rows; what they return is bit-identical to the full call."""
     from linear_cross_entropy_loss_amd import linear_cross_entropy
 
     print("partial gradients", flush=True)
-    x, y, w = make_inputs(1300, 264, 5000, torch.float16, seed=77, ignore_frac=0.35, device="cuda")
+    x, y, w = make_inputs(1300, 264, 5000, dtype, seed=77, ignore_frac=0.35, device="cuda")
     _, dx_full, dw_full = _fb(x, y, w, z_reg=1e-4, scale=0.5, n_chunk=64)
     xo = x.clone().requires_grad_(True)
     linear_cross_entropy(xo, y, w, -1, 1e-4, 0.5, 64)[0].backward()
