@@ -368,3 +368,41 @@ def test_library_imports_no_allocation_or_synchronisation_routine():
     assert set(hip) <= allowed, set(hip) - allowed
     for banned in ("Malloc", "Free", "Synchronize", "Memcpy", "Memset", "MemPool"):
         assert not any(banned in name for name in hip), (banned, hip)
+
+
+def test_backward_plan_invariants_on_random_problems():
+    """Seeded random problems: the slabs cover the vocabulary, widths are tile multiples, the reported scratch
+    is what the bound allows whenever the narrowest split could meet it, a larger bound never means more
+    slabs, and forward scratch never depends on more than one chunk of tokens."""
+    import random
+
+    from linear_cross_entropy_loss_amd import _lib
+
+    rng = random.Random(7)
+    dts = (torch.bfloat16, torch.float16, torch.float32)
+    for it in range(300):
+        N = rng.choice([1, 100, 255, 256, 1000, 4096, 16384, 40000, 65536, 300000])
+        H = rng.choice([8, 64, 264, 768, 2048, 4096, 8192])
+        V = rng.choice([8, 1000, 4096, 32000, 50264, 131072, 262144])
+        nc = rng.choice([16, 512, 2048, 4096, 8192, 65536])
+        xd = rng.choice(dts)
+        wd = xd if xd == torch.float32 else rng.choice((xd, torch.float32))
+        pack = rng.choice((_lib.PACK_AUTO, _lib.PACK_ALWAYS, _lib.PACK_NEVER))
+        mk = lambda n: _prob(N=N, H=H, V=V, ldx=H, ldw=V, lddx=H, lddw=V, n_chunk=n, x_dtype=xd, w_dtype=wd,
+                             dx_dtype=xd, dw_dtype=wd, pack_rows=pack)
+        p = mk(nc)
+        fwd, bwd = _lib.workspace_bytes(p)
+        slabs, width = _lib.backward_plan(p)
+        Vp = -(-V // 256) * 256
+        assert width % 256 == 0 and 1 <= slabs and (slabs - 1) * width < Vp <= slabs * width, (it, slabs, width)
+        assert fwd > 0 and bwd > 0
+        # a larger bound never needs more slabs
+        slabs2, _ = _lib.backward_plan(mk(nc * 4))
+        assert slabs2 <= slabs, (it, slabs, slabs2)
+        # forward: partial sums of one chunk of tokens at most, whatever N
+        chunk = max(-(-nc // 256) * 256, 65536 if wd == torch.float32 and xd != torch.float32 or xd == torch.float32 else 16384)
+        Np = -(-N // 256) * 256
+        part = (Vp // 128) * min(Np, chunk) * 4
+        split = 3 if xd == torch.float32 else 1
+        slab_copy = (256 << 20) + 256 * H * 2 * split if wd == torch.float32 else 0
+        assert fwd <= part + Np * 16 + N * (split * H + 8) * 2 + slab_copy + N * 16 + 8192, (it, fwd)
