@@ -25,6 +25,7 @@ CASES = [
     dict(name="bf16_ignore_zreg", N=512, H=256, V=4096, dtype="bfloat16", seed=102, ignore_frac=0.1, z_reg=1e-4, scale=1.0),
     dict(name="f16_scale_half", N=512, H=256, V=4096, dtype="float16", seed=103, ignore_frac=0.1, z_reg=1e-4, scale=0.5),
     dict(name="f16_zipf", N=1024, H=256, V=8192, dtype="float16", seed=104, ignore_frac=0.1, z_reg=0.0, scale=1.0, zipf=True),
+    dict(name="f32_ignore_zreg", N=512, H=264, V=4104, dtype="float32", seed=105, ignore_frac=0.1, z_reg=1e-4, scale=1.0),
 ]
 PROBES = [(0, 0), (1, 7), (17, 100), (255, 255), (100, 3)]
 

@@ -52,17 +52,20 @@ def test_hip_path_matches_golden(name):
     out = linear_cross_entropy(xd, y.cuda(), wd, -1, c["z_reg"], c["scale"], 512, True)
     out[0].backward()
     torch.cuda.synchronize()
-    assert abs(out[0].item() - g["loss"]) <= 1e-3 * abs(g["loss"])
-    assert abs(out[1].item() - g["z_reg"]) <= 1e-3 * abs(g["z_reg"])
-    assert abs(out[2].item() - g["logit_max"]) <= 1e-2 * abs(g["logit_max"])
+    # fp32 tensors are computed as bf16 pairs and held to 1e-5 (loss) / 1e-3 (gradients); 16-bit ones to 1e-3 / 2e-2
+    f32 = c["dtype"] == "float32"
+    ltol, gtol = (1e-5, 1e-3) if f32 else (1e-3, 2e-2)
+    assert abs(out[0].item() - g["loss"]) <= ltol * abs(g["loss"])
+    assert abs(out[1].item() - g["z_reg"]) <= ltol * abs(g["z_reg"])
+    assert abs(out[2].item() - g["logit_max"]) <= 1e-3 * abs(g["logit_max"])
     assert abs(out[3].item() - g["logit_entropy"]) <= 2e-3 * abs(g["logit_entropy"])
     assert abs(out[4].item() - g["logit_norm"]) <= 2e-3 * abs(g["logit_norm"])
     dx, dw = xd.grad.double().cpu(), wd.grad.double().cpu()
-    # 16-bit outputs: norms within 2e-2, probes within 2e-2 of the largest entry scale
-    assert abs(dx.norm().item() - g["dx_norm"]) <= 2e-2 * g["dx_norm"]
-    assert abs(dw.norm().item() - g["dw_norm"]) <= 2e-2 * g["dw_norm"]
+    # norms within the gradient tolerance, probes within it relative to the largest entry
+    assert abs(dx.norm().item() - g["dx_norm"]) <= gtol * g["dx_norm"]
+    assert abs(dw.norm().item() - g["dw_norm"]) <= gtol * g["dw_norm"]
     dx_scale, dw_scale = dx.abs().max().item(), dw.abs().max().item()
     for i, j, v in g["dx_probes"]:
-        assert abs(dx[i % c["N"], j % c["H"]].item() - v) <= 2e-2 * dx_scale
+        assert abs(dx[i % c["N"], j % c["H"]].item() - v) <= gtol * dx_scale
     for i, j, v in g["dw_probes"]:
-        assert abs(dw[i % c["H"], j % c["V"]].item() - v) <= 2e-2 * dw_scale
+        assert abs(dw[i % c["H"], j % c["V"]].item() - v) <= gtol * dw_scale
