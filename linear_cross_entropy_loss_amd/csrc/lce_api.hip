@@ -483,6 +483,8 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.ignore_index = p->ignore_index;
   a.scale = p->logit_scale; a.z_reg = p->z_reg;
   a.dx = dx; a.dw = dw;
+  // fp16 staging of dz: times 2^10, unless z_reg is so large that (1 + 2 * z_reg * lse) * 2^10 could leave fp16's range
+  a.dz_shift = p->x_dtype == LCE_F16 && p->z_reg <= 0.03125f ? 10 : 0;
   a.dz = base + b.dz;
   a.dx_acc = b.slabs > 1 || splits(p) ? (float*)(base + b.dx_acc) : nullptr;
   a.dx_part = b.parts_on ? (float*)(base + b.dx_part) : nullptr;

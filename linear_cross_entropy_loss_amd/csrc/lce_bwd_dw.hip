@@ -25,7 +25,7 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
   const bool tail = part != nullptr;
-  const float coef = tail ? 1.f : final_factor_of(a, dz_unscale<T>());
+  const float coef = tail ? 1.f : final_factor_of(a);
   // fp32 destination addressed as [h][v] with v counted over the whole vocabulary
   float* f32dst = tail ? part - (h0 * kTile + a.v0 + vl0) : reinterpret_cast<float*>(a.dw);
   const int64_t f32ld = tail ? kTile : a.lddw;
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256) void dw_tail_kernel(const BwdArgs a) {
   if (b >= plan.tail_tiles) return;
   int tp, tq;
   tile_coords(plan.full + b, plan.tiles, (int)(a.vs / kTile), (int)(a.Hp / kTile), 8, tp, tq);
-  const float coef = final_factor_of(a, dz_unscale<T>());
+  const float coef = final_factor_of(a);
   const float* part = a.dw_part + (int64_t)b * plan.nseg * kTile * kTile;
   constexpr int kQuads = kTile * kTile / 4 / kTailParts;
   for (int i = piece * kQuads + threadIdx.x; i < (piece + 1) * kQuads; i += 256) {

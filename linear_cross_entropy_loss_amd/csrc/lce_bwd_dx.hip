@@ -33,7 +33,7 @@ LCE_DEV void dx_epilogue(const BwdArgs& a, int64_t rows, void* out, int64_t ldo,
   const int tid = opaque_tid();
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
-  const float coef = final_factor_of(a, dz_unscale<T>());
+  const float coef = final_factor_of(a);
   const int es = a.dx_dtype == DT_F32 ? 4 : 2;
   // descriptor over the rows of this tile: base = first row, range = bytes to the end of dx
   // (scattered rows: base = dx, all of it in range; rows that do not exist get an out-of-range offset below)
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
   void* out = copy ? a.dxc : a.dx;
   const int64_t ldo = copy ? a.lddxc : a.lddx;
   const int* perm = packed && !copy ? a.perm : nullptr;
-  const float coef = final_factor_of(a, dz_unscale<T>());
+  const float coef = final_factor_of(a);
   const float* part = a.dx_part + (int64_t)b * plan.nseg * kTile * kTile;
   constexpr int kQuads = kTile * kTile / 4 / kTailParts;  // quads of this workgroup: 16 rows of the tile
   for (int i = piece * kQuads + threadIdx.x; i < (piece + 1) * kQuads; i += 256) {

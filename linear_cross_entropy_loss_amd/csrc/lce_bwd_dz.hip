@@ -79,7 +79,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
     const bool valid = yy != a.ignore_index;
     const float l = exists ? a.lse[tok] : 0.f;
     // (the power-of-two factor of the staged dz rides along in the exponent)
-    nlse[qb] = valid ? fmaf(-l, kLog2e, (float)dz_shift<T>::value) : -INFINITY;
+    nlse[qb] = valid ? fmaf(-l, kLog2e, (float)a.dz_shift) : -INFINITY;
     gain[qb] = 1.f + 2.f * a.z_reg * l;
     // target column inside this wave's slice, only in the lane half that holds it
     ykey[qb] = (valid && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == half) ? (int)rel : -1;
@@ -153,7 +153,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
             if (want == pp * 16 + r) zt = acc[2 * ph + pp][qb][r];
         float p = __builtin_amdgcn_exp2f(fmaf(zt, c1, nlse[qb]));
         if (ZREG) p *= gain[qb];
-        float tv = p - dz_scale<T>();
+        float tv = p - __builtin_bit_cast(float, (127 + a.dz_shift) << 23);  // the one, times 2^dz_shift
         if (SPLIT && part == 1) tv = bf16_lo(tv);
         *reinterpret_cast<unsigned short*>(lrow + (((yl >> 3) ^ sw) << 4) + (yl & 7) * 2) = to_bits<T>(tv);
       }

@@ -72,16 +72,6 @@ template <class T> LCE_DEV unsigned short to_bits(float f) {
 template <class T> LCE_DEV unsigned int pack2(float lo, float hi) {
   return (unsigned int)to_bits<T>(lo) | ((unsigned int)to_bits<T>(hi) << 16);
 }
-// The staged dz = softmax * gain - onehot is multiplied by 2^dz_shift before it is rounded to the 16-bit
-// compute type, and the dx / dW kernels fold 2^-dz_shift into their final factor.  bf16 has fp32's exponent
-// range and needs none; in fp16 the softmax probabilities of a large vocabulary (of order 1/V) would fall
-// below the normal range (6.1e-5) and lose precision bit by bit -- with 2^10 they stay normal down to 6e-8
-// while |dz| * 2^10 stays far below fp16's maximum for any gain = 1 + 2*z_reg*lse below 63.
-template <class T> struct dz_shift { static constexpr int value = 0; };
-template <> struct dz_shift<F16> { static constexpr int value = 10; };
-template <class T> constexpr float dz_scale() { return (float)(1 << dz_shift<T>::value); }
-template <class T> constexpr float dz_unscale() { return 1.f / (float)(1 << dz_shift<T>::value); }
-
 // fp32 operands are carried as two bf16 numbers, v = hi + lo with hi = bf16(v) and lo = bf16(v - hi): 16
 // bits of mantissa instead of 8.  A product a*b is then taken as a_hi*b_hi + a_hi*b_lo + a_lo*b_hi (the
 // a_lo*b_lo term is of relative order 2^-18 and dropped), which the kernels get by running along a K axis

@@ -91,6 +91,13 @@ struct BwdArgs {
   // The same for dW (K = tokens): dw_part holds dw_tail_blocks() blocks, dw_grid = workgroups of the tile kernel.
   int dw_grid;
   float* dw_part;
+  // The staged dz = softmax * gain - onehot is multiplied by 2^dz_shift before it is rounded to the 16-bit compute
+  // type, and the dx / dW kernels fold 2^-dz_shift into their final factor.  bf16 has fp32's exponent range and
+  // needs none (0); in fp16 the softmax probabilities of a large vocabulary (of order 1/V) would fall below the
+  // normal range (6.1e-5) and lose precision bit by bit -- with 10 they stay normal down to 6e-8, while
+  // |dz| * 2^10 stays below fp16's maximum for any gain = 1 + 2 * z_reg * lse below 63 (the host takes 0 instead
+  // when z_reg is large enough for that to matter).
+  int dz_shift;
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
   // fp32 tensors carried as bf16 pairs (lce_gemm.h): dz is staged as three blocks of Np rows,
@@ -112,10 +119,11 @@ struct BwdArgs {
 
 // Factor applied to dx and dW after their fp32 accumulation: grad_out * logit_scale / n_valid
 // (linear_cross_entropy/ops.py:332, 443-447, 810), times the power of two that undoes the scaling of the staged
-// dz (`unscale`).  With no valid label at all every dz is zero and the factor is taken as 0, so both
+// dz.  With no valid label at all every dz is zero and the factor is taken as 0, so both
 // gradients are exact zeros (what F.cross_entropy's backward gives for such a batch; the loss itself is NaN).
-__device__ __forceinline__ float final_factor_of(const BwdArgs& a, float unscale) {
+__device__ __forceinline__ float final_factor_of(const BwdArgs& a) {
   const int64_t n = a.n_valid[0];
+  const float unscale = __builtin_bit_cast(float, (127 - a.dz_shift) << 23);  // 2^-dz_shift
   return n > 0 ? a.grad_out[0] * a.scale / (float)n * unscale : 0.f;
 }
 

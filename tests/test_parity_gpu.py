@@ -327,3 +327,20 @@ def test_many_tokens_go_through_the_forward_in_chunks(mon):
     assert nv.item() == int(keep.sum().item())
     assert torch.allclose(lse[keep].double(), ref.lse[keep], rtol=2e-4, atol=2e-4)
     assert torch.equal(out5[0], out[0])
+
+
+@pytest.mark.parametrize("z_reg", [0.03125, 0.5])
+def test_fp16_with_a_large_z_regularisation(z_reg):
+    """fp16 stages dz times 2^10 to keep small probabilities normal; the factor 1 + 2 * z_reg * lse rides on top
+    of that, so from z_reg > 1/32 on the staging is left unscaled instead.  Either side of the switch against
+    the oracle, with logits large enough for lse to be of order 10."""
+    print(f"fp16 z_reg={z_reg}", flush=True)
+    x, y, w = make_inputs(512, 256, 4096, torch.float16, seed=91, ignore_frac=0.1, w_std=0.2)
+    out, dx, dw = _run(x, y, w, -1, z_reg, 1.0, 512, False, grad_output=64.0)
+    ref = _oracle(x, y, w, -1, z_reg, 1.0, grad_output=64.0)
+    assert torch.isfinite(dx).all() and torch.isfinite(dw).all()
+    assert ref.lse.abs().max().item() > 8
+    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item())
+    for got, want in ((dx, ref.dx), (dw, ref.dw)):
+        emax, el2 = rel_errors(got, want)
+        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (emax, el2)
