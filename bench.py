@@ -300,7 +300,8 @@ def _load_probe_lib():
 
 def probe_ceiling(torch):
     """What bounds the tile kernels on this part: (1) a register-only loop of the same MFMA instruction over
-    the same 128 x 128 wave tile, on constant and on random operands, on all and on half of the compute units;
+    the same 128 x 128 wave tile, on constant and on random operands, and with the tile kernels' LDS reads and
+    writes added (still no global loads, barriers or epilogues), on all and on half of the compute units;
     (2) the vendor GEMM (torch.matmul -> hipBLASLt) on the four contractions of the default workload; (3) the
     operator's forward tile kernel on all and on half of the compute units (a chip-level power limit shows as a
     higher rate per compute unit when fewer of them run)."""
@@ -314,7 +315,8 @@ def probe_ceiling(torch):
     buf = torch.empty(cus * 256 * 4, dtype=torch.float32, device="cuda")
     iters = 200000
     for wgs in (cus, cus // 2):
-        for pattern, name in ((0, "constant operands"), (1, "random bf16 operands")):
+        for pattern, name in ((0, "constant operands"), (1, "random bf16 operands"),
+                              (2, "random, fragments re-read from LDS"), (3, "random, LDS reads + LDS writes")):
             def run():
                 rc = probe.lce_probe_mfma(pattern, wgs, iters, ctypes.c_void_p(buf.data_ptr()), stream)
                 assert rc == 0

@@ -4,6 +4,9 @@
 //                     keeps 4 A and 4 B fragments in registers and issues v_mfma_f32_32x32x16_bf16 over a
 //                     4 x 4 grid of accumulator blocks (the 128 x 128 wave tile of the operator's kernels),
 //                     on constant or on random operands.  The ceiling the tile kernels are measured against.
+//                     Two further patterns add the LDS traffic of the tile kernels and nothing else (no global
+//                     loads, no barriers, no epilogue): every k step's 8 fragments are re-read from LDS, and
+//                     4 x 16 bytes per lane are written to it.
 //   lce_probe_flush   what adding 256 x 256 fp32 blocks of partial sums into a matrix in memory costs, with
 //                     atomics or as plain read-modify-write: the traffic a backward that fed dz straight into
 //                     the dx and dW contractions would generate once per dz tile (its H-wide accumulators do
@@ -69,6 +72,63 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int pattern, int iters, 
   out[tid] = s;
 }
 
+// pattern 2: random operands, the 4 + 4 fragments of every k step read from LDS (8 ds_read_b128 per 16 MFMAs, the
+// rate of the operator's tile kernels), one k step ahead; pattern 3: additionally 4 ds_write_b128 per 16 MFMAs (the
+// rate at which those kernels refill their LDS stages).  Reads and writes are interleaved with the MFMAs one by one.
+template <bool WRITES>
+__global__ __launch_bounds__(256) void mfma_lds_loop_kernel(int iters, float* out) {
+  __shared__ __attribute__((aligned(16))) short lds[65536];  // 128 KiB, the two stages of a tile kernel
+  const unsigned tid = blockIdx.x * 256u + threadIdx.x;
+  for (int i = threadIdx.x; i < 65536; i += 256) lds[i] = random_bf16(blockIdx.x * 65536u + i);
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  s16x8_t fa[8], fb[8];
+  const s16x8_t* rd = reinterpret_cast<const s16x8_t*>(lds);  // 8192 pieces of 16 bytes
+  s16x8_t* wr = reinterpret_cast<s16x8_t*>(lds);
+#pragma unroll
+  for (int f = 0; f < 8; ++f) fa[f] = rd[(wave * 2048 + f * 64 + lane) & 8191];
+  auto step = [&](s16x8_t (&cur)[8], s16x8_t (&nxt)[8], int it) {
+    const int o = (it + 1) * 512 + wave * 2048;
+#pragma unroll
+    for (int f = 0; f < 8; ++f) nxt[f] = rd[(o + f * 64 + lane) & 8191];
+    if (WRITES) {
+#pragma unroll
+      for (int f = 0; f < 4; ++f) wr[(o + 4096 + f * 64 + lane) & 8191] = cur[f];
+    }
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      const int i = s >> 2, j = (i & 1) ? 3 - (s & 3) : (s & 3);
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, cur[i]),
+                                                          __builtin_bit_cast(bf16x8_t, cur[4 + j]), acc[i][j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                       // one MFMA
+      if (s < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                            // one LDS read
+      if (WRITES && s >= 8 && (s & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
+    }
+  };
+  for (int it = 0; it < iters; it += 2) {  // (the two fragment sets change roles: no register moves)
+    step(fa, fb, it);
+    step(fb, fa, it + 1);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s += acc[i][j][r];
+  out[tid] = s;
+}
+
 // Each workgroup adds `tiles` blocks of 256 x 256 floats into dst[rows][ld]: it walks down the row tiles of
 // column tile b / 4, then of the next one, so that (as in a tile order that shares operand bands between
 // neighbouring workgroups) four workgroups add into the same block at about the same time -- the pattern
@@ -98,11 +158,16 @@ __global__ __launch_bounds__(256) void flush_kernel(float* dst, int64_t rows, in
 
 extern "C" {
 
-// Launches `wgs` workgroups of 4 waves, each wave issuing iters * 16 MFMAs (32 x 32 x 16, bf16).
+// Launches `wgs` workgroups of 4 waves, each wave issuing iters * 16 MFMAs (32 x 32 x 16, bf16); iters even.
+// pattern 0 constant / 1 random operands in registers; 2 random operands re-read from LDS; 3 plus LDS writes.
 // out: wgs * 256 floats.  FLOPs = wgs * 4 * iters * 16 * 32768.
 int lce_probe_mfma(int pattern, int wgs, int iters, float* out, void* stream) {
-  if (pattern < 0 || pattern > 1 || wgs <= 0 || iters <= 0 || !out) return -3;
-  hipLaunchKernelGGL(mfma_loop_kernel, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, pattern, iters, out);
+  if (pattern < 0 || pattern > 3 || wgs <= 0 || iters <= 0 || (iters & 1) || !out) return -3;
+  const dim3 grid((unsigned)wgs), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  if (pattern == 2) hipLaunchKernelGGL(mfma_lds_loop_kernel<false>, grid, block, 0, s, iters, out);
+  else if (pattern == 3) hipLaunchKernelGGL(mfma_lds_loop_kernel<true>, grid, block, 0, s, iters, out);
+  else hipLaunchKernelGGL(mfma_loop_kernel, grid, block, 0, s, pattern, iters, out);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
