@@ -184,6 +184,46 @@ def test_runs_are_deterministic_and_backward_can_repeat():
     assert torch.equal(g1[0], a[1])
 
 
+def test_two_threads_on_two_streams_do_not_disturb_each_other():
+    """The library keeps no state between calls and none that two calls share (lce.h): two host threads, each
+    with a stream, inputs and scratch of its own, run forward + backward at the same time, several times over;
+    every result is bit-identical to the same call made alone."""
+    import contextvars
+    import threading
+
+    print("two threads, two streams", flush=True)
+    cases = [make_inputs(1024, 512, 8192, torch.bfloat16, seed=61, ignore_frac=0.1, device="cuda") + (1e-4, 0.5),
+             make_inputs(768, 256, 12288, torch.float16, seed=62, ignore_frac=0.3, device="cuda") + (0.0, 1.0)]
+    alone = [_fb(x, y, w, z_reg=z, scale=s, mon=True) for x, y, w, z, s in cases]
+    torch.cuda.synchronize()
+    failures = []
+
+    def worker(k):
+        try:
+            x, y, w, z, s = cases[k]
+            stream = torch.cuda.Stream()  # (default priority)
+            for _ in range(5):
+                with torch.cuda.stream(stream):
+                    out, dx, dw = _fb(x, y, w, z_reg=z, scale=s, mon=True)
+                stream.synchronize()
+                for t, u in zip(out, alone[k][0]):
+                    if not torch.equal(t, u):
+                        failures.append((k, "output"))
+                if not (torch.equal(dx, alone[k][1]) and torch.equal(dw, alone[k][2])):
+                    failures.append((k, "gradient"))
+        except Exception as exc:  # surfaced below: an exception in a thread would otherwise pass silently
+            failures.append((k, repr(exc)))
+
+    # (each thread runs in a copy of this context, so that it packs ignored tokens, or not, as the calls above did)
+    threads = [threading.Thread(target=contextvars.copy_context().run, args=(worker, k)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=120)
+    assert not any(t.is_alive() for t in threads)
+    assert not failures, failures
+
+
 def test_upstream_gradient_scales_linearly():
     print("grad_output linearity", flush=True)
     # bf16 on purpose: gradients of order 1/N are subnormal in fp16, where scaling by 4 is not exact
