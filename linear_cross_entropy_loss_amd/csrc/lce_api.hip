@@ -166,16 +166,17 @@ size_t dw_part_bytes(size_t Np, size_t Hp, int64_t vs, int64_t last_vs) {
   return (size_t)(b0 > b1 ? b0 : b1) * 256 * 256 * 4;
 }
 
-// Fewest vocabulary slabs (of a width that is a multiple of 256 columns; the last
-// one may be narrower) whose staging fits the scratch bound.  The dz stage itself
-// is additionally capped at 1 GiB: wider slabs are not faster, so a generous
-// N_chunk_size does not translate into a larger footprint.
+// Vocabulary slabs (of a width that is a multiple of 256 columns; the last one may be narrower) whose staging
+// fits the scratch bound: the fewest that fit, or somewhat more of them when a model of the three kernels'
+// rounds of workgroups says that those run faster (slab_cost below).  The dz stage itself is additionally
+// capped at 1 GiB: wider slabs are not faster, so a generous N_chunk_size does not translate into a larger
+// footprint.
 //
 // The bound is n_chunk * V * 4 bytes, what the reference spends on its logits
 // chunk (ops.py:700).  Everything counts towards it: the dz stage, the fp32 running dx, the packed rows and
-// the partial sums of split tail tiles.  When that leaves only narrow slabs (under 8192 columns: few dW
-// tiles per launch), the two optional items are given up first if that buys wider slabs -- `lean`: tokens
-// with an ignored label are then not packed away in the backward and tail tiles are not split.
+// the partial sums of split tail tiles.  The two optional items are given up when the plan without them is
+// the faster one by the same model -- `lean`: tokens with an ignored label are then not packed away in the
+// backward and tail tiles are not split, which buys wider slabs under a tight bound.
 // Shapes with a small vocabulary and many tokens cannot meet the bound at all (the fp32 running dx alone is
 // larger, and a split into very narrow slabs leaves the GPU idle); for those the bound is widened by
 // N * H * 4 bytes, the fp32 x_grad buffer the reference allocates next to its logits chunk (ops.py:693) and
@@ -194,8 +195,36 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   b->lse_c = b->pack.end;
   b->dxc = b->lse_c + align_up((size_t)p->N * 4);
 
-  // mode 0: everything; mode 1: lean (at the strict bound only); mode 2: everything, widened bound
-  auto fits = [&](int mode, BwdPlan* out) -> bool {
+  // Modelled time of the three kernels over one slab of `w` columns, in units of one 64-deep K tile of a 256 x 256
+  // output tile on a full chip.  A kernel runs its T tiles in rounds of kPlanCUs; a last round that fills a
+  // fraction f of the compute units runs 1 + 0.9 (1 - f) times faster per compute unit (the part is limited by
+  // power: measured 1.14 / 1.30 / 1.46 / 1.54 at f = 0.81 / 0.69 / 0.47 / 0.34), and is cut along K when the
+  // partial-sum blocks exist (`parts`; a small kernel then adds the segments: 12 units).  Per tile, the epilogues
+  // cost about 6 (dz), 21 (dx adding into the fp32 running sum: 512 KiB of traffic at a compute unit's share of the
+  // memory bandwidth; 5 when it is written once) and 5 (dW) units; a launch about 10.  The model ranks the slab
+  // widths measured at N = 16384, H = 2048, V = 32768 and 65536 (2 ... 18 slabs) in their measured order.
+  constexpr double kPlanCUs = 256.0;
+  auto kernel_cost = [&](double T, double L, double e, bool parts) -> double {
+    const double full = (double)(int64_t)(T / kPlanCUs), r = T - full * kPlanCUs;
+    double cost = full * (L + e) + 10.0;
+    if (r > 0) {
+      double seg = 1;
+      if (parts) while (r * seg * 2 <= kPlanCUs && L / (seg * 2) >= 16) seg *= 2;
+      const double f = r * seg / kPlanCUs;
+      cost += (L / seg + e) / (1.0 + 0.9 * (1.0 - f)) + (seg > 1 ? 12.0 : 0.0);
+    }
+    return cost;
+  };
+  auto slab_cost = [&](int64_t w, bool parts, bool sums) -> double {
+    const double tq = (double)(Np / 256), th = (double)(Hp / 256), tv = (double)(w / 256), k3 = split ? 3.0 : 1.0;
+    return kernel_cost(tq * tv, k3 * (double)((p->H + 63) / 64), 6.0, false) +
+           k3 * kernel_cost(tq * th, (double)(w / 64), sums ? 21.0 : 5.0, parts) +
+           kernel_cost(tv * th, k3 * (double)(Np / 64), 5.0, parts);
+  };
+
+  // mode 0: everything; mode 1: lean (at the strict bound only); mode 2: everything, widened bound.
+  // Tries a split into `s` slabs of equal width (the last one may be narrower); cost: its modelled time.
+  auto fits = [&](int mode, int64_t s, BwdPlan* out, double* cost) -> bool {
     const bool lean = mode == 1;
     const bool pack = packs_rows(p) && !(lean && p->pack_rows == LCE_PACK_AUTO);
     // The dx kernels store packed rows straight to their tokens' places through 32-bit offsets into dx; a dx
@@ -205,47 +234,60 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
     if (pack) fixed = b->dxc + (stage_dx ? align_up((size_t)p->N * (size_t)b->lddxc * dxes) : 0);
     else if (split) fixed = b->pack.end;
     const size_t budget = strict + (mode == 2 ? (size_t)p->N * (size_t)p->H * 4 : 0);
+    const int64_t vs = (cols + s - 1) / s * 256;
+    const int64_t slabs = (Vp + vs - 1) / vs;
+    // (bf16 pairs: three blocks of dz, and dx is summed over three passes per slab, so it always needs the running sum)
+    const size_t dz = align_up(Np * (size_t)vs * 2 * (split ? 3 : 1));
+    const size_t acc = slabs > 1 || split ? align_up(Np * Hp * 4) : 0;
+    const int64_t last_vs = Vp - (slabs - 1) * vs;  // padded width of the last slab
+    const size_t dxp = lean ? 0 : dx_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
+    const size_t dwp = lean ? 0 : dw_part_bytes(split ? 3 * Np : Np, Hp, vs, last_vs);
+    const size_t part = dxp + dwp;
+    const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2 * (split ? 3 : 1)) : 0;  // 16-bit copy of the slab of W
+    // the widened bound is for the staging proper; the split-K partial sums (at most 64 MiB each for dx
+    // and dW) and the packed rows come on top of it there
+    // (reserve: what the caller holds besides the workspace between forward and backward -- lse and a few scalars)
+    const size_t reserve = align_up((size_t)p->N * 4) + 4096;
+    const size_t counted = dz + acc + w16 + (mode != 2 ? fixed + part + reserve : 0);
+    if (!((counted <= budget && (dz <= dz_cap || vs == 256)) || (mode == 2 && vs == 256))) return false;
+    out->slabs = slabs;
+    out->vs = vs;
+    out->pack_on = pack;
+    out->parts_on = !lean;
+    out->stage_dx = stage_dx;
+    out->dz = fixed;
+    out->dx_acc = fixed + dz;
+    out->dx_part = fixed + dz + acc;
+    out->dw_part = fixed + dz + acc + dxp;
+    out->w16 = fixed + dz + acc + part;
+    out->total = fixed + dz + acc + part + w16;
+    // (a lean plan computes the tokens with an ignored label too; how many there are is not known here)
+    *cost = ((double)(slabs - 1) * slab_cost(vs, !lean, acc != 0) + slab_cost(last_vs, !lean, acc != 0)) *
+            (lean && packs_rows(p) ? 1.02 : 1.0);
+    return true;
+  };
+  // The fewest slabs that fit, or a few more of them when the model says that their tiles fill the rounds of
+  // workgroups better (four slabs of 8192 columns against three of 11008 at H = 2048, say).
+  auto choose = [&](int mode, BwdPlan* out, double* cost) -> bool {
+    int64_t first = 0;
+    BwdPlan cand = *out;
+    double c = 0;
     for (int64_t s = 1; s <= cols; ++s) {
-      const int64_t vs = (cols + s - 1) / s * 256;
-      if (s > 1 && (cols + s - 2) / (s - 1) * 256 == vs) continue;  // same width as with one slab fewer
-      const int64_t slabs = (Vp + vs - 1) / vs;
-      // (bf16 pairs: three blocks of dz, and dx is summed over three passes per slab, so it always needs the running sum)
-      const size_t dz = align_up(Np * (size_t)vs * 2 * (split ? 3 : 1));
-      const size_t acc = slabs > 1 || split ? align_up(Np * Hp * 4) : 0;
-      const int64_t last_vs = Vp - (slabs - 1) * vs;  // padded width of the last slab
-      const size_t dxp = lean ? 0 : dx_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
-      const size_t dwp = lean ? 0 : dw_part_bytes(split ? 3 * Np : Np, Hp, vs, last_vs);
-      const size_t part = dxp + dwp;
-      const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2 * (split ? 3 : 1)) : 0;  // 16-bit copy of the slab of W
-      // the widened bound is for the staging proper; the split-K partial sums (at most 64 MiB each for dx
-      // and dW) and the packed rows come on top of it there
-      // (reserve: what the caller holds besides the workspace between forward and backward -- lse and a few scalars)
-      const size_t reserve = align_up((size_t)p->N * 4) + 4096;
-      const size_t counted = dz + acc + w16 + (mode != 2 ? fixed + part + reserve : 0);
-      if ((counted <= budget && (dz <= dz_cap || vs == 256)) || (mode == 2 && vs == 256)) {
-        out->slabs = slabs;
-        out->vs = vs;
-        out->pack_on = pack;
-        out->parts_on = !lean;
-        out->stage_dx = stage_dx;
-        out->dz = fixed;
-        out->dx_acc = fixed + dz;
-        out->dx_part = fixed + dz + acc;
-        out->dw_part = fixed + dz + acc + dxp;
-        out->w16 = fixed + dz + acc + part;
-        out->total = fixed + dz + acc + part + w16;
-        return true;
-      }
+      if (s > 1 && (cols + s - 2) / (s - 1) == (cols + s - 1) / s) continue;  // same width as with one slab fewer
+      if (first != 0 && (mode == 2 || s > 4 * first + 8)) break;
+      if (!fits(mode, s, &cand, &c)) continue;
+      if (first == 0 || c < *cost) { *out = cand; *cost = c; }
+      if (first == 0) first = s;
     }
-    return false;
+    return first != 0;
   };
   BwdPlan full = *b, lean = *b;
-  const bool ok_full = fits(0, &full);
-  if (ok_full && (full.vs >= 8192 || full.slabs == 1)) { *b = full; return LCE_OK; }
-  const bool ok_lean = fits(1, &lean);
-  if (ok_lean && (!ok_full || lean.vs > full.vs)) { *b = lean; return LCE_OK; }
-  if (ok_full) { *b = full; return LCE_OK; }
-  if (fits(2, b)) return LCE_OK;
+  double cost_full = 0, cost_lean = 0;
+  const bool ok_full = choose(0, &full, &cost_full), ok_lean = choose(1, &lean, &cost_lean);
+  if (ok_full && (!ok_lean || cost_full <= cost_lean)) { *b = full; return LCE_OK; }
+  if (ok_lean) { *b = lean; return LCE_OK; }
+  double unused = 0;
+  if (choose(2, b, &unused)) return LCE_OK;
   return LCE_EWORKSPACE;
 }
 

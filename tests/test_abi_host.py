@@ -372,8 +372,8 @@ def test_library_imports_no_allocation_or_synchronisation_routine():
 
 def test_backward_plan_invariants_on_random_problems():
     """Seeded random problems: the slabs cover the vocabulary, widths are tile multiples, the reported scratch
-    is what the bound allows whenever the narrowest split could meet it, a larger bound never means more
-    slabs, and forward scratch never depends on more than one chunk of tokens."""
+    is what the bound allows whenever the narrowest split could meet it, a larger bound keeps the slab count
+    inside the planner's search window, and forward scratch never depends on more than one chunk of tokens."""
     import random
 
     from linear_cross_entropy_loss_amd import _lib
@@ -396,9 +396,10 @@ def test_backward_plan_invariants_on_random_problems():
         Vp = -(-V // 256) * 256
         assert width % 256 == 0 and 1 <= slabs and (slabs - 1) * width < Vp <= slabs * width, (it, slabs, width)
         assert fwd > 0 and bwd > 0
-        # a larger bound never needs more slabs
+        # The planner takes the fewest slabs that fit or, when its model of the kernels' rounds of workgroups says
+        # that more of them run faster, up to 4 * fewest + 8.  A larger bound cannot raise the fewest that fit.
         slabs2, _ = _lib.backward_plan(mk(nc * 4))
-        assert slabs2 <= slabs, (it, slabs, slabs2)
+        assert slabs2 <= 4 * slabs + 8, (it, slabs, slabs2)
         # forward: partial sums of one chunk of tokens at most, whatever N
         chunk = max(-(-nc // 256) * 256, 65536 if wd == torch.float32 and xd != torch.float32 or xd == torch.float32 else 16384)
         Np = -(-N // 256) * 256
