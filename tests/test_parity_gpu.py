@@ -344,3 +344,22 @@ def test_fp16_with_a_large_z_regularisation(z_reg):
     for got, want in ((dx, ref.dx), (dw, ref.dw)):
         emax, el2 = rel_errors(got, want)
         assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (emax, el2)
+
+
+@pytest.mark.parametrize("dtype,w_std,scale", [(torch.bfloat16, 5.0, 1.0), (torch.float16, 1.0, 8.0),
+                                               (torch.float32, 5.0, 1.0)])
+def test_saturated_softmax_with_logits_in_the_hundreds(dtype, w_std, scale):
+    """Logits of standard deviation 80 or more (max beyond 300): exp(logit) alone would overflow fp32, most
+    probabilities underflow to zero and every row's softmax is close to one-hot.  The running-maximum form of
+    lse must keep loss and gradients finite and equal to the fp64 oracle's, to the tolerances of the dtype."""
+    print(f"saturated softmax {dtype}", flush=True)
+    x, y, w = make_inputs(512, 256, 4096, dtype, seed=77, ignore_frac=0.1, w_std=w_std)
+    out, dx, dw = _run(x, y, w, -1, 0.0, scale, 512, False)
+    ref = _oracle(x, y, w, -1, 0.0, scale)
+    assert ref.lse.abs().max().item() > 300
+    assert torch.isfinite(out[0]) and torch.isfinite(dx).all() and torch.isfinite(dw).all()
+    loss_rtol, grad_tol = _tols(dtype)
+    assert abs(out[0].item() - ref.loss.item()) <= loss_rtol * abs(ref.loss.item())
+    for got, want in ((dx, ref.dx), (dw, ref.dw)):
+        emax, el2 = rel_errors(got, want)
+        assert emax <= grad_tol and el2 <= grad_tol, (emax, el2)
