@@ -240,11 +240,11 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
     const size_t dz = align_up(Np * (size_t)vs * 2 * (split ? 3 : 1));
     const size_t acc = slabs > 1 || split ? align_up(Np * Hp * 4) : 0;
     const int64_t last_vs = Vp - (slabs - 1) * vs;  // padded width of the last slab
-    const size_t dxp = lean ? 0 : dx_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB each
+    const size_t dxp = lean ? 0 : dx_part_bytes(Np, Hp, vs, last_vs);  // at most 64 MiB
     const size_t dwp = lean ? 0 : dw_part_bytes(split ? 3 * Np : Np, Hp, vs, last_vs);
-    const size_t part = dxp + dwp;
+    const size_t part = dxp > dwp ? dxp : dwp;  // one buffer: the dx kernels are done with it before the dW kernels start
     const size_t w16 = p->w_dtype == LCE_F32 ? align_up((size_t)p->H * (size_t)vs * 2 * (split ? 3 : 1)) : 0;  // 16-bit copy of the slab of W
-    // the widened bound is for the staging proper; the split-K partial sums (at most 64 MiB each for dx
+    // the widened bound is for the staging proper; the split-K partial sums (at most 64 MiB, shared by dx
     // and dW) and the packed rows come on top of it there
     // (reserve: what the caller holds besides the workspace between forward and backward -- lse and a few scalars)
     const size_t reserve = align_up((size_t)p->N * 4) + 4096;
@@ -258,7 +258,7 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
     out->dz = fixed;
     out->dx_acc = fixed + dz;
     out->dx_part = fixed + dz + acc;
-    out->dw_part = fixed + dz + acc + dxp;
+    out->dw_part = out->dx_part;
     out->w16 = fixed + dz + acc + part;
     out->total = fixed + dz + acc + part + w16;
     // (a lean plan computes the tokens with an ignored label too; how many there are is not known here)

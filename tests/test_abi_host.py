@@ -181,7 +181,8 @@ def test_backward_plan_is_consistent_with_workspace():
         part = dx_part_bytes(Np, Hp, width, pad(V, 256) - (slabs - 1) * width)
         partw = dw_part_bytes(Np, Hp, width, pad(V, 256) - (slabs - 1) * width)
         assert part <= 64 << 20 and partw <= 64 << 20
-        assert bwd == _pack_bytes(N, H) + Np * width * 2 + (Np * Hp * 4 if slabs > 1 else 0) + part + partw
+        # (one buffer serves both: the dx kernels are done with it before the dW kernels start)
+        assert bwd == _pack_bytes(N, H) + Np * width * 2 + (Np * Hp * 4 if slabs > 1 else 0) + max(part, partw)
         assert Np * width * 2 <= max(1 << 30, Np * 256 * 2)   # dz stage capped at 1 GiB
         # without the packing of ignored tokens: the same minus its buffers, if the split stays the same;
         # by default the library packs from 8*N*H*V = 2^41 FLOPs on
