@@ -48,6 +48,8 @@ CASES = [
     (512, 768, 4096, torch.bfloat16, torch.float32, 0.0, 1e-2, 1.0, 4096, True),
     (512, 256, 4096, torch.float32, None, 0.05, 1e-4, 1.0, 512, True),
     (2048, 256, 12288, torch.bfloat16, None, 0.5, 0.0, 0.7, 512, False),
+    (512, 16384, 4096, torch.bfloat16, None, 0.1, 1e-4, 1.0, 512, True),              # a hidden size beyond any config's
+    (256, 12288, 2048, torch.float16, torch.float32, 0.0, 0.0, 1.0, 4096, False),
 ]
 
 
