@@ -169,6 +169,32 @@ def test_arbitrary_shapes_match_oracle(N, H, V, dtype, w_dtype, ign, z_reg, scal
         assert (dx.cpu()[ignored] == 0).all()
 
 
+def test_a_vocabulary_of_a_million_columns():
+    """V = 1000003 (not a multiple of anything), few tokens: 3907 vocabulary tiles per token tile, a target in the
+    last column, many vocabulary slabs under a small N_chunk_size; oracle in fp64 on the GPU."""
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+    from oracle import lce_forward_backward_fp64
+
+    print("vocabulary of 1000003", flush=True)
+    N, H, V = 300, 128, 1000003
+    x, y, w = make_inputs(N, H, V, torch.bfloat16, seed=1000003, ignore_frac=0.1, device="cuda")
+    y[0] = V - 1
+    xd = x.clone().requires_grad_(True)
+    wd = w.clone().requires_grad_(True)
+    out = linear_cross_entropy(xd, y, wd, -1, 1e-4, 1.0, 64, True)
+    out[0].backward()
+    ref = lce_forward_backward_fp64(x, y, w, -1, 1e-4, 1.0, chunk=64)
+    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item())
+    assert abs(out[2].item() - ref.logit_max.item()) <= 1e-3 * abs(ref.logit_max.item())
+    for name, got, want in (("dx", xd.grad, ref.dx), ("dw", wd.grad, ref.dw)):
+        d = got.double() - want
+        emax = (d.abs().max() / want.abs().max()).item()
+        el2 = (d.norm() / want.norm()).item()
+        print(f"  {name}: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
+        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (name, emax, el2)
+    assert (xd.grad[y == -1] == 0).all()
+
+
 def test_strided_inputs_and_garbage_in_the_stride_padding():
     """x and W handed over as views with padded row strides whose padding holds large finite garbage: the
     result must be bit-identical to the dense call (the kernels never let the padding reach a valid output)."""
