@@ -90,6 +90,8 @@ MID_CASES = [
     (2048, 1024, 32768, torch.float16, torch.float32, True, 0.1, 0.0, 1.0, 512, False),  # config-5 style: fp32 master W
     (4096, 512, 65536, torch.bfloat16, None, False, 0.05, 0.0, 1.0, 512, False),        # several vocabulary slabs
     (2048, 2048, 16384, torch.float32, None, False, 0.0, 0.0, 1.0, 4096, False),        # config 1 (fp32 tensors)
+    (300001, 72, 1000, torch.bfloat16, None, False, 0.2, 1e-4, 1.0, 512, True),         # many tokens: 19 forward chunks
+    (131073, 64, 520, torch.float16, torch.float32, True, 0.5, 0.0, 2.0, 64, False),     # fp32 W: 3 forward chunks
 ]
 
 
