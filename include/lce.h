@@ -74,9 +74,9 @@ typedef struct lce_problem {
   int64_t H;            /* in_features                                         */
   int64_t V;            /* out_features (vocabulary)                           */
   int64_t ldx;          /* row stride of x, elements                           */
-  int64_t ldw;          /* row stride of w, elements                           */
+  int64_t ldw;          /* row stride of w, elements (see w_layout)            */
   int64_t lddx;         /* row stride of dx, elements (backward only)          */
-  int64_t lddw;         /* row stride of dw, elements (backward only)          */
+  int64_t lddw;         /* row stride of dw, elements (backward only; see w_layout) */
   int32_t x_dtype;      /* LCE_BF16 | LCE_F16 | LCE_F32 (see "Arithmetic" below)  */
   int32_t w_dtype;      /* same as x_dtype, or LCE_F32 (master weight, rounded slab by slab in ws) */
   int32_t dx_dtype;     /* x_dtype or LCE_F32                                  */
@@ -89,7 +89,27 @@ typedef struct lce_problem {
   int32_t phases;       /* 0 = everything; otherwise a mask of LCE_PHASE_* (profiling aid) */
   int32_t pack_rows;    /* LCE_PACK_AUTO | LCE_PACK_ALWAYS | LCE_PACK_NEVER: see below        */
   int32_t max_workgroups; /* profiling aid: cap on the persistent workgroups of the tile kernels (0 = one per compute unit) */
+  int32_t w_layout;     /* LCE_W_HV (0) | LCE_W_VH: how w and dw are stored, see below */
+  int32_t reserved;     /* 0 */
 } lce_problem;
+
+/*
+ * Layout of the weight and of its gradient.  The reference takes At of shape
+ * (H, V) with whatever strides the tensor has (ops.py:733-734 pass
+ * At.stride(0), At.stride(1) to the kernels, and At_grad = zeros_like(At) keeps
+ * them, ops.py:693), so a tied embedding matrix stored (V, H) can be handed
+ * over as its transposed view without a copy.  Here the two dense cases are:
+ *   LCE_W_HV  w[h * ldw + v],  ldw  >= V   -- At stored row-major (H, V)
+ *   LCE_W_VH  w[v * ldw + h],  ldw  >= H   -- At is the transposed view of a
+ *             row-major (V, H) matrix (an nn.Embedding / nn.Linear(H, V) weight)
+ * dw has the layout of w with row stride lddw.  LCE_W_VH needs 16-bit x, and
+ * H a multiple of 8 (both operands of the logit contraction then run along
+ * H in memory, and no 16-byte piece may straddle the end of a row).
+ */
+enum {
+  LCE_W_HV = 0,
+  LCE_W_VH = 1
+};
 
 /*
  * Arithmetic.  16-bit x: products of 16-bit operands (an fp32 master weight is

@@ -35,8 +35,15 @@ int check(const lce_problem* p, bool backward) {
   if (!(p->logit_scale > 0.f) || !(p->z_reg >= 0.f)) return LCE_EINVAL_ARG;
   if (p->pack_rows != LCE_PACK_AUTO && p->pack_rows != LCE_PACK_ALWAYS && p->pack_rows != LCE_PACK_NEVER) return LCE_EINVAL_ARG;
   if (p->max_workgroups < 0) return LCE_EINVAL_ARG;
+  if (p->w_layout != LCE_W_HV && p->w_layout != LCE_W_VH) return LCE_EINVAL_ARG;
+  const bool vh = p->w_layout == LCE_W_VH;
+  // (V, H) weight: both operands of the logit contraction run along H in memory, so no 16-byte piece may
+  // straddle the end of a row (H a multiple of 8), and there is no bf16-pair form of it
+  if (vh && xd == LCE_F32) return LCE_EINVAL_DTYPE;
+  if (vh && p->H % 8) return LCE_EINVAL_ARG;
+  const int64_t w_cols = vh ? p->H : p->V;  // row length of w and dw as stored
   const int64_t xa = xd == LCE_F32 ? 4 : 8, wa = wd == LCE_F32 ? 4 : 8;  // 16-byte rows
-  if (p->ldx < p->H || p->ldx % xa || p->ldw < p->V || p->ldw % wa) return LCE_EINVAL_ARG;
+  if (p->ldx < p->H || p->ldx % xa || p->ldw < w_cols || p->ldw % wa) return LCE_EINVAL_ARG;
   // The kernels address a 256-row tile of x, of a 16-bit W and of dx with 32-bit byte offsets: 256 rows must
   // stay below 2 GiB.  (An fp32 W is only read by the slab conversion, which uses 64-bit addresses.)
   const int64_t tile_limit = ((int64_t)1 << 31) / 256;
@@ -48,7 +55,7 @@ int check(const lce_problem* p, bool backward) {
     if (p->dx_dtype != xd && p->dx_dtype != LCE_F32) return LCE_EINVAL_DTYPE;
     if (p->dw_dtype != wd && p->dw_dtype != LCE_F32) return LCE_EINVAL_DTYPE;
     // dx is stored in 8-byte (16-bit types) or 16-byte pieces, dW in 16-byte pieces
-    if (p->lddx < p->H || p->lddx % 4 || p->lddw < p->V || p->lddw % (p->dw_dtype == LCE_F32 ? 4 : 8)) return LCE_EINVAL_ARG;
+    if (p->lddx < p->H || p->lddx % 4 || p->lddw < w_cols || p->lddw % (p->dw_dtype == LCE_F32 ? 4 : 8)) return LCE_EINVAL_ARG;
     if (p->lddx * (p->dx_dtype == LCE_F32 ? 4 : 2) > tile_limit) return LCE_EINVAL_ARG;
   }
   return LCE_OK;
@@ -346,6 +353,7 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
   a.N = p->N; a.H = p->H; a.V = p->V; a.ldx = p->ldx; a.ldw = p->ldw;
   a.Np = lce::padded_tokens(p->N); a.Vp = lce::padded_vocab(p->V);
   a.x_dtype = p->x_dtype; a.w_dtype = p->w_dtype;
+  a.w_vh = p->w_layout == LCE_W_VH;
   a.ignore_index = p->ignore_index;
   a.scale = p->logit_scale; a.z_reg = p->z_reg; a.monitoring = p->monitoring ? 1 : 0;
   a.lse = lse; a.out5 = out5; a.n_valid = n_valid;
@@ -403,9 +411,11 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
         t.v0 = v0;
         t.vw = p->V - v0 < f.vs ? p->V - v0 : f.vs;
         if (p->w_dtype == LCE_F32) {
-          const int64_t ld16 = lce::pad_to(t.vw, 256);
-          e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, v0, t.vw, base + f.w16, ld16, compute_dtype(p),
-                                         splits(p), s);
+          const int64_t ld16 = a.w_vh ? p->H : lce::pad_to(t.vw, 256);
+          e = a.w_vh ? lce::launch_convert_w_rows((const float*)w, p->ldw, p->H, v0, t.vw, base + f.w16, ld16,
+                                                  compute_dtype(p), s)
+                     : lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, v0, t.vw, base + f.w16, ld16,
+                                                  compute_dtype(p), splits(p), s);
           if (e != hipSuccess) return hip_fail(e, "convert_w");
           t.w = base + f.w16; t.ldw = ld16; t.w_dtype = compute_dtype(p); t.wv0 = v0; t.Vw = t.vw;
         } else {
@@ -431,7 +441,7 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
 
 extern "C" {
 
-int lce_version(void) { return 300; }  // 0.3.0: lce_forward_static, lce_problem.max_workgroups, fp32 tensors as bf16 pairs
+int lce_version(void) { return 400; }  // 0.4.0: lce_problem.w_layout (weight and dW stored (V, H))
 
 const char* lce_strerror(int status) {
   switch (status) {
@@ -522,6 +532,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.Np = lce::padded_tokens(p->N); a.Hp = lce::padded_hidden(p->H);
   a.ldx = p->ldx; a.ldw = p->ldw; a.lddx = p->lddx; a.lddw = p->lddw;
   a.x_dtype = p->x_dtype; a.w_dtype = p->w_dtype; a.dx_dtype = p->dx_dtype; a.dw_dtype = p->dw_dtype;
+  a.w_vh = p->w_layout == LCE_W_VH;
   a.ignore_index = p->ignore_index;
   a.scale = p->logit_scale; a.z_reg = p->z_reg;
   a.dx = dx; a.dw = dw;
@@ -582,11 +593,13 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     if (p->w_dtype == LCE_F32) {
       // dz and dx of this slab read a 16-bit copy of its columns of the fp32 weight
       if ((ph & LCE_PHASE_BWD_DZ) || (dx && (ph & LCE_PHASE_BWD_DX))) {
-        e = lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, a.v0, a.vw, base + b.w16, a.vs, compute_dtype(p),
-                                       split, s);
+        e = a.w_vh ? lce::launch_convert_w_rows((const float*)w, p->ldw, p->H, a.v0, a.vw, base + b.w16, p->H,
+                                                compute_dtype(p), s)
+                   : lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, a.v0, a.vw, base + b.w16, a.vs,
+                                                compute_dtype(p), split, s);
         if (e != hipSuccess) return hip_fail(e, "convert_w");
       }
-      a.w = base + b.w16; a.ldw = a.vs; a.w_dtype = compute_dtype(p); a.wv0 = a.v0; a.Vw = a.vw;
+      a.w = base + b.w16; a.ldw = a.w_vh ? p->H : a.vs; a.w_dtype = compute_dtype(p); a.wv0 = a.v0; a.Vw = a.vw;
     } else {
       a.wv0 = 0; a.Vw = p->V;
     }

@@ -7,6 +7,15 @@
 // in the output dtype after scaling by grad_out * logit_scale / n_valid
 // (ops.py:443-447, 810).  Only the tiles of a mostly idle last round of
 // workgroups are cut along K instead and summed by a second kernel (DwPlan).
+//
+// x is the P operand of the tile loop and dz the Q operand, for either layout of dW: bands of tiles that
+// span all of H then walk along the vocabulary, so that dz streams through once while the small x is re-read
+// (measured 5-7 % faster than the other way round).  What changes with the layout is which operand goes
+// to which side of the matrix instruction, i.e. which index runs along the accumulator registers:
+//   dW stored (H, V) row-major: dz feeds the A side, v runs along registers, a lane stores runs of 8 v for its h;
+//   dW stored (V, H) row-major (WVH): x feeds the A side, h runs along registers, a lane stores runs of 8 h for its v.
+#include <type_traits>
+
 #include "lce_gemm3.h"
 #include "lce_internal.h"
 
@@ -14,49 +23,154 @@ namespace lce {
 
 namespace {
 
-// `part` != null: this is a K segment of a tail tile (see DwPlan); its raw fp32 sum goes to that
-// 256(h) x 256(v) block, through the statements of the fp32 output path (another destination, row
-// stride and factor, no bounds) -- a separate code path behind a branch would read the accumulator twice.
-template <class T>
-LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
+// First row / column of tile (tp = h tile, tq = v tile of the slab) in the stored matrix, and the matrix' limits.
+template <bool WVH> struct DwTileGeom {
+  int64_t row0, col0, row_limit, col_limit;
+  LCE_DEV DwTileGeom(const BwdArgs& a, int tp, int tq) {
+    if (WVH) {
+      row0 = a.v0 + (int64_t)tq * kTile; row_limit = a.V;
+      col0 = (int64_t)tp * kTile;        col_limit = a.H;
+    } else {
+      row0 = (int64_t)tp * kTile;        row_limit = a.H;
+      col0 = a.v0 + (int64_t)tq * kTile; col_limit = a.V;
+    }
+  }
+};
+
+// dW stored (H, V) row-major: its rows are V elements apart (256 KiB for 16-bit data at V = 131072), and the
+// 32-byte pieces that the lanes of a wave hold for 32 different rows make poor use of the memory channels
+// (measured: the tile kernel 5-7 % slower than with the 4 KiB rows of the (V, H) layout).  So a wave stages its
+// own 128 (h) x 128 (v) sub-tile through a private 16 KiB slice of `scratch` (main-loop stage 1, idle during an
+// epilogue) in passes of 128 bytes per row -- two of 64 columns for 16-bit dW, four of 32 columns for fp32 dW --
+// and reads each pass back as whole 128-byte rows: dW leaves the compute unit as full lines.  Staging rows have
+// their 16-byte piece index XOR-ed by (row & 7) ^ ((row >> 3) & 1), as in the dz staging of lce_bwd_dz.hip; no
+// other wave is involved until the barrier at the end.
+constexpr int kDwSliceBytes = kWaveTile * 128;
+static_assert(4 * kDwSliceBytes <= kMainloopLds - kStageBytes, "four wave slices must fit beside one stage");
+
+template <class T, bool F32OUT>
+LCE_DEV void dw_store_rows_hv(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
   typedef typename elem_of<T>::type E;
-  const int64_t vl0 = (int64_t)tp * kTile, h0 = (int64_t)tq * kTile;
+  typedef typename std::conditional<F32OUT, float, E>::type O;
+  constexpr int kPasses = F32OUT ? 4 : 2, kPassCols = kWaveTile / kPasses, kPieceCols = 16 / (int)sizeof(O);
   const int tid = opaque_tid();
   const int lane = tid & 63, wave = tid >> 6;
-  const int wp = wave & 1, wq = wave >> 1;
+  const int wp = wave & 1, wq = wave >> 1;  // rows h come from the P half, columns v from the Q half
+  const int half = lane >> 5;
+  const float coef = final_factor_of(a);
+  char* mine = scratch + wave * kDwSliceBytes;
+  const int64_t h0 = (int64_t)tp * kTile + wp * kWaveTile;             // first row of this wave's sub-tile
+  const int64_t v0 = a.v0 + (int64_t)tq * kTile + wq * kWaveTile;      // its first column
+  O* out = reinterpret_cast<O*>(a.dw) + h0 * a.lddw + v0;
+#pragma unroll
+  for (int ph = 0; ph < kPasses; ++ph) {
+#pragma unroll
+    for (int rb = 0; rb < kNB; ++rb) {
+      const int row = rb * kBlk + (lane & 31);
+      char* lrow = mine + row * 128;
+      const int sw = (row & 7) ^ ((row >> 3) & 1);
+      if (F32OUT) {
+        // one 32-column block per pass; a register quad is a 16-byte piece as it stands
+        const f32x16_t& blk = acc[rb][ph];
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          f32x4_t o;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o[j] = blk[rq * 4 + j] * coef;
+          *reinterpret_cast<f32x4_t*>(lrow + (((2 * rq + half) ^ sw) << 4)) = o;
+        }
+      } else {
+#pragma unroll
+        for (int pp = 0; pp < 2; ++pp) {
+          const f32x16_t& blk = acc[rb][2 * ph + pp];
+#pragma unroll
+          for (int gq = 0; gq < 4; gq += 2) {
+            // lanes l and l+32 hold the two halves of every run of 8 columns: one lane-half swap per pair of
+            // register quads gives each lane a whole run (16 bytes)
+            float d[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d[i] = blk[gq * 4 + i] * coef;
+            const unsigned x0 = pack2<T>(d[0], d[1]), x1 = pack2<T>(d[2], d[3]);
+            const unsigned y0 = pack2<T>(d[4], d[5]), y1 = pack2<T>(d[6], d[7]);
+            const auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+            u32x4_t o;
+            o[0] = s0[0];
+            o[1] = s1[0];
+            o[2] = s0[1];
+            o[3] = s1[1];
+            const int chunk = pp * 4 + gq + half;  // 16-byte piece of the 64-column pass
+            *reinterpret_cast<u32x4_t*>(lrow + ((chunk ^ sw) << 4)) = o;
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);  // (keeps the register footprint small: an operand tile is in flight)
+    }
+    // read the pass back as 128-byte rows and send it out: 8 rows per instruction, 8 lanes each; the upper 32
+    // lanes take their four rows in the order 5, 4, 7, 6 so that lanes l and l+32 sit in rows of opposite parity
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = i * 8 + (lane >> 3) + ((lane >> 5) ? 1 - 2 * ((lane >> 3) & 1) : 0), chunk = lane & 7;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * 128 + ((chunk ^ (row & 7) ^ ((row >> 3) & 1)) << 4));
+      // Pieces (8 columns of 16-bit data, 4 of fp32) that start at or past V are not stored; one that V cuts
+      // through is written whole, into the stride padding of its row.  (Streaming store: nothing reads dW back.)
+      const int64_t col = ph * kPassCols + chunk * kPieceCols;
+      if (h0 + row < a.H && v0 + col < a.V)
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + (int64_t)row * a.lddw + col));
+      if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most 4 rows in registers at a time
+    }
+  }
+  __syncthreads();  // scratch is handed back to the main loop
+}
+
+// acc[pb][qb] is the block of P block pb (h) and Q block qb (v).  The index fed to the B side of the matrix
+// instruction runs along lanes and is the row of the stored matrix; the other runs along registers (runs of 8
+// per lane pair) and is the column: WVH rows = v (Q), columns = h (P); otherwise rows = h (P), columns = v (Q).
+// `part` != null: this is a K segment of a tail tile (see DwPlan); its raw fp32 sum goes to that
+// 256 (rows) x 256 (columns) block, through the statements of the fp32 output path (another destination, row
+// stride and factor, no bounds) -- a separate code path behind a branch would read the accumulator twice.
+template <class T, bool WVH>
+LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
+  typedef typename elem_of<T>::type E;
+  const DwTileGeom<WVH> g(a, tp, tq);
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wp = wave & 1, wq = wave >> 1;          // this wave's half of the P and of the Q extent
+  const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
   const bool tail = part != nullptr;
   const float coef = tail ? 1.f : final_factor_of(a);
-  // fp32 destination addressed as [h][v] with v counted over the whole vocabulary
-  float* f32dst = tail ? part - (h0 * kTile + a.v0 + vl0) : reinterpret_cast<float*>(a.dw);
+  // fp32 destination addressed as [row][col] of the whole stored matrix
+  float* f32dst = tail ? part - (g.row0 * kTile + g.col0) : reinterpret_cast<float*>(a.dw);
   const int64_t f32ld = tail ? kTile : a.lddw;
   const int half = lane >> 5;
 #pragma unroll
-  for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t h = h0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-    const bool row_exists = h < a.H;
+  for (int rb = 0; rb < kNB; ++rb) {
+    const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + (lane & 31);
+    const bool row_exists = row < g.row_limit;
 #pragma unroll
-    for (int pb = 0; pb < kNB; ++pb) {
-      const int64_t vb = a.v0 + vl0 + wp * kWaveTile + pb * kBlk;
-      // Pieces (4 columns in fp32, 8 in the 16-bit types) that start at or past V are not
-      // stored; one that V cuts through is written whole, into the stride padding of its row.
+    for (int cbk = 0; cbk < kNB; ++cbk) {
+      const f32x16_t& blk = WVH ? acc[cbk][rb] : acc[rb][cbk];
+      const int64_t cb = g.col0 + w_col * kWaveTile + cbk * kBlk;
+      // Pieces (4 columns in fp32, 8 in the 16-bit types) that start at or past the last column are not
+      // stored; one that it cuts through is written whole, into the stride padding of its row.
       if (a.dw_dtype == DT_F32 || tail) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-          if (!tail && (vb + 8 * rq + 4 * half >= a.V || !row_exists)) continue;
+          if (!tail && (cb + 8 * rq + 4 * half >= g.col_limit || !row_exists)) continue;
           f32x4_t o;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) o[j] = acc[pb][qb][rq * 4 + j] * coef;
-          *reinterpret_cast<f32x4_t*>(f32dst + h * f32ld + vb + 8 * rq + 4 * half) = o;
+          for (int j = 0; j < 4; ++j) o[j] = blk[rq * 4 + j] * coef;
+          *reinterpret_cast<f32x4_t*>(f32dst + row * f32ld + cb + 8 * rq + 4 * half) = o;
         }
       } else {
         // Lanes l and l+32 hold the two halves of every run of 8 columns; one
         // lane-half swap per pair of register quads gives each lane a whole run,
         // so a store writes 32 contiguous bytes (a full sector) per row of dW.
 #pragma unroll
-        for (int g = 0; g < 4; g += 2) {
+        for (int gq = 0; gq < 4; gq += 2) {
           float d[8];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) d[i] = acc[pb][qb][g * 4 + i] * coef;
+          for (int i = 0; i < 8; ++i) d[i] = blk[gq * 4 + i] * coef;
           const unsigned x0 = pack2<T>(d[0], d[1]), x1 = pack2<T>(d[2], d[3]);
           const unsigned y0 = pack2<T>(d[4], d[5]), y1 = pack2<T>(d[6], d[7]);
           const auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
@@ -66,8 +180,8 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
           o[1] = s1[0];
           o[2] = s0[1];
           o[3] = s1[1];
-          if (vb + 8 * (g + half) < a.V && row_exists)
-            *reinterpret_cast<u32x4_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + vb + 8 * (g + half)) = o;
+          if (cb + 8 * (gq + half) < g.col_limit && row_exists)
+            *reinterpret_cast<u32x4_t*>(reinterpret_cast<E*>(a.dw) + row * a.lddw + cb + 8 * (gq + half)) = o;
         }
       }
     }
@@ -108,25 +222,40 @@ LCE_DEV DwPlan dw_plan(const BwdArgs& a, int64_t rows) {
   return p;
 }
 
-template <class T> struct DwProblem {
+// Which work items of the plan a launch covers, and how whole tiles leave the registers.  A kernel holds one
+// epilogue only: two of them behind a run-time branch make the compiler read all 256 accumulator registers for
+// both arms at once.
+//   kDwAll       every item, direct stores (dW stored (V, H))
+//   kDwStaged    whole tiles only, stored as full lines through LDS (16-bit dW stored (H, V))
+//   kDwStaged32  the same for fp32 dW
+//   kDwTails     the K segments of the tail tiles only (their launch follows that of the whole tiles)
+enum { kDwAll = 0, kDwStaged = 1, kDwTails = 2, kDwStaged32 = 3 };
+
+template <class T, bool WVH, int MODE> struct DwProblem {
+  static constexpr bool kSwapAB = !WVH;  // (H, V) output: dz, the Q operand, feeds the A side (v along registers)
   static constexpr bool kVarK = true;    // whole tiles and segment items have different K extents
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows (the K extent): all of x, or the packed rows (see BwdArgs)
   const E* x;
-  int tiles_p, tiles_q;
+  int tiles_p, tiles_q;  // P = x: tiles over h; Q = dz: tiles over the columns of the slab
   DwPlan plan;
-  LCE_DEV DwProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.vs / kTile)), tiles_q((int)(a_.Hp / kTile)) {
+  int first, count;      // this launch's items of the plan: [first, first + count)
+  LCE_DEV DwProblem(const BwdArgs& a_) : a(a_), tiles_p((int)(a_.Hp / kTile)), tiles_q((int)(a_.vs / kTile)) {
     rows = packed_rows(a.n_rows, a.N);
     const bool packed = rows != a.N;
     x = reinterpret_cast<const E*>(packed ? a.xc : a.x);
     ldx = packed ? a.ldxc : a.ldx;
     plan = dw_plan(a, rows);
+    const int tails = plan.tail_tiles * plan.nseg;
+    first = MODE == kDwTails ? plan.full : 0;
+    count = MODE == kDwAll ? plan.full + tails : (MODE == kDwTails ? tails : plan.full);
   }
-  LCE_DEV int num_tiles() const { return plan.full + plan.tail_tiles * plan.nseg; }
-  // seg < 0: a whole tile
-  LCE_DEV void decode(int item, int& tp, int& tq, int& seg) const {
+  LCE_DEV int num_tiles() const { return count; }
+  // `local` counts this launch's items; seg < 0: a whole tile
+  LCE_DEV void decode(int local, int& item, int& tp, int& tq, int& seg) const {
+    item = first + local;
     int tile = item;
     seg = -1;
     if (item >= plan.full) {
@@ -136,92 +265,108 @@ template <class T> struct DwProblem {
     }
     tile_coords(tile, plan.tiles, tiles_p, tiles_q, 8, tp, tq);
   }
-  LCE_DEV int item_ktiles(int item) const { return item < plan.full ? plan.kt : plan.kseg; }
-  LCE_DEV void origins(int item, const void*& p, const void*& q) const {
-    int tp, tq, seg;
-    decode(item, tp, tq, seg);
+  LCE_DEV int item_ktiles(int local) const { return first + local < plan.full ? plan.kt : plan.kseg; }
+  LCE_DEV void origins(int local, const void*& p, const void*& q) const {
+    int item, tp, tq, seg;
+    decode(local, item, tp, tq, seg);
     const int64_t k0 = seg < 0 ? 0 : (int64_t)seg * plan.kseg * kBK;  // first token of the segment
-    p = reinterpret_cast<const E*>(a.dz) + k0 * a.vs + (int64_t)tp * kTile;
-    q = x + k0 * ldx + (int64_t)tq * kTile;
+    p = x + k0 * ldx + (int64_t)tp * kTile;
+    q = reinterpret_cast<const E*>(a.dz) + k0 * a.vs + (int64_t)tq * kTile;
   }
-  // dz is written for whole token tiles; x rows past the last one read as zeros
-  LCE_DEV const void* p_end() const {
+  // x rows past the last one read as zeros; dz is written for whole token tiles
+  LCE_DEV const void* p_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
+  LCE_DEV const void* q_end() const {
     return reinterpret_cast<const E*>(a.dz) + (rows + kTile - 1) / kTile * kTile * a.vs;
   }
-  LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.Np; }
-  LCE_DEV void epilogue(int item, f32x16_t (&acc)[kNB][kNB], char*) const {
-    int tp, tq, seg;
-    decode(item, tp, tq, seg);
-    float* part = seg >= 0 ? a.dw_part + (int64_t)(item - plan.full) * kTile * kTile : nullptr;
-    dw_epilogue<T>(a, part, acc, tp, tq);
+  LCE_DEV void epilogue(int local, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
+    int item, tp, tq, seg;
+    decode(local, item, tp, tq, seg);
+    if (MODE == kDwStaged || MODE == kDwStaged32) {
+      dw_store_rows_hv<T, MODE == kDwStaged32>(a, acc, tp, tq, scratch);
+    } else {
+      float* part = seg >= 0 ? a.dw_part + (int64_t)(item - plan.full) * kTile * kTile : nullptr;
+      dw_epilogue<T, WVH>(a, part, acc, tp, tq);
+    }
   }
 };
 
-template <class T>
+template <class T, bool WVH, int MODE>
 __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DwProblem<T> prob(a);
-  Pipe3<T, E, false, E, false, DwProblem<T>> pipe(prob);
-  pipe.run(a.vs, prob.ldx, prob.plan.kt, lds);
+  DwProblem<T, WVH, MODE> prob(a);
+  Pipe3<T, E, false, E, false, DwProblem<T, WVH, MODE>> pipe(prob);
+  pipe.run(prob.ldx, a.vs, prob.plan.kt, lds);
 }
 
-// Second step for the tail tiles: kTailParts workgroups share tail tile b (16 rows of h each) -- they sum
-// its segments in order, scale, and store dW[:, slab] in the output dtype.
+// Second step for the tail tiles: kTailParts workgroups share tail tile b (16 of its rows each) -- they sum
+// its segments in order, scale, and store the tile of dW in the output dtype.
 constexpr int kTailParts = 16;
-template <class T>
+template <class T, bool WVH>
 __global__ __launch_bounds__(256) void dw_tail_kernel(const BwdArgs a) {
   typedef typename elem_of<T>::type E;
   const DwPlan plan = dw_plan(a, packed_rows(a.n_rows, a.N));
   const int b = (int)blockIdx.x / kTailParts, piece = (int)blockIdx.x % kTailParts;
   if (b >= plan.tail_tiles) return;
   int tp, tq;
-  tile_coords(plan.full + b, plan.tiles, (int)(a.vs / kTile), (int)(a.Hp / kTile), 8, tp, tq);
+  tile_coords(plan.full + b, plan.tiles, (int)(a.Hp / kTile), (int)(a.vs / kTile), 8, tp, tq);
+  const DwTileGeom<WVH> g(a, tp, tq);
   const float coef = final_factor_of(a);
   const float* part = a.dw_part + (int64_t)b * plan.nseg * kTile * kTile;
   constexpr int kQuads = kTile * kTile / 4 / kTailParts;
   for (int i = piece * kQuads + threadIdx.x; i < (piece + 1) * kQuads; i += 256) {
-    const int row = i / (kTile / 4), vl = (i - row * (kTile / 4)) * 4;
-    const int64_t h = (int64_t)tq * kTile + row, v = a.v0 + (int64_t)tp * kTile + vl;
-    if (h >= a.H || v >= a.V) continue;  // a quad that V cuts through is written whole, into the stride padding of its row
-    f32x4_t acc = *reinterpret_cast<const f32x4_t*>(part + row * kTile + vl);
+    const int r = i / (kTile / 4), c = (i - r * (kTile / 4)) * 4;
+    const int64_t row = g.row0 + r, col = g.col0 + c;
+    if (row >= g.row_limit || col >= g.col_limit) continue;  // a quad that the last column cuts through is written whole, into the stride padding of its row
+    f32x4_t acc = *reinterpret_cast<const f32x4_t*>(part + r * kTile + c);
 #pragma unroll 4
     for (int s = 1; s < plan.nseg; ++s)
-      acc += *reinterpret_cast<const f32x4_t*>(part + (int64_t)s * kTile * kTile + row * kTile + vl);
+      acc += *reinterpret_cast<const f32x4_t*>(part + (int64_t)s * kTile * kTile + r * kTile + c);
     if (a.dw_dtype == DT_F32) {
-      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + h * a.lddw + v) = acc * coef;
+      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + row * a.lddw + col) = acc * coef;
     } else {
       u32x2_t o;
       o[0] = pack2<T>(acc[0] * coef, acc[1] * coef);
       o[1] = pack2<T>(acc[2] * coef, acc[3] * coef);
-      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dw) + h * a.lddw + v) = o;
+      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dw) + row * a.lddw + col) = o;
     }
   }
 }
 
-template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dw_persistent_kernel<T>;
+template <class T, bool WVH, int MODE> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dw_persistent_kernel<T, WVH, MODE>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(a.dw_grid), dim3(kThreads), kMainloopLds, s, a);
-  e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  if (a.dw_part == nullptr || dw_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // this launch cannot have a split tail
-  // (the tile count does not depend on the rows: no second kernel when the last round is not split)
-  if (!has_split_tail((a.vs / kTile) * (a.Hp / kTile), a.dw_grid)) return hipSuccess;
+  return hipGetLastError();
+}
+
+template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  // a last round of tiles may be split along K (the tile count does not depend on the rows; whether its K
+  // extent is long enough to split is decided on the device, and a launch without items returns at once)
+  const bool tails = a.dw_part != nullptr && dw_tail_blocks(a.Np, a.Hp, a.vs) != 0 &&
+                     has_split_tail((a.vs / kTile) * (a.Hp / kTile), a.dw_grid);
+  hipError_t e;
+  if constexpr (WVH) {
+    e = launch_tiles<T, true, kDwAll>(a, s);
+  } else {
+    e = a.dw_dtype == DT_F32 ? launch_tiles<T, false, kDwStaged32>(a, s) : launch_tiles<T, false, kDwStaged>(a, s);
+    if (e == hipSuccess && tails) e = launch_tiles<T, false, kDwTails>(a, s);
+  }
+  if (e != hipSuccess || !tails) return e;
   // at most dw_grid / 2 tail tiles can be split (two segments each)
   const unsigned tail_most = (unsigned)(a.dw_grid / 2 > 0 ? a.dw_grid / 2 : 1);
-  hipLaunchKernelGGL(dw_tail_kernel<T>, dim3(tail_most * kTailParts), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((dw_tail_kernel<T, WVH>), dim3(tail_most * kTailParts), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s) {
-  if (a.x_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
-  if (a.x_dtype == DT_F16) return launch_persistent<F16>(a, s);
+  if (a.x_dtype == DT_BF16) return a.w_vh ? launch_persistent<BF16, true>(a, s) : launch_persistent<BF16, false>(a, s);
+  if (a.x_dtype == DT_F16) return a.w_vh ? launch_persistent<F16, true>(a, s) : launch_persistent<F16, false>(a, s);
   return hipErrorInvalidValue;
 }
 

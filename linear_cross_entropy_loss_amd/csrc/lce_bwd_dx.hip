@@ -119,8 +119,11 @@ LCE_DEV DxPlan dx_plan(const BwdArgs& a, int tiles) {
   return p;
 }
 
-template <class T, bool KMASK> struct DxProblem {
+// WVH: the weight is stored (V, H) row-major: the P tile then has K = v as its slow index (read through the
+// LDS transpose path) and only dz, the K-contiguous operand, carries the K mask.
+template <class T, bool KMASK, bool WVH> struct DxProblem {
   static constexpr bool kKMask = KMASK;
+  static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = true;  // whole tiles and segment items have different K extents
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
@@ -149,10 +152,13 @@ template <class T, bool KMASK> struct DxProblem {
     int tp, tq, seg;
     decode(item, tp, tq, seg);
     const int64_t k0 = k0_of(seg);
-    p = reinterpret_cast<const E*>(a.w) + (int64_t)tp * kTile * a.ldw + (a.v0 - a.wv0) + k0;
+    p = WVH ? reinterpret_cast<const E*>(a.w) + ((a.v0 - a.wv0) + k0) * a.ldw + (int64_t)tp * kTile
+            : reinterpret_cast<const E*>(a.w) + (int64_t)tp * kTile * a.ldw + (a.v0 - a.wv0) + k0;
     q = reinterpret_cast<const E*>(a.dz) + (int64_t)tq * kTile * a.vs + k0;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<E>(a.w, a.H, a.ldw, a.Vw); }
+  LCE_DEV const void* p_end() const {
+    return WVH ? matrix_end<E>(a.w, a.Vw, a.ldw, a.H) : matrix_end<E>(a.w, a.H, a.ldw, a.Vw);
+  }
   LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + (int64_t)tiles_q * kTile * a.vs; }
   LCE_DEV int k_valid(int item) const {
     int tp, tq, seg;
@@ -170,12 +176,12 @@ template <class T, bool KMASK> struct DxProblem {
   }
 };
 
-template <class T, bool KMASK>
+template <class T, bool KMASK, bool WVH>
 __global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DxProblem<T, KMASK> prob(a);
-  Pipe3<T, E, true, E, true, DxProblem<T, KMASK>> pipe(prob);
+  DxProblem<T, KMASK, WVH> prob(a);
+  Pipe3<T, E, !WVH, E, true, DxProblem<T, KMASK, WVH>> pipe(prob);
   pipe.run(a.ldw, a.vs, (int)(a.vs / kBK), lds);
 }
 
@@ -225,8 +231,8 @@ __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
   }
 }
 
-template <class T, bool KMASK> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dx_persistent_kernel<T, KMASK>;
+template <class T, bool KMASK, bool WVH> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dx_persistent_kernel<T, KMASK, WVH>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -237,7 +243,8 @@ template <class T, bool KMASK> hipError_t launch_tiles(const BwdArgs& a, hipStre
 template <class T> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
   // the K mask is only needed when the K tiles of a work item can run past the columns that exist
   const bool exact_k = a.vw == a.vs && dx_segments_exact(a.vs);
-  hipError_t e = exact_k ? launch_tiles<T, false>(a, s) : launch_tiles<T, true>(a, s);
+  hipError_t e = a.w_vh ? (exact_k ? launch_tiles<T, false, true>(a, s) : launch_tiles<T, true, true>(a, s))
+                        : (exact_k ? launch_tiles<T, false, false>(a, s) : launch_tiles<T, true, false>(a, s));
   if (e != hipSuccess) return e;
   if (a.dx_part == nullptr || dx_tail_blocks(a.Np, a.Hp, a.vs) == 0) return hipSuccess;  // no shape of this launch can have a split tail
   // without packed rows the tile count is known here: no second kernel when its last round is not split

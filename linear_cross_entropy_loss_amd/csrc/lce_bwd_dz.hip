@@ -184,9 +184,11 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
 // The launch covers `tiles_p` tile columns of the slab starting at column tile
 // `tp0`: all the full ones, or (VTAIL) those from the one straddling the end
 // of the vocabulary to the end of the padded slab.
-template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT> struct DzProblem {
+// WVH: the weight is stored (V, H) row-major, so that the P operand runs along K in memory like x does.
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> struct DzProblem {
   typedef typename elem_of<T>::type E;
   static constexpr bool kKMask = KMASK;
+  static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows: all of x, or the packed rows (see BwdArgs)
@@ -211,10 +213,13 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT> struct DzProbl
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     coords(tile, tp, tq);
-    p = reinterpret_cast<const E*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
+    const int64_t v = (a.v0 - a.wv0) + (int64_t)tp * kTile;  // first column of the tile inside the buffer `w`
+    p = reinterpret_cast<const E*>(a.w) + (WVH ? v * a.ldw : v);
     q = x + (int64_t)tq * kTile * ldx;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<E>(a.w, a.H, a.ldw, a.Vw); }
+  LCE_DEV const void* p_end() const {
+    return WVH ? matrix_end<E>(a.w, a.Vw, a.ldw, a.H) : matrix_end<E>(a.w, a.H, a.ldw, a.Vw);
+  }
   LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
@@ -224,18 +229,18 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT> struct DzProbl
   }
 };
 
-template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT>
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH>
 __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DzProblem<T, ZREG, VTAIL, KMASK, SPLIT> prob(a);
-  Pipe3<T, E, false, E, true, DzProblem<T, ZREG, VTAIL, KMASK, SPLIT>> pipe(prob);
+  DzProblem<T, ZREG, VTAIL, KMASK, SPLIT, WVH> prob(a);
+  Pipe3<T, E, WVH, E, true, DzProblem<T, ZREG, VTAIL, KMASK, SPLIT, WVH>> pipe(prob);
   pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
-template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT>
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH>
 hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = bwd_dz_persistent_kernel<T, ZREG, VTAIL, KMASK, SPLIT>;
+  auto kern = bwd_dz_persistent_kernel<T, ZREG, VTAIL, KMASK, SPLIT, WVH>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e != hipSuccess) return e;
@@ -245,29 +250,35 @@ hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
 }
 
 // All full tile columns of the slab, then the column that straddles the end of the vocabulary.
-template <class T, bool ZREG, bool SPLIT> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
+template <class T, bool ZREG, bool SPLIT, bool WVH> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
   const int64_t tq = a.Np / kTile, full = a.vw / kTile, tail = a.vs / kTile - full;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = exact_k ? launch_one<T, ZREG, false, false, SPLIT>(a, full * tq, s)
-                           : launch_one<T, ZREG, false, true, SPLIT>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, ZREG, false, false, SPLIT, WVH>(a, full * tq, s)
+                           : launch_one<T, ZREG, false, true, SPLIT, WVH>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (tail > 0) return launch_one<T, ZREG, true, true, SPLIT>(a, tail * tq, s);
+  if (tail > 0) return launch_one<T, ZREG, true, true, SPLIT, WVH>(a, tail * tq, s);
   return hipSuccess;
 }
 
-template <class T, bool SPLIT> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
-  return a.z_reg != 0.f ? launch_persistent_z<T, true, SPLIT>(a, s)
-                        : launch_persistent_z<T, false, SPLIT>(a, s);
+template <class T, bool SPLIT, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  return a.z_reg != 0.f ? launch_persistent_z<T, true, SPLIT, WVH>(a, s)
+                        : launch_persistent_z<T, false, SPLIT, WVH>(a, s);
 }
 
 }  // namespace
 
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
+  if (a.w_vh) {  // (never with bf16 pairs)
+    if (a.split) return hipErrorInvalidValue;
+    if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16, false, true>(a, s);
+    if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, false, true>(a, s);
+    return hipErrorInvalidValue;
+  }
   if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16)
-    return a.split ? launch_persistent<BF16, true>(a, s) : launch_persistent<BF16, false>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, false>(a, s);
+    return a.split ? launch_persistent<BF16, true, false>(a, s) : launch_persistent<BF16, false, false>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, false, false>(a, s);
   // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as bf16 pairs with split set)
   return hipErrorInvalidValue;
 }

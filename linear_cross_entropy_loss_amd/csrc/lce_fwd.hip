@@ -156,9 +156,11 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
 // starting at its column tile `tp0` (all full columns, or the one straddling V
 // for the VTAIL variant).  The token rows are those of x, or -- when the tokens with ignored
 // labels were packed away -- the first `rows` rows of the packed copy (the count lives on the device).
-template <class T, bool VTAIL, bool KMASK> struct FwdProblem {
+// WVH: the weight is stored (V, H) row-major, so that the P operand runs along K in memory like x does.
+template <class T, bool VTAIL, bool KMASK, bool WVH> struct FwdProblem {
   typedef typename elem_of<T>::type E;
   static constexpr bool kKMask = KMASK;
+  static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
   const FwdArgs& a;
   int64_t rows, ldx;
@@ -183,10 +185,13 @@ template <class T, bool VTAIL, bool KMASK> struct FwdProblem {
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {
     int tp, tq;
     coords(tile, tp, tq);
-    p = reinterpret_cast<const E*>(a.w) + (a.v0 - a.wv0) + (int64_t)tp * kTile;
+    const int64_t v = (a.v0 - a.wv0) + (int64_t)tp * kTile;  // first column of the tile inside the buffer `w`
+    p = reinterpret_cast<const E*>(a.w) + (WVH ? v * a.ldw : v);
     q = x + (a.row0 + (int64_t)tq * kTile) * ldx;
   }
-  LCE_DEV const void* p_end() const { return matrix_end<E>(a.w, a.H, a.ldw, a.Vw); }
+  LCE_DEV const void* p_end() const {
+    return WVH ? matrix_end<E>(a.w, a.Vw, a.ldw, a.H) : matrix_end<E>(a.w, a.H, a.ldw, a.Vw);
+  }
   LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
@@ -196,12 +201,12 @@ template <class T, bool VTAIL, bool KMASK> struct FwdProblem {
   }
 };
 
-template <class T, bool VTAIL, bool KMASK>
+template <class T, bool VTAIL, bool KMASK, bool WVH>
 __global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  FwdProblem<T, VTAIL, KMASK> prob(a);
-  Pipe3<T, E, false, E, true, FwdProblem<T, VTAIL, KMASK>> pipe(prob);
+  FwdProblem<T, VTAIL, KMASK, WVH> prob(a);
+  Pipe3<T, E, WVH, E, true, FwdProblem<T, VTAIL, KMASK, WVH>> pipe(prob);
   pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
@@ -354,9 +359,9 @@ __global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
   }
 }
 
-template <class T, bool VTAIL, bool KMASK>
+template <class T, bool VTAIL, bool KMASK, bool WVH>
 hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = fwd_tiles_persistent_kernel<T, VTAIL, KMASK>;
+  auto kern = fwd_tiles_persistent_kernel<T, VTAIL, KMASK, WVH>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -366,24 +371,26 @@ hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
 }
 
 // All full tile columns of the vocabulary, then the column that straddles V.
-template <class T> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
+template <class T, bool WVH> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
   const int64_t left = a.Np - a.row0;  // token tiles of this chunk at most
   const int64_t tq = (left < a.nc ? left : a.nc) / kTile, full = a.vw / kTile;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = exact_k ? launch_one<T, false, false>(a, full * tq, s)
-                           : launch_one<T, false, true>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, false, false, WVH>(a, full * tq, s)
+                           : launch_one<T, false, true, WVH>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (a.vw % kTile) return launch_one<T, true, true>(a, tq, s);
+  if (a.vw % kTile) return launch_one<T, true, true, WVH>(a, tq, s);
   return hipSuccess;
 }
 
 }  // namespace
 
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return launch_persistent<BF16>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16>(a, s);
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16)
+    return a.w_vh ? launch_persistent<BF16, true>(a, s) : launch_persistent<BF16, false>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16)
+    return a.w_vh ? launch_persistent<F16, true>(a, s) : launch_persistent<F16, false>(a, s);
   // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as the bf16 packed copy)
   return hipErrorInvalidValue;
 }

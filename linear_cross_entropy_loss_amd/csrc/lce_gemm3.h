@@ -135,6 +135,9 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //   const void* p_end(), q_end()                  one past the last valid byte of each operand
 //   static constexpr bool kVarK                   true if work items differ in their number of K tiles; then
 //   int  item_ktiles(int tile)                    gives it (even, at least 4) -- otherwise run() is told once
+//   static constexpr bool kSwapAB                 false: P fragments feed the A side of the matrix instruction (the P index
+//        runs along accumulator registers, Q along lanes); true: the Q fragments do (acc[i][j] is still the block
+//        of P block i and Q block j, with Q along its registers and P along its lanes)
 //   static constexpr bool kKMask                  false if `ktiles * 64 == k_valid` for every tile of the launch
 //   int  k_valid(int tile)                        K extent of that tile's contraction; the K tiles of the
 //        loop may run past it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
@@ -235,7 +238,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
         } else {
           c = acc[i][j];
         }
-        acc[i][j] = mfma32<T>(pf[buf][i], qf[buf][j], c);
+        acc[i][j] = Problem::kSwapAB ? mfma32<T>(qf[buf][j], pf[buf][i], c) : mfma32<T>(pf[buf][i], qf[buf][j], c);
       }
   }
 

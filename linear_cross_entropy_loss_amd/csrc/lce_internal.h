@@ -38,6 +38,9 @@ struct FwdArgs {
   // window of W that the buffer `w` holds: columns [wv0, wv0 + Vw) of the weight, row stride ldw.
   // (`w` is the caller's matrix, wv0 = 0, Vw = V -- or a 16-bit copy of one slab of an fp32 weight.)
   int64_t v0, vw, wv0, Vw;
+  // w_vh != 0: the weight is stored with the vocabulary as its row index, w[v * ldw + h] (the buffer `w` then
+  // holds ROWS [wv0, wv0 + Vw)); otherwise w[h * ldw + v].
+  int w_vh;
   int x_dtype, w_dtype;  // compute type = x_dtype (bf16 / f16)
   int64_t ignore_index;
   float scale, z_reg;
@@ -81,6 +84,9 @@ struct BwdArgs {
   int64_t v0, vs;   // first column and padded width (multiple of 256) of the vocabulary slab
   int64_t vw;       // columns of the slab that exist: min(vs, V - v0)
   int64_t wv0, Vw;  // `w` holds columns [wv0, wv0 + Vw) of the weight (the whole matrix, or a 16-bit copy of this slab)
+  // w_vh != 0: weight and dW are stored with the vocabulary as their row index, w[v * ldw + h], dw[v * lddw + h]
+  // (and the buffer `w` holds ROWS [wv0, wv0 + Vw)); otherwise w[h * ldw + v], dw[h * lddw + v].
+  int w_vh;
   void* dz;         // [Np][vs] staged dz in the compute type (exact zeros outside N x vw)
   float* dx_acc;    // [Np][Hp] fp32 running dx (null when there is a single slab)
   // dx: tiles of a last, mostly idle round of workgroups are cut along K instead (planned on the device,
@@ -138,6 +144,9 @@ hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
 // compute_dtype: DT_BF16 or DT_F16.  split: dst has 3 H rows, [bf16 hi ; bf16 lo ; bf16 hi] of the fp32 values.
 hipError_t launch_convert_w_slab(const float* src, int64_t ld, int64_t H, int64_t v0, int64_t vw, void* dst,
                                  int64_t dst_ld, int compute_dtype, bool split, hipStream_t s);
+// The same for a weight stored (V, H) row-major (H a multiple of 8): rows [v0, v0 + vw) go to dst[vw][dst_ld].
+hipError_t launch_convert_w_rows(const float* src, int64_t ld, int64_t H, int64_t v0, int64_t vw, void* dst,
+                                 int64_t dst_ld, int compute_dtype, hipStream_t s);
 
 // Row count / row -> token map of the packed rows as the kernels read them from device memory, forced
 // into range: a call restricted to some phases on a workspace whose packing pre-pass did not run must

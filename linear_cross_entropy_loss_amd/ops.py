@@ -70,6 +70,29 @@ def _aligned_rows(t):
     return padded[:, :cols]
 
 
+def _weight_layout(At, x_dtype):
+    """_lib.W_VH when `At` (H, V) is the transposed view of a row-major (V, H) matrix -- a tied embedding or
+    an ``nn.Linear(H, V)`` weight handed over as ``weight.T`` -- that the kernels can read in place, as the
+    reference's kernels do through At's strides (ops.py:733-734); else _lib.W_HV.  Decided from shape,
+    strides and dtypes alone, so that a traced (fake) tensor gives the same answer."""
+    H, V = At.shape
+    m = _row_multiple(At.dtype)
+    if At.stride(1) == 1 and At.stride(0) % m == 0 and At.stride(0) >= V:
+        return _lib.W_HV  # row-major (H, V): read in place
+    if (x_dtype != torch.float32 and H % 8 == 0 and V > 1 and At.stride(0) == 1 and At.stride(1) % m == 0
+            and At.stride(1) >= H):
+        return _lib.W_VH
+    return _lib.W_HV  # any other striding: copied into a row-major (H, V) matrix
+
+
+def _weight_rows(At, layout):
+    """The matrix the kernels read: (H, V) rows for W_HV, (V, H) rows for W_VH (no copy unless misaligned)."""
+    if layout == _lib.W_VH:
+        w = At.t()
+        return w if w.data_ptr() % 16 == 0 else w.clone(memory_format=torch.contiguous_format)
+    return _aligned_rows(At)
+
+
 def _empty_rows(rows, cols, dtype, device):
     """Uninitialised (rows, cols) matrix whose row stride satisfies the kernels' alignment rule."""
     m = 8  # gradients are stored in pieces of up to 8 elements
@@ -105,22 +128,24 @@ def _check_dtypes(x, At):
 
 
 def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack):
-    """Runs lce_forward.  Returns (out5, lse, n_valid) and the (x, y, w) views the kernels read."""
+    """Runs lce_forward.  Returns (out5, lse, n_valid), the (x, y, w) views the kernels read and w's layout."""
     _check_inputs(x_in, y, At)
     _check_dtypes(x_in, At)
     with torch.cuda.device(x_in.device):
         x = _aligned_rows(x_in.reshape(-1, x_in.shape[-1]))
         y1 = y.reshape(-1).contiguous()
-        w = _aligned_rows(At)
         N, H = x.shape
-        H_A, V = w.shape
+        H_A, V = At.shape
         if H_A != H:
             raise ValueError(f"weight has in_features={H_A}, input has {H}")
         if y1.shape != (N,):
             raise ValueError("labels must have one entry per input row")
+        layout = _weight_layout(At, x.dtype)
+        w = _weight_rows(At, layout)
+        lddw = (H if layout == _lib.W_VH else V + (-V) % 8)  # (not used by the forward)
         prob = _lib.make_problem(
-            N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-            ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring, 0, pack,
+            N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, lddw, x.dtype, w.dtype, x.dtype, w.dtype,
+            ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring, 0, pack, 0, layout,
         )
         lib = _lib.load()
         _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")
@@ -135,23 +160,26 @@ def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_ch
                              _ptr(n_valid), _ptr(ws), fwd_bytes, ctypes.c_void_p(stream))
         _lib.raise_for_status(rc, "lce_forward")
         del ws
-    return out5, lse, n_valid, x, y1, w
+    return out5, lse, n_valid, x, y1, w, layout
 
 
 def _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,
-                   N_chunk_size, need_dx, need_dw, pack):
-    """Runs lce_backward on what _forward_impl returned.  dx is (N, H), dw is (H, V); None when not needed."""
+                   N_chunk_size, need_dx, need_dw, pack, layout=0):
+    """Runs lce_backward on what _forward_impl returned.  dx is (N, H); dw is (H, V) -- for a weight stored
+    (V, H) (layout W_VH) the transposed view of a gradient stored the same way; None when not needed."""
     N, H = x.shape
-    V = w.shape[1]
+    vh = layout == _lib.W_VH
+    V = w.shape[0] if vh else w.shape[1]
+    w_cols = H if vh else V
     with torch.cuda.device(x.device):
         dev = x.device
         dx = _empty_rows(N, H, x.dtype, dev) if need_dx else None
-        dw = _empty_rows(H, V, w.dtype, dev) if need_dw else None
+        dw = (_empty_rows(V, H, w.dtype, dev) if vh else _empty_rows(H, V, w.dtype, dev)) if need_dw else None
         if need_dx or need_dw:
             prob = _lib.make_problem(
                 N, H, V, x.stride(0), w.stride(0), dx.stride(0) if need_dx else H + (-H) % 8,
-                dw.stride(0) if need_dw else V + (-V) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-                ignore_index, logit_scale, z_regularization, N_chunk_size, False, 0, pack,
+                dw.stride(0) if need_dw else w_cols + (-w_cols) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
+                ignore_index, logit_scale, z_regularization, N_chunk_size, False, 0, pack, 0, layout,
             )
             lib = _lib.load()
             _, bwd_bytes = _lib.workspace_bytes(prob)
@@ -166,6 +194,8 @@ def _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regulari
         dx = dx.contiguous()  # H not a multiple of 8
     if dw is not None and not dw.is_contiguous():
         dw = dw.contiguous()  # V not a multiple of 8
+    if dw is not None and vh:
+        dw = dw.t()
     return dx, dw
 
 
@@ -190,10 +220,10 @@ class LinearXentImplementation(torch.autograd.Function):
         # workspace.
         x_in = _autocast_x(x_in, At)
         pack = _pack_mode()
-        out5, lse, n_valid, x, y1, w = _forward_impl(
+        out5, lse, n_valid, x, y1, w, layout = _forward_impl(
             x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack)
         ctx.save_for_backward(x, y1, w, lse, n_valid)
-        ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size, pack)
+        ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size, pack, layout)
         ctx.x_shape = x_in.shape
         loss, z_reg, logit_max, logit_ent, logit_norm = out5.unbind(0)
         ctx.mark_non_differentiable(z_reg, logit_max, logit_ent, logit_norm)
@@ -203,9 +233,9 @@ class LinearXentImplementation(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output, void0=None, void1=None, void2=None, void3=None):
         x, y1, w, lse, n_valid = ctx.saved_tensors
-        ignore_index, z_regularization, logit_scale, N_chunk_size, pack = ctx.lce_cfg
+        ignore_index, z_regularization, logit_scale, N_chunk_size, pack, layout = ctx.lce_cfg
         dx, dw = _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,
-                                N_chunk_size, ctx.needs_input_grad[0], ctx.needs_input_grad[2], pack)
+                                N_chunk_size, ctx.needs_input_grad[0], ctx.needs_input_grad[2], pack, layout)
         if dx is not None:
             dx = dx.view(ctx.x_shape)
         return dx, None, dw, None, None, None, None, None
@@ -222,8 +252,8 @@ class LinearXentImplementation(torch.autograd.Function):
 def _op_forward(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, ignore_index: int, z_regularization: float,
                 logit_scale: float, N_chunk_size: int, monitoring: bool,
                 pack_rows_mode: int = 0) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    out5, lse, n_valid, _, _, _ = _forward_impl(x, y, At, ignore_index, z_regularization, logit_scale,
-                                                N_chunk_size, monitoring, pack_rows_mode)
+    out5, lse, n_valid, _, _, _, _ = _forward_impl(x, y, At, ignore_index, z_regularization, logit_scale,
+                                                   N_chunk_size, monitoring, pack_rows_mode)
     return out5, lse, n_valid
 
 
@@ -240,9 +270,10 @@ def _op_backward(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, lse: torch.
                  N_chunk_size: int, need_dx: bool, need_dw: bool,
                  pack_rows_mode: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
     x2 = _aligned_rows(x.reshape(-1, x.shape[-1]))
-    dx, dw = _backward_impl(x2, y.reshape(-1).contiguous(), _aligned_rows(At), lse, n_valid, grad_loss,
+    layout = _weight_layout(At, x2.dtype)
+    dx, dw = _backward_impl(x2, y.reshape(-1).contiguous(), _weight_rows(At, layout), lse, n_valid, grad_loss,
                             ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw,
-                            pack_rows_mode)
+                            pack_rows_mode, layout)
     dx = dx.view(x.shape) if dx is not None else x.new_empty((0,))
     dw = dw if dw is not None else At.new_empty((0,))
     return dx, dw
@@ -251,8 +282,13 @@ def _op_backward(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, lse: torch.
 @_op_backward.register_fake
 def _(x, y, At, lse, n_valid, grad_loss, ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw,
       pack_rows_mode=0):
-    return (torch.empty_like(x, memory_format=torch.contiguous_format) if need_dx else x.new_empty((0,)),
-            torch.empty_like(At, memory_format=torch.contiguous_format) if need_dw else At.new_empty((0,)))
+    if not need_dw:
+        dw = At.new_empty((0,))
+    elif _weight_layout(At, x.dtype) == _lib.W_VH:
+        dw = At.new_empty((At.shape[1], At.shape[0])).t()  # stored like the weight: (V, H) rows
+    else:
+        dw = torch.empty_like(At, memory_format=torch.contiguous_format)
+    return (torch.empty_like(x, memory_format=torch.contiguous_format) if need_dx else x.new_empty((0,))), dw
 
 
 def _op_setup_context(ctx, inputs, output):

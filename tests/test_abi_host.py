@@ -49,7 +49,7 @@ def test_struct_layout_matches_header():
     fields = re.findall(r"^\s*(int64_t|int32_t|float)\s+(\w+);", body, flags=re.M)
     ctype = {"int64_t": ctypes.c_int64, "int32_t": ctypes.c_int32, "float": ctypes.c_float}
     assert [(n, ctype[t]) for t, n in fields] == list(_lib.LceProblem._fields_)
-    assert ctypes.sizeof(_lib.LceProblem) == 7 * 8 + 4 * 4 + 8 + 2 * 4 + 8 + 4 * 4
+    assert ctypes.sizeof(_lib.LceProblem) == 7 * 8 + 4 * 4 + 8 + 2 * 4 + 8 + 6 * 4
 
 
 def test_shape_contract(lib):
@@ -408,3 +408,29 @@ def test_backward_plan_invariants_on_random_problems():
         split = 3 if xd == torch.float32 else 1
         slab_copy = (256 << 20) + 256 * H * 2 * split if wd == torch.float32 else 0
         assert fwd <= part + Np * 16 + N * (split * H + 8) * 2 + slab_copy + N * 16 + 8192, (it, fwd)
+
+
+def test_vocabulary_major_weight_layout_is_checked_and_detected():
+    """lce_problem.w_layout = LCE_W_VH: row strides are checked against H, fp32 activations and hidden sizes
+    that are not multiples of 8 are refused; the Python host picks the layout from the strides alone."""
+    from linear_cross_entropy_loss_amd import _lib, ops
+
+    lib = _lib.load()
+    ok = dict(N=512, H=256, V=1000, ldx=256, ldw=256, lddx=256, lddw=256, n_chunk=512, w_layout=_lib.W_VH)
+    assert lib.lce_check_problem(ctypes.byref(_prob(**ok))) == 0
+    assert _lib.workspace_bytes(_prob(**ok)) == _lib.workspace_bytes(_prob(**dict(ok, ldw=1000, lddw=1000, w_layout=_lib.W_HV)))
+    assert lib.lce_check_problem(ctypes.byref(_prob(**dict(ok, ldw=248)))) == _lib.LCE_EINVAL_ARG      # shorter than a row
+    assert lib.lce_check_problem(ctypes.byref(_prob(**dict(ok, w_layout=2)))) == _lib.LCE_EINVAL_ARG
+    assert lib.lce_check_problem(ctypes.byref(_prob(**dict(ok, H=252, ldx=256)))) == _lib.LCE_EINVAL_ARG  # H % 8
+    f32 = dict(ok, x_dtype=torch.float32, w_dtype=torch.float32, dx_dtype=torch.float32, dw_dtype=torch.float32)
+    assert lib.lce_check_problem(ctypes.byref(_prob(**f32))) == _lib.LCE_EINVAL_DTYPE
+    # a row-major (H, V) problem with the same numbers is refused for its strides (1000 columns need ldw >= 1000)
+    assert lib.lce_check_problem(ctypes.byref(_prob(**dict(ok, w_layout=_lib.W_HV)))) == _lib.LCE_EINVAL_ARG
+
+    w = torch.zeros(1000, 256, dtype=torch.bfloat16)     # (V, H) as a model stores it
+    assert ops._weight_layout(w.t(), torch.bfloat16) == _lib.W_VH
+    assert ops._weight_layout(w.t().contiguous(), torch.bfloat16) == _lib.W_HV
+    assert ops._weight_layout(w.t(), torch.float32) == _lib.W_HV                      # fp32 activations: copied
+    assert ops._weight_layout(torch.zeros(1000, 100, dtype=torch.bfloat16).t(), torch.bfloat16) == _lib.W_HV  # H % 8
+    assert ops._weight_layout(torch.zeros(1000, 264, dtype=torch.bfloat16)[:, :256].t(), torch.bfloat16) == _lib.W_VH
+    assert ops._weight_layout(torch.zeros(1000, 256, dtype=torch.float32).t(), torch.float16) == _lib.W_VH  # master weight
