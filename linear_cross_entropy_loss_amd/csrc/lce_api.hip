@@ -134,6 +134,11 @@ FwdPlan plan_fwd(const lce_problem* p) {
   f.blk = o; o += align_up(Np / lce::kMergeRows * 8 * sizeof(double));
   f.w16 = o;
   f.vs = (int64_t)Vp;
+  // A chunk of activations that does not fit the 256 MB Infinity Cache (more than 128 MiB of it) is streamed from
+  // memory by all eight XCDs; over a long launch they drift apart and stop sharing what they fetch.  Launches
+  // of 32768 columns bring them back in step (measured at N = 16384, H = 8192, V = 131072: 24.6 ms against 27.3
+  // in one launch; no difference at H = 2048, where x stays in the cache).
+  if ((size_t)f.nc * (size_t)p->H * 2 > ((size_t)128 << 20) && f.vs > 32768) f.vs = 32768;
   if (p->w_dtype == LCE_F32) {
     // slab copies of at most 256 MiB (at least one tile column)
     const int64_t hw = splits(p) ? 3 * p->H : p->H;  // rows of the copy
@@ -365,6 +370,7 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
   a.blk = (float*)(base + f.blk);
   rc = current_num_cus(&a.num_cus, p->max_workgroups);
   if (rc != LCE_OK) return rc;
+  a.live = lce::live_bands(lce::padded_k(splits(p) ? 3 * p->H : p->H) * 2);
 
   const int ph = p->phases ? p->phases : ~0;
   hipError_t e;
@@ -544,6 +550,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.dw_part = b.parts_on ? (float*)(base + b.dw_part) : nullptr;
   rc = current_num_cus(&a.num_cus, p->max_workgroups);
   if (rc != LCE_OK) return rc;
+  a.live = lce::live_bands(lce::padded_k(splits(p) ? 3 * p->H : p->H) * 2);
   const int ph = p->phases ? p->phases : ~0;
 
   // Tokens with an ignored label have dz == 0: the kernels run on the other rows only, packed to the front.

@@ -263,7 +263,7 @@ template <class T, bool WVH, int MODE> struct DwProblem {
       tile = plan.full + j / plan.nseg;
       seg = j % plan.nseg;
     }
-    tile_coords(tile, plan.tiles, tiles_p, tiles_q, 8, tp, tq);
+    tile_coords(tile, plan.tiles, tiles_p, tiles_q, 8, 8, tp, tq);
   }
   LCE_DEV int item_ktiles(int local) const { return first + local < plan.full ? plan.kt : plan.kseg; }
   LCE_DEV void origins(int local, const void*& p, const void*& q) const {
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(256) void dw_tail_kernel(const BwdArgs a) {
   const int b = (int)blockIdx.x / kTailParts, piece = (int)blockIdx.x % kTailParts;
   if (b >= plan.tail_tiles) return;
   int tp, tq;
-  tile_coords(plan.full + b, plan.tiles, (int)(a.Hp / kTile), (int)(a.vs / kTile), 8, tp, tq);
+  tile_coords(plan.full + b, plan.tiles, (int)(a.Hp / kTile), (int)(a.vs / kTile), 8, 8, tp, tq);
   const DwTileGeom<WVH> g(a, tp, tq);
   const float coef = final_factor_of(a);
   const float* part = a.dw_part + (int64_t)b * plan.nseg * kTile * kTile;

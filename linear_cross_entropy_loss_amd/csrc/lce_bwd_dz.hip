@@ -207,7 +207,7 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> stru
   }
   LCE_DEV int num_tiles() const { return tiles_p * tiles_q; }
   LCE_DEV void coords(int tile, int& tp, int& tq) const {
-    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, tp, tq);
+    tile_coords(tile, num_tiles(), tiles_p, tiles_q, 8, a.live, tp, tq);
     tp += tp0;
   }
   LCE_DEV void origins(int tile, const void*& p, const void*& q) const {

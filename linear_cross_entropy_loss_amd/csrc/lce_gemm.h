@@ -96,10 +96,28 @@ LCE_DEV int opaque_tid() {
 // each with its own L2, so consecutive ids are first regrouped per XCD and
 // then walked in bands of `band` P-tiles with Q fastest: the 32 workgroups an
 // XCD runs at a time then cover a compact (band x 32/band) patch of tiles.
+//
+// `live`: how many bands the 8 XCDs work on at the same time.  8 (the plain regrouping: every XCD walks its
+// own eighth of the ids, so each is in a band of its own) keeps 8 P bands in flight; each is re-read once
+// per round from the 256 MB Infinity Cache, and with a long K they no longer fit there together (a band of
+// 8 P-tiles is 32 MiB at K = 8192: the forward ran 7 % slower on 128 vocabulary tiles than on 32).  With
+// live = 4, 2 or 1 the bands are taken `live` at a time and 8 / live XCDs share a band, each walking its own
+// part of the band's Q range.  Needs tiles_p to be a multiple of band * live (else the plain regrouping).
 // ---------------------------------------------------------------------------
-LCE_DEV void tile_coords(int bid, int nblocks, int tiles_p, int tiles_q, int band, int& tp, int& tq) {
+LCE_DEV void tile_coords(int bid, int nblocks, int tiles_p, int tiles_q, int band, int live, int& tp, int& tq) {
   int id = bid;
-  if ((nblocks & 7) == 0) id = (bid & 7) * (nblocks >> 3) + (bid >> 3);
+  if ((nblocks & 7) == 0) {
+    const int xcd = bid & 7, seq = bid >> 3;
+    if (live >= 8 || tiles_p % (band * live) != 0) {
+      id = xcd * (nblocks >> 3) + seq;
+    } else {
+      const int per = 8 / live;                      // XCDs per band
+      const int band_ids = band * tiles_q;
+      const int share = band_ids / per;              // ids of a band that one XCD walks (band * tiles_q * live / 8)
+      const int step = seq / share, r = seq - step * share;
+      id = (step * live + xcd / per) * band_ids + (xcd % per) * share + r;
+    }
+  }
   const int per_band = band * tiles_q;
   const int b = id / per_band;
   const int within = id - b * per_band;

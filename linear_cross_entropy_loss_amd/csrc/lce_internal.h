@@ -54,6 +54,7 @@ struct FwdArgs {
   const int* perm;
   const int64_t* y0;
   int num_cus;  // compute units of the device: grid size of the persistent kernels
+  int live;     // bands of W that the XCDs keep in flight together (lce_gemm.h, tile_coords)
   // outputs / scratch
   float* lse;        // [N]
   float* out5;       // [5]
@@ -106,6 +107,7 @@ struct BwdArgs {
   int dz_shift;
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
+  int live;         // bwd_dz: bands of W that the XCDs keep in flight together (lce_gemm.h, tile_coords)
   // fp32 tensors carried as bf16 pairs (lce_gemm.h): dz is staged as three blocks of Np rows,
   // [hi ; lo ; hi], `dz` pointing at the first; only bwd_dz looks at this flag (the dx and dW launches get
   // plain 16-bit problems over these blocks).
@@ -184,6 +186,16 @@ hipError_t launch_gather_rows_split(const float* x, int64_t ldx, int64_t H, cons
 hipError_t launch_scatter_rows(const void* dxc, int64_t lddxc_bytes, const int* perm, const int64_t* n_rows,
                                int64_t N, const int64_t* y, int64_t ignore_index, void* dx, int64_t lddx_bytes,
                                int64_t row_bytes, int num_cus, hipStream_t s);
+
+// Bands to keep in flight (tile_coords in lce_gemm.h) for P bands of 8 tiles of 256 rows and `k_bytes` bytes per row:
+// as many of 8, 4, 2, 1 as stay within a quarter of the Infinity Cache together (measured at H = 8192, where a band is
+// 32 MiB: bwd_dz 27.5 / 26.4 / 25.0 / 25.2 ms with 8 / 4 / 2 / 1 bands in flight; no difference at H = 4096; 8 best at H = 2048).
+inline int live_bands(int64_t k_bytes) {
+  const int64_t band_bytes = 8 * 256 * k_bytes;
+  int live = 8;
+  while (live > 1 && live * band_bytes > ((int64_t)64 << 20)) live /= 2;
+  return live;
+}
 
 // dx of one slab: at most (Np/256) x (Hp/256) tiles, K = vs columns.  Upper bound on the 256 x 256 fp32
 // blocks of partial sums that the device-side plan of the dx kernel can ask for (0: it never splits).
