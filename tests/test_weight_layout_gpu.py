@@ -79,6 +79,26 @@ def test_vocabulary_major_weight_matches_oracle_and_the_row_major_call(N, H, V, 
     assert emax <= 1e-6 and el2 <= 1e-6, (emax, el2)
 
 
+def test_weights_the_kernels_cannot_read_in_place_are_copied():
+    """fp32 tensors (computed as bf16 pairs, which have no (V, H) form) and a hidden size that is not a multiple
+    of 8: the transposed view is copied into a row-major (H, V) matrix and everything else stays the same."""
+    from oracle import lce_forward_backward_fp64
+
+    for dtype, H, loss_tol, grad_tol in ((torch.float32, 256, 1e-5, 1e-3), (torch.bfloat16, 100, LOSS_RTOL, GRAD_TOL)):
+        print(f"(V, H) weight, copied: {dtype} H={H}", flush=True)
+        N, V = 300, 1000
+        x, y, w = make_inputs(N, H, V, dtype, seed=17, ignore_frac=0.1, device="cuda")
+        wt = w.t().contiguous().requires_grad_(True)
+        xd = x.clone().requires_grad_(True)
+        out = _run(xd, y, wt.t(), 1e-4, 1.0, 512, False, g=1.0)
+        ref = lce_forward_backward_fp64(x, y, w, -1, 1e-4, 1.0, chunk=512)
+        assert abs(out[0].item() - ref.loss.item()) <= loss_tol * abs(ref.loss.item())
+        assert wt.grad.shape == (V, H)
+        for got, want in ((xd.grad, ref.dx), (wt.grad.t(), ref.dw)):
+            emax, el2 = rel_errors(got, want)
+            assert emax <= grad_tol and el2 <= grad_tol, (emax, el2)
+
+
 def test_strided_vocabulary_major_weight_with_garbage_in_the_padding():
     """(V, H) rows with a stride longer than H whose padding holds large finite garbage: same bits as dense."""
     print("(V, H) weight, padded rows", flush=True)
