@@ -79,6 +79,40 @@ def test_vocabulary_major_weight_matches_oracle_and_the_row_major_call(N, H, V, 
     assert emax <= 1e-6 and el2 <= 1e-6, (emax, el2)
 
 
+def test_randomized_shapes_with_a_vocabulary_major_weight():
+    """Twenty seeded draws over token counts, hidden sizes (multiples of 8), vocabularies, dtypes, fp32 master
+    weight, ignore fraction, z-regularisation, scale, N_chunk_size and monitoring, each against the fp64 oracle."""
+    import random
+
+    from linear_cross_entropy_loss_amd import _lib, ops
+    from oracle import lce_forward_backward_fp64
+
+    rng = random.Random(4321)
+    for it in range(20):
+        N = rng.choice([1, 7, 100, 255, 256, 257, 600, 1024, 1500, 3000])
+        H = rng.choice([8, 24, 104, 128, 136, 256, 264, 520, 776, 1024])
+        V = rng.choice([8, 9, 255, 256, 263, 1000, 1001, 4096, 5000, 10008, 12000])
+        dt = rng.choice([torch.bfloat16, torch.float16])
+        wdt = rng.choice([None, torch.float32])
+        ign, zreg, scale = rng.choice([0.0, 0.1, 0.5]), rng.choice([0.0, 1e-4, 1e-2]), rng.choice([1.0, 0.5, 2.0])
+        n_chunk, mon = rng.choice([16, 64, 512, 4096]), rng.choice([False, True])
+        print(f"draw {it}: N={N} H={H} V={V} {dt} w={wdt} ign={ign} zreg={zreg} scale={scale} chunk={n_chunk} mon={mon}",
+              flush=True)
+        x, y, w = make_inputs(N, H, V, dt, seed=1000 + it, ignore_frac=ign, w_dtype=wdt, device="cuda")
+        if (y != -1).sum() == 0:
+            y[0] = 0
+        wt = w.t().contiguous().requires_grad_(True)
+        assert ops._weight_layout(wt.t(), dt) == _lib.W_VH
+        xd = x.clone().requires_grad_(True)
+        out = _run(xd, y, wt.t(), zreg, scale, n_chunk, mon, g=0.7)
+        ref = lce_forward_backward_fp64(x, y, w, -1, zreg, scale, grad_output=0.7, chunk=512)
+        assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item()), (it, out[0].item(), ref.loss.item())
+        for name, got, want in (("dx", xd.grad, ref.dx), ("dw", wt.grad.t(), ref.dw)):
+            emax, el2 = rel_errors(got, want)
+            assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (it, name, emax, el2)
+        assert (xd.grad[y == -1] == 0).all()
+
+
 def test_weights_the_kernels_cannot_read_in_place_are_copied():
     """fp32 tensors (computed as bf16 pairs, which have no (V, H) form) and a hidden size that is not a multiple
     of 8: the transposed view is copied into a row-major (H, V) matrix and everything else stays the same."""
