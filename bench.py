@@ -29,6 +29,9 @@ REFERENCE_PUBLISHED_TFLOPS_8NHV = 115.6
 WORKLOADS = {
     "c2_bf16_N16384_H2048_V131072": dict(N=16384, H=2048, V=131072, dtype="bf16", ignore=0.05, n_chunk=4096,
                                           z_reg=0.0, scale=1.0, monitoring=False, seed=2),
+    # the headline shape with the weight stored (V, H) -- a tied embedding handed over as weight.T, read in place
+    "c2_bf16_N16384_H2048_V131072_weight_VH": dict(N=16384, H=2048, V=131072, dtype="bf16", ignore=0.05, n_chunk=4096,
+                                                    z_reg=0.0, scale=1.0, monitoring=False, seed=2, w_vh=True),
     # the small fp32 case (fp32 tensors, computed as bf16 pairs)
     "c1_f32_N2048_H2048_V16384": dict(N=2048, H=2048, V=16384, dtype="f32", ignore=0.0, n_chunk=4096,
                                        z_reg=0.0, scale=1.0, monitoring=False, seed=1),
@@ -60,6 +63,8 @@ def make_gpu_inputs(cfg, torch):
         y = torch.randint(0, V, (N,), device="cuda", generator=g)
     if cfg["ignore"] > 0:
         y[torch.rand(N, device="cuda", generator=g) < cfg["ignore"]] = -1
+    if cfg.get("w_vh"):
+        w = w.t().contiguous().t()  # shape (H, V), stored (V, H) row-major
     return x, y, w
 
 
@@ -71,9 +76,14 @@ def time_phases(cfg, x, y, w, torch, reps=5):
     N, H, V = cfg["N"], cfg["H"], cfg["V"]
     dev = x.device
 
+    vh = bool(cfg.get("w_vh"))
+    w = w.t() if vh else w  # the rows the kernels read
+    ldw = w.stride(0)
+
     def prob(phases):
-        return _lib.make_problem(N, H, V, x.stride(0), w.stride(0), H, V, x.dtype, w.dtype, x.dtype, w.dtype,
-                                 -1, cfg["scale"], cfg["z_reg"], cfg["n_chunk"], cfg["monitoring"], phases)
+        return _lib.make_problem(N, H, V, x.stride(0), ldw, H, ldw, x.dtype, w.dtype, x.dtype, w.dtype,
+                                 -1, cfg["scale"], cfg["z_reg"], cfg["n_chunk"], cfg["monitoring"], phases, 0, 0,
+                                 _lib.W_VH if vh else _lib.W_HV)
 
     fwd_b, bwd_b = _lib.workspace_bytes(prob(0))
     # one workspace per call: a call restricted to one kernel relies on what the full call left in it
