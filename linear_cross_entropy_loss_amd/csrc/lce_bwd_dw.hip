@@ -279,6 +279,7 @@ template <class T, bool WVH, int MODE> struct DwProblem {
     return reinterpret_cast<const E*>(a.dz) + (rows + kTile - 1) / kTile * kTile * a.vs;
   }
   LCE_DEV int k_valid(int) const { return (int)a.Np; }
+  LCE_DEV void prefetch(int) {}
   LCE_DEV void epilogue(int local, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int item, tp, tq, seg;
     decode(local, item, tp, tq, seg);

@@ -185,6 +185,7 @@ template <class T, bool KMASK, bool WVH, int MODE> struct DxProblem {
     tile_coords(tile, plan.tiles, tiles_p, tiles_q, 8, 8, tp, tq);
   }
   LCE_DEV int item_ktiles(int) const { return plan.kseg; }
+  LCE_DEV void prefetch(int) {}
   LCE_DEV int64_t k0_of(int seg) const { return seg < 0 ? 0 : (int64_t)seg * plan.kseg * kBK; }
   LCE_DEV void origins(int local, const void*& p, const void*& q) const {
     int item, tp, tq, seg;

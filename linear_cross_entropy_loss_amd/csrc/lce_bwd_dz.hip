@@ -49,8 +49,10 @@ static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must
 // SPLIT (fp32 tensors carried as bf16 pairs, lce_gemm.h): dz is staged as hi = bf16(dz) and lo = bf16(dz - hi)
 // in three blocks of Np rows, [hi ; lo ; hi].  The staging sequence simply runs twice, once per part (this
 // path serves accuracy, not speed).
+// `pf_y`, `pf_lse`: label and lse of this lane's four tokens (DzProblem::prefetch), ignore_index / 0 for rows that do not exist.
 template <class T, bool ZREG, bool VTAIL, bool SPLIT>
-LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
+LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], const float (&pf_lse)[kNB],
+                              f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
   typedef typename elem_of<T>::type E;
   const int64_t v0 = a.v0 + (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
   const int tid = opaque_tid();
@@ -72,12 +74,10 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, int64_t rows, f32x16_t (&acc)[kN
   int ykey[kNB];
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t tok = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
-    const bool exists = tok < rows;  // rows past the last one are staged as zeros, like ignored tokens
-    const int64_t yy = exists ? a.y[tok] : a.ignore_index;
+    const int64_t yy = pf_y[qb];  // (rows past the last one are staged as zeros, like ignored tokens)
     const int64_t rel = yy - slice_v0;
     const bool valid = yy != a.ignore_index;
-    const float l = exists ? a.lse[tok] : 0.f;
+    const float l = pf_lse[qb];
     // (the power-of-two factor of the staged dz rides along in the exponent)
     nlse[qb] = valid ? fmaf(-l, kLog2e, (float)a.dz_shift) : -INFINITY;
     gain[qb] = 1.f + 2.f * a.z_reg * l;
@@ -222,10 +222,26 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> stru
   }
   LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
+  // The epilogue starts with the label and lse of each of this lane's four tokens: fetched while the last K tiles
+  // of the tile are still being multiplied, instead of one exposed round trip to memory per tile.
+  int64_t pf_y[kNB];
+  float pf_lse[kNB];
+  LCE_DEV void prefetch(int tile) {
+    int tp, tq;
+    coords(tile, tp, tq);
+    const int lane = threadIdx.x & 63, wq = threadIdx.x >> 7;
+#pragma unroll
+    for (int qb = 0; qb < kNB; ++qb) {
+      const int64_t tok = (int64_t)tq * kTile + wq * kWaveTile + qb * kBlk + (lane & 31);
+      const bool exists = tok < rows;
+      pf_y[qb] = exists ? a.y[tok] : a.ignore_index;
+      pf_lse[qb] = exists ? a.lse[tok] : 0.f;
+    }
+  }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
     coords(tile, tp, tq);
-    dz_epilogue_impl<T, ZREG, VTAIL, SPLIT>(a, rows, acc, tp, tq, scratch);
+    dz_epilogue_impl<T, ZREG, VTAIL, SPLIT>(a, pf_y, pf_lse, acc, tp, tq, scratch);
   }
 };
 

@@ -194,6 +194,7 @@ template <class T, bool VTAIL, bool KMASK, bool WVH> struct FwdProblem {
   }
   LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
+  LCE_DEV void prefetch(int) {}
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     coords(tile, tp, tq);

@@ -138,6 +138,8 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //   static constexpr bool kSwapAB                 false: P fragments feed the A side of the matrix instruction (the P index
 //        runs along accumulator registers, Q along lanes); true: the Q fragments do (acc[i][j] is still the block
 //        of P block i and Q block j, with Q along its registers and P along its lanes)
+//   void prefetch(int tile)                       called three K tiles before the tile's epilogue: the place to issue loads
+//        of per-row data the epilogue starts with (kept in members), so that their latency is not exposed there
 //   static constexpr bool kKMask                  false if `ktiles * 64 == k_valid` for every tile of the launch
 //   int  k_valid(int tile)                        K extent of that tile's contraction; the K tiles of the
 //        loop may run past it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
@@ -355,6 +357,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
         }
         step<0, false, false, false>(acc, sp, sq);
       }
+      prob.prefetch(tile);  // three K tiles ahead of the epilogue
       step<1, false, true, false>(acc, sp, sq);
       step<0, false, false, false>(acc, sp, sq);
       step<1, false, false, true>(acc, sp, sq);
