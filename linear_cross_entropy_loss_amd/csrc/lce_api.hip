@@ -216,6 +216,9 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   // memory bandwidth; 5 when it is written once) and 5 (dW) units; a launch about 10.  The model ranks the slab
   // widths measured at N = 16384, H = 2048, V = 32768 and 65536 (2 ... 18 slabs) in their measured order.
   constexpr double kPlanCUs = 256.0;
+  // bands of W tiles that bwd_dz keeps in flight (tile_coords in lce_gemm.h), and the slab width that is a whole group of them
+  const int live = lce::live_bands(lce::padded_k(split ? 3 * p->H : p->H) * 2);
+  const int64_t gran = live < 8 ? (int64_t)256 * 8 * live : 256;
   auto kernel_cost = [&](double T, double L, double e, bool parts) -> double {
     const double full = (double)(int64_t)(T / kPlanCUs), r = T - full * kPlanCUs;
     double cost = full * (L + e) + 10.0;
@@ -229,14 +232,16 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   };
   auto slab_cost = [&](int64_t w, bool parts, bool sums) -> double {
     const double tq = (double)(Np / 256), th = (double)(Hp / 256), tv = (double)(w / 256), k3 = split ? 3.0 : 1.0;
-    return kernel_cost(tq * tv, k3 * (double)((p->H + 63) / 64), 6.0, false) +
+    // (bwd_dz runs about 4 % slower on a slab that is not whole groups of the bands it keeps in flight when K is long)
+    const double dz_order = live < 8 && (w / 256) % (8 * live) != 0 ? 1.04 : 1.0;
+    return dz_order * kernel_cost(tq * tv, k3 * (double)((p->H + 63) / 64), 6.0, false) +
            k3 * kernel_cost(tq * th, (double)(w / 64), sums ? 21.0 : 5.0, parts) +
            kernel_cost(tv * th, k3 * (double)(Np / 64), 5.0, parts);
   };
 
   // mode 0: everything; mode 1: lean (at the strict bound only); mode 2: everything, widened bound.
   // Tries a split into `s` slabs of equal width (the last one may be narrower); cost: its modelled time.
-  auto fits = [&](int mode, int64_t s, BwdPlan* out, double* cost) -> bool {
+  auto fits = [&](int mode, int64_t s, bool whole_groups, BwdPlan* out, double* cost) -> bool {
     const bool lean = mode == 1;
     const bool pack = packs_rows(p) && !(lean && p->pack_rows == LCE_PACK_AUTO);
     // The dx kernels store packed rows straight to their tokens' places through 32-bit offsets into dx; a dx
@@ -246,7 +251,8 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
     if (pack) fixed = b->dxc + (stage_dx ? align_up((size_t)p->N * (size_t)b->lddxc * dxes) : 0);
     else if (split) fixed = b->pack.end;
     const size_t budget = strict + (mode == 2 ? (size_t)p->N * (size_t)p->H * 4 : 0);
-    const int64_t vs = (cols + s - 1) / s * 256;
+    int64_t vs = (cols + s - 1) / s * 256;
+    if (whole_groups) vs = (vs + gran - 1) / gran * gran;  // the next width that is whole groups of bands
     const int64_t slabs = (Vp + vs - 1) / vs;
     // (bf16 pairs: three blocks of dz, and dx is summed over three passes per slab, so it always needs the running sum)
     const size_t dz = align_up(Np * (size_t)vs * 2 * (split ? 3 : 1));
@@ -287,9 +293,11 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
     for (int64_t s = 1; s <= cols; ++s) {
       if (s > 1 && (cols + s - 2) / (s - 1) == (cols + s - 1) / s) continue;  // same width as with one slab fewer
       if (first != 0 && (mode == 2 || s > 4 * first + 8)) break;
-      if (!fits(mode, s, &cand, &c)) continue;
-      if (first == 0 || c < *cost) { *out = cand; *cost = c; }
-      if (first == 0) first = s;
+      for (int whole = 0; whole < (gran > 256 ? 2 : 1); ++whole) {
+        if (!fits(mode, s, whole != 0, &cand, &c)) continue;
+        if (first == 0 || c < *cost) { *out = cand; *cost = c; }
+        if (first == 0) first = s;
+      }
     }
     return first != 0;
   };

@@ -132,6 +132,23 @@ def test_config5_long_sequence_fp32_master_weight_full_size():
     torch.cuda.empty_cache()
 
 
+def test_long_hidden_size_with_activations_beyond_the_infinity_cache():
+    """N=16384, H=8192, V=65536, bf16: a chunk of x is 256 MiB, so the forward runs as two launches of 32768
+    columns, and a band of W tiles is 32 MiB, so forward and dz keep two bands in flight instead of eight (the
+    tile order of lce_gemm.h) -- paths no benchmark configuration with a 16-bit weight takes."""
+    from oracle import lce_forward_backward_fp64
+
+    print("N=16384 H=8192 V=65536 bf16, 5 % ignored", flush=True)
+    N, H, V = 16384, 8192, 65536
+    x, y, w = _inputs(N, H, V, torch.bfloat16, seed=8, ignore=0.05)
+    out, dx, dw, extra = _step(x, y, w, 1e-4, 1.0, 4096, True)
+    assert extra <= 4096 * V * 4 + N * H * 4, extra  # (the bound is widened by the fp32 running dx when it cannot be met)
+    ref = lce_forward_backward_fp64(x, y, w, -1, 1e-4, 1.0, chunk=1024)
+    _check_against_oracle(out, dx, dw, ref, y, True)
+    del ref, dx, dw, x, w
+    torch.cuda.empty_cache()
+
+
 # config 4: inputs of one vocabulary size at a time, and what the N_chunk_size = 4096 point of that size gave
 _c4 = {}
 
