@@ -87,7 +87,11 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
 
   const int64_t blk = a.Np * a.vs;  // SPLIT: elements between the three blocks of the stage
 #pragma unroll
-  for (int part = 0; part < (SPLIT ? 2 : 1); ++part)
+  for (int part = 0; part < (SPLIT ? 2 : 1); ++part) {
+  // (SPLIT: an opaque copy of the scale per part, so that the compiler recomputes the exponentials of part 1 instead of
+  // keeping all 256 of part 0 alive across the staging of that part, which spilled 2 KiB per lane)
+  float c1p = c1;
+  if (SPLIT) asm volatile("" : "+v"(c1p));
 #pragma unroll
   for (int ph = 0; ph < 2; ++ph) {
 #pragma unroll
@@ -106,13 +110,13 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
             if (!VTAIL || pb * 4 + g + h2 < nq) {
 #pragma unroll
               for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
-                d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
+                d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1p, nlse[qb]));
                 if (ZREG) d[i] *= gain[qb];
               }
             } else if (pb * 4 + g + h2 == nq && cut != 0) {
 #pragma unroll
               for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
-                d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
+                d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1p, nlse[qb]));
                 if (ZREG) d[i] *= gain[qb];
                 d[i] = (i - 4 * h2) < cut_mine ? d[i] : 0.f;
               }
@@ -151,7 +155,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
 #pragma unroll
           for (int r = 0; r < 16; ++r)
             if (want == pp * 16 + r) zt = acc[2 * ph + pp][qb][r];
-        float p = __builtin_amdgcn_exp2f(fmaf(zt, c1, nlse[qb]));
+        float p = __builtin_amdgcn_exp2f(fmaf(zt, c1p, nlse[qb]));
         if (ZREG) p *= gain[qb];
         float tv = p - __builtin_bit_cast(float, (127 + a.dz_shift) << 23);  // the one, times 2^dz_shift
         if (SPLIT && part == 1) tv = bf16_lo(tv);
@@ -174,6 +178,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
       if (SPLIT && part == 0) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(dst + 2 * blk));
       if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most 4 rows in registers at a time
     }
+  }
   }
   __syncthreads();  // scratch is handed back to the main loop
 }
