@@ -349,11 +349,16 @@ template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipS
   // extent is long enough to split is decided on the device, and a launch without items returns at once)
   const bool tails = a.dw_part != nullptr && dw_tail_blocks(a.Np, a.Hp, a.vs) != 0 &&
                      has_split_tail((a.vs / kTile) * (a.Hp / kTile), a.dw_grid);
-  hipError_t e;
+  hipError_t e = hipSuccess;
   if constexpr (WVH) {
     e = launch_tiles<T, true, kDwAll>(a, s);
   } else {
-    e = a.dw_dtype == DT_F32 ? launch_tiles<T, false, kDwStaged32>(a, s) : launch_tiles<T, false, kDwStaged>(a, s);
+    // (a small problem whose tiles are all split along K has no whole tile to launch; known here when rows are not packed)
+    const int64_t kt2 = (a.N + 2 * kBK - 1) / (2 * kBK) * 2;
+    const bool none_whole = tails && a.n_rows == nullptr &&
+                            all_tiles_are_tails((a.vs / kTile) * (a.Hp / kTile), a.dw_grid, kt2 < 4 ? 4 : kt2);
+    if (!none_whole)
+      e = a.dw_dtype == DT_F32 ? launch_tiles<T, false, kDwStaged32>(a, s) : launch_tiles<T, false, kDwStaged>(a, s);
     if (e == hipSuccess && tails) e = launch_tiles<T, false, kDwTails>(a, s);
   }
   if (e != hipSuccess || !tails) return e;

@@ -283,7 +283,11 @@ template <class T, bool KMASK, bool WVH, int MODE> hipError_t launch_tiles(const
 }
 
 template <class T, bool KMASK, bool WVH> hipError_t launch_layout(const BwdArgs& a, bool tails, hipStream_t s) {
-  hipError_t e = a.first ? (a.last ? launch_tiles<T, KMASK, WVH, kDxOnly>(a, s) : launch_tiles<T, KMASK, WVH, kDxFirst>(a, s))
+  // (a small problem whose tiles are all split along K has no whole tile to launch; known here when rows are not packed)
+  const bool none_whole = tails && a.n_rows == nullptr &&
+                          all_tiles_are_tails((a.Np / kTile) * (a.Hp / kTile), a.dx_grid, a.vs / kBK);
+  hipError_t e = none_whole ? hipSuccess
+               : a.first ? (a.last ? launch_tiles<T, KMASK, WVH, kDxOnly>(a, s) : launch_tiles<T, KMASK, WVH, kDxFirst>(a, s))
                          : (a.last ? launch_tiles<T, KMASK, WVH, kDxLast>(a, s) : launch_tiles<T, KMASK, WVH, kDxMiddle>(a, s));
   if (e == hipSuccess && tails) e = launch_tiles<T, KMASK, WVH, kDxTails>(a, s);
   return e;

@@ -217,6 +217,11 @@ inline bool has_split_tail(int64_t T, int64_t G) {
   const int64_t r = T % G, cap = G < kTailBlocks ? G : kTailBlocks;
   return r > 0 && r * 2 <= cap;
 }
+// Whether every one of T output tiles with `kt` K tiles each is a tail tile of the device-side plans (dx_plan,
+// dw_plan): fewer tiles than workgroups, few enough to split, and a K extent long enough for two segments.
+inline bool all_tiles_are_tails(int64_t T, int64_t G, int64_t kt) {
+  return T < G && has_split_tail(T, G) && kt / 2 >= 16;
+}
 // true if every split the dx kernel may choose cuts the K tiles of a slab into equal, even segments
 inline bool dx_segments_exact(int64_t vs) { return (vs / 64) % (2 * max_k_segments(vs / 64)) == 0; }
 // dW of one slab: (vs/256) x (Hp/256) tiles, K = at most Np tokens.  The same bound for the dW kernel, whose
