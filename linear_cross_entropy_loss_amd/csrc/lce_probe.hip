@@ -7,6 +7,10 @@
 //                     Two further patterns add the LDS traffic of the tile kernels and nothing else (no global
 //                     loads, no barriers, no epilogue): every k step's 8 fragments are re-read from LDS, and
 //                     4 x 16 bytes per lane are written to it.
+//   lce_probe_mfma_loads  the same loop with the tile kernels' operand fetch added as well: 4 x 16 bytes per lane
+//                     and k step are fetched with buffer loads (64 KiB per workgroup and 64-deep K tile, the window
+//                     shared by all workgroups so that it is served by the L2s) and are what the LDS writes store;
+//                     optionally with the one workgroup barrier per K tile that the tile kernels need.
 //   lce_probe_flush   what adding 256 x 256 fp32 blocks of partial sums into a matrix in memory costs, with
 //                     atomics or as plain read-modify-write: the traffic a backward that fed dz straight into
 //                     the dx and dW contractions would generate once per dz tile (its H-wide accumulators do
@@ -20,6 +24,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) short s16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
 
 __device__ __forceinline__ unsigned hash32(unsigned x) {
   x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
@@ -75,8 +80,12 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int pattern, int iters, 
 // pattern 2: random operands, the 4 + 4 fragments of every k step read from LDS (8 ds_read_b128 per 16 MFMAs, the
 // rate of the operator's tile kernels), one k step ahead; pattern 3: additionally 4 ds_write_b128 per 16 MFMAs (the
 // rate at which those kernels refill their LDS stages).  Reads and writes are interleaved with the MFMAs one by one.
-template <bool WRITES>
-__global__ __launch_bounds__(256) void mfma_lds_loop_kernel(int iters, float* out) {
+// LOADS (lce_probe_mfma_loads): the 4 pieces written per k step come from memory, loaded three k steps earlier
+// (the tile kernels give a load one K tile = four k steps) with buffer loads, one after every fourth MFMA: `src`
+// holds `src_bytes` (a power of two) bytes, and all workgroups walk the same window of it, 16 KiB per k step.
+// BARRIER: a workgroup barrier after every fourth k step (one per 64-deep K tile).
+template <bool WRITES, bool LOADS, bool BARRIER>
+__global__ __launch_bounds__(256) void mfma_lds_loop_kernel(int iters, float* out, const char* src, unsigned src_bytes) {
   __shared__ __attribute__((aligned(16))) short lds[65536];  // 128 KiB, the two stages of a tile kernel
   const unsigned tid = blockIdx.x * 256u + threadIdx.x;
   for (int i = threadIdx.x; i < 65536; i += 256) lds[i] = random_bf16(blockIdx.x * 65536u + i);
@@ -94,13 +103,33 @@ __global__ __launch_bounds__(256) void mfma_lds_loop_kernel(int iters, float* ou
   s16x8_t* wr = reinterpret_cast<s16x8_t*>(lds);
 #pragma unroll
   for (int f = 0; f < 8; ++f) fa[f] = rd[(wave * 2048 + f * 64 + lane) & 8191];
-  auto step = [&](s16x8_t (&cur)[8], s16x8_t (&nxt)[8], int it) {
+  u32x4_t g[4][4];  // LOADS: four sets of pieces in flight
+  // (raw 32-bit data format, as in the tile kernels; the scalar offset selects the piece, the vector offset the lane)
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(src), 0, LOADS ? (int)src_bytes : 0, 0x00020000);
+  const unsigned voff = threadIdx.x * 16u;
+  auto load = [&](int it, int f) -> u32x4_t {
+    const unsigned o = ((unsigned)(it * 16384 + f * 4096)) & (src_bytes - 1);
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, (int)o, 0);
+  };
+  if (LOADS) {
+#pragma unroll
+    for (int u = 1; u < 4; ++u)
+#pragma unroll
+      for (int f = 0; f < 4; ++f) g[u][f] = load(u, f);
+  }
+  auto step = [&](s16x8_t (&cur)[8], s16x8_t (&nxt)[8], u32x4_t (&fill)[4], u32x4_t (&drain)[4], int it) {
     const int o = (it + 1) * 512 + wave * 2048;
 #pragma unroll
     for (int f = 0; f < 8; ++f) nxt[f] = rd[(o + f * 64 + lane) & 8191];
     if (WRITES) {
 #pragma unroll
-      for (int f = 0; f < 4; ++f) wr[(o + 4096 + f * 64 + lane) & 8191] = cur[f];
+      for (int f = 0; f < 4; ++f)
+        wr[(o + 4096 + f * 64 + lane) & 8191] = LOADS ? __builtin_bit_cast(s16x8_t, drain[f]) : cur[f];
+    }
+    if (LOADS) {
+#pragma unroll
+      for (int f = 0; f < 4; ++f) fill[f] = load(it + 4, f);
     }
 #pragma unroll
     for (int s = 0; s < 16; ++s) {
@@ -113,11 +142,18 @@ __global__ __launch_bounds__(256) void mfma_lds_loop_kernel(int iters, float* ou
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                       // one MFMA
       if (s < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                            // one LDS read
       if (WRITES && s >= 8 && (s & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
+      if (LOADS && (s & 3) == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);            // one buffer load
     }
+    __builtin_amdgcn_sched_barrier(0);
   };
-  for (int it = 0; it < iters; it += 2) {  // (the two fragment sets change roles: no register moves)
-    step(fa, fb, it);
-    step(fb, fa, it + 1);
+  // (the fragment sets and the sets of loaded pieces change roles: no register moves; a set written to LDS in one k
+  // step is refilled in the same step, after the writes)
+  for (int it = 0; it < iters; it += 4) {
+    step(fa, fb, g[0], g[1], it);
+    step(fb, fa, g[1], g[2], it + 1);
+    step(fa, fb, g[2], g[3], it + 2);
+    step(fb, fa, g[3], g[0], it + 3);
+    if (BARRIER) __syncthreads();
   }
   float s = 0.f;
 #pragma unroll
@@ -158,16 +194,30 @@ __global__ __launch_bounds__(256) void flush_kernel(float* dst, int64_t rows, in
 
 extern "C" {
 
-// Launches `wgs` workgroups of 4 waves, each wave issuing iters * 16 MFMAs (32 x 32 x 16, bf16); iters even.
+// Launches `wgs` workgroups of 4 waves, each wave issuing iters * 16 MFMAs (32 x 32 x 16, bf16); iters a multiple of 4.
 // pattern 0 constant / 1 random operands in registers; 2 random operands re-read from LDS; 3 plus LDS writes.
 // out: wgs * 256 floats.  FLOPs = wgs * 4 * iters * 16 * 32768.
 int lce_probe_mfma(int pattern, int wgs, int iters, float* out, void* stream) {
-  if (pattern < 0 || pattern > 3 || wgs <= 0 || iters <= 0 || (iters & 1) || !out) return -3;
+  if (pattern < 0 || pattern > 3 || wgs <= 0 || iters <= 0 || (iters & 3) || !out) return -3;
   const dim3 grid((unsigned)wgs), block(256);
   hipStream_t s = (hipStream_t)stream;
-  if (pattern == 2) hipLaunchKernelGGL(mfma_lds_loop_kernel<false>, grid, block, 0, s, iters, out);
-  else if (pattern == 3) hipLaunchKernelGGL(mfma_lds_loop_kernel<true>, grid, block, 0, s, iters, out);
+  if (pattern == 2) hipLaunchKernelGGL((mfma_lds_loop_kernel<false, false, false>), grid, block, 0, s, iters, out, nullptr, 1u);
+  else if (pattern == 3) hipLaunchKernelGGL((mfma_lds_loop_kernel<true, false, false>), grid, block, 0, s, iters, out, nullptr, 1u);
   else hipLaunchKernelGGL(mfma_loop_kernel, grid, block, 0, s, pattern, iters, out);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+// Pattern 3 of lce_probe_mfma with the pieces written to LDS loaded from `src` (device memory, `src_bytes` of it: a
+// power of two from 64 KiB to 1 GiB): 16 KiB per workgroup and k step, every workgroup walking the same window.
+// barrier != 0: with a workgroup barrier after every fourth k step.
+int lce_probe_mfma_loads(int wgs, int iters, const void* src, uint64_t src_bytes, int barrier, float* out, void* stream) {
+  if (wgs <= 0 || iters <= 0 || (iters & 3) || !out || !src) return -3;
+  if (src_bytes < 65536 || (src_bytes & (src_bytes - 1)) || src_bytes > (1ull << 30)) return -3;
+  const dim3 grid((unsigned)wgs), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  const char* p = reinterpret_cast<const char*>(src);
+  if (barrier) hipLaunchKernelGGL((mfma_lds_loop_kernel<true, true, true>), grid, block, 0, s, iters, out, p, (unsigned)src_bytes);
+  else hipLaunchKernelGGL((mfma_lds_loop_kernel<true, true, false>), grid, block, 0, s, iters, out, p, (unsigned)src_bytes);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
