@@ -393,3 +393,55 @@ def test_saturated_softmax_with_logits_in_the_hundreds(dtype, w_std, scale):
     for got, want in ((dx, ref.dx), (dw, ref.dw)):
         emax, el2 = rel_errors(got, want)
         assert emax <= grad_tol and el2 <= grad_tol, (emax, el2)
+
+
+@pytest.mark.pack_auto  # (run once: every draw picks its own packing mode)
+def test_two_hundred_draws_over_layouts_packing_and_sizes_around_a_round_of_tiles():
+    """Seeded draws over everything a call can vary at once: both weight layouts, the three packing modes, 16-bit and
+    fp32 tensors, fp32 master weights, ignore fractions up to 95 %, and sizes up to 12000 tokens x 2056 hidden units,
+    where the dx / dW tile counts pass through one round of 256 workgroups (whole tiles only, split tails only, both).
+    Inputs and the fp64 oracle live on the GPU.  A gradient is allowed, on top of its tolerance, what rounding the
+    exact result to the output type costs (the fp16 dx of a mean over 12000 tokens lies in fp16's subnormal range)."""
+    import random
+
+    from linear_cross_entropy_loss_amd import linear_cross_entropy, ops
+    from oracle import lce_forward_backward_fp64
+
+    rng = random.Random(20)
+    for it in range(200):
+        N = rng.choice([1, 7, 100, 255, 256, 257, 600, 1024, 1500, 3000, 4096, 5000, 8192, 8200, 12000])
+        H = rng.choice([8, 24, 104, 128, 136, 256, 264, 520, 776, 1024, 2048, 2056])
+        V = rng.choice([8, 9, 255, 256, 263, 1000, 1001, 2048, 4096, 5000, 8192, 10008, 12000, 16384, 20000, 32768])
+        dt = rng.choice([torch.bfloat16, torch.float16, torch.bfloat16, torch.float16, torch.float32])
+        wdt = None if dt == torch.float32 else rng.choice([None, None, torch.float32])
+        vh = dt != torch.float32 and rng.random() < 0.5
+        ign, zreg, scale = rng.choice([0.0, 0.1, 0.5, 0.95]), rng.choice([0.0, 1e-4, 1e-2]), rng.choice([1.0, 0.5, 2.0])
+        nc, mon, pack = rng.choice([16, 64, 512, 4096, 4096]), rng.choice([False, True]), rng.choice([0, 1, 2])
+        if N * V > 2.2e8:  # keeps the fp64 oracle's N x V matrices below 2 GiB
+            V = max(8, int(2.2e8 // N) // 8 * 8)
+        print(f"draw {it}: N={N} H={H} V={V} {dt} w={wdt} vh={vh} ign={ign} zreg={zreg} scale={scale} chunk={nc} "
+              f"mon={mon} pack={pack}", flush=True)
+        x, y, w = make_inputs(N, H, V, dt, seed=7000 + it, ignore_frac=ign, w_dtype=wdt, device="cuda")
+        if (y != -1).sum() == 0:
+            y[0] = 0
+        wt = (w.t().contiguous() if vh else w.clone()).requires_grad_(True)
+        xd = x.clone().requires_grad_(True)
+        token = ops.pack_rows.set(pack)
+        try:
+            out = linear_cross_entropy(xd, y, wt.t() if vh else wt, -1, zreg, scale, nc, mon)
+            (out[0] * 0.7).backward()
+            torch.cuda.synchronize()
+        finally:
+            ops.pack_rows.reset(token)
+        ref = lce_forward_backward_fp64(x, y, w, -1, zreg, scale, grad_output=0.7, chunk=512)
+        loss_tol, grad_tol = _tols(dt)
+        # (relative to max(loss, 1): with one or a few tokens the loss can be a fraction of the logits it is made of,
+        # which carry the rounding of the 16-bit operands)
+        assert abs(out[0].item() - ref.loss.item()) <= loss_tol * max(abs(ref.loss.item()), 1.0), it
+        for name, got, want in (("dx", xd.grad, ref.dx), ("dw", wt.grad.t() if vh else wt.grad, ref.dw)):
+            assert torch.isfinite(got).all(), (it, name)
+            emax, el2 = rel_errors(got, want)
+            rmax, rl2 = rel_errors(want.to(got.dtype), want)
+            assert emax <= grad_tol + rmax and el2 <= grad_tol + rl2, (it, name, emax, el2)
+        assert (xd.grad[y == -1] == 0).all(), it
+        del x, y, w, wt, xd, out, ref
