@@ -305,7 +305,7 @@ def _load_probe_lib():
     lib.lce_probe_mfma.restype = ctypes.c_int
     lib.lce_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp]
     lib.lce_probe_mfma_loads.restype = ctypes.c_int
-    lib.lce_probe_mfma_loads.argtypes = [ctypes.c_int, ctypes.c_int, vp, ctypes.c_uint64, ctypes.c_int, vp, vp]
+    lib.lce_probe_mfma_loads.argtypes = [ctypes.c_int, ctypes.c_int, vp, ctypes.c_uint64, ctypes.c_int, ctypes.c_int, vp, vp]
     lib.lce_probe_flush.restype = ctypes.c_int
     lib.lce_probe_flush.argtypes = [ctypes.c_int, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, vp]
     return lib
@@ -314,8 +314,8 @@ def _load_probe_lib():
 def probe_ceiling(torch):
     """What bounds the tile kernels on this part: (1) a register-only loop of the same MFMA instruction over
     the same 128 x 128 wave tile, on constant and on random operands, with the tile kernels' LDS reads and
-    writes added, with their operand loads from L2 added as well, and with their one barrier per K tile (still no
-    epilogues), on all and on half of the compute units;
+    writes added, with their operand loads from L2 added as well, with their one barrier per K tile, and with a
+    quarter of the loads missing L2 (still no epilogues), on all and on half of the compute units;
     (2) the vendor GEMM (torch.matmul -> hipBLASLt) on the four contractions of the default workload; (3) the
     operator's forward tile kernel on all and on half of the compute units (a chip-level power limit shows as a
     higher rate per compute unit when fewer of them run)."""
@@ -328,17 +328,21 @@ def probe_ceiling(torch):
            "vendor_gemm": [], "fwd_tiles": []}
     buf = torch.empty(cus * 256 * 4, dtype=torch.float32, device="cuda")
     iters = 200000
-    # operand window of the loads pattern: 2 MiB of random bf16 in [-2, 2) (stays in every L2), walked by all workgroups
-    window = (torch.rand(1 << 20, device="cuda") * 4 - 2).to(torch.bfloat16)
+    # operand windows of the loads patterns: 2 MiB of random bf16 in [-2, 2) each.  One window walked by all workgroups
+    # stays in every L2; with 64 of them (128 MiB: resident in the Infinity Cache, 16 MiB per XCD: not in its L2), one per
+    # four workgroups of an XCD, a quarter of the requests goes over the fabric, as in the tile kernels
+    window = (torch.rand(64 << 20, device="cuda") * 4 - 2).to(torch.bfloat16)
     for wgs in (cus, cus // 2):
         for pattern, name in ((0, "constant operands"), (1, "random bf16 operands"),
                               (2, "random, fragments re-read from LDS"), (3, "random, LDS reads + LDS writes"),
                               (4, "random, LDS traffic + operand loads"),
-                              (5, "random, LDS traffic + loads + barrier")):
+                              (5, "random, LDS traffic + loads + barrier"),
+                              (6, "same, a quarter of the loads over fabric")):
             def run():
                 if pattern >= 4:
-                    rc = probe.lce_probe_mfma_loads(wgs, iters, ctypes.c_void_p(window.data_ptr()), window.numel() * 2,
-                                                    pattern - 4, ctypes.c_void_p(buf.data_ptr()), stream)
+                    rc = probe.lce_probe_mfma_loads(wgs, iters, ctypes.c_void_p(window.data_ptr()), 2 << 20,
+                                                    64 if pattern == 6 else 1, int(pattern >= 5),
+                                                    ctypes.c_void_p(buf.data_ptr()), stream)
                 else:
                     rc = probe.lce_probe_mfma(pattern, wgs, iters, ctypes.c_void_p(buf.data_ptr()), stream)
                 assert rc == 0

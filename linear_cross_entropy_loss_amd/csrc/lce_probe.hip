@@ -84,8 +84,13 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int pattern, int iters, 
 // (the tile kernels give a load one K tile = four k steps) with buffer loads, one after every fourth MFMA: `src`
 // holds `src_bytes` (a power of two) bytes, and all workgroups walk the same window of it, 16 KiB per k step.
 // BARRIER: a workgroup barrier after every fourth k step (one per 64-deep K tile).
+// `grouped`: instead of one window for all, every four workgroups of an XCD (workgroup b runs on XCD b % 8) walk a
+// window of their own, `src_bytes` long, 64 windows in all: three of four requests hit in L2, as for the tile kernels'
+// operand bands, and the rest comes over the fabric.
 template <bool WRITES, bool LOADS, bool BARRIER>
-__global__ __launch_bounds__(256) void mfma_lds_loop_kernel(int iters, float* out, const char* src, unsigned src_bytes) {
+__global__ __launch_bounds__(256) void mfma_lds_loop_kernel(int iters, float* out, const char* src, unsigned src_bytes,
+                                                            int grouped) {
+  if (LOADS && grouped) src += (size_t)((blockIdx.x & 7) * 8 + ((blockIdx.x >> 3) / 4 & 7)) * src_bytes;
   __shared__ __attribute__((aligned(16))) short lds[65536];  // 128 KiB, the two stages of a tile kernel
   const unsigned tid = blockIdx.x * 256u + threadIdx.x;
   for (int i = threadIdx.x; i < 65536; i += 256) lds[i] = random_bf16(blockIdx.x * 65536u + i);
@@ -201,23 +206,27 @@ int lce_probe_mfma(int pattern, int wgs, int iters, float* out, void* stream) {
   if (pattern < 0 || pattern > 3 || wgs <= 0 || iters <= 0 || (iters & 3) || !out) return -3;
   const dim3 grid((unsigned)wgs), block(256);
   hipStream_t s = (hipStream_t)stream;
-  if (pattern == 2) hipLaunchKernelGGL((mfma_lds_loop_kernel<false, false, false>), grid, block, 0, s, iters, out, nullptr, 1u);
-  else if (pattern == 3) hipLaunchKernelGGL((mfma_lds_loop_kernel<true, false, false>), grid, block, 0, s, iters, out, nullptr, 1u);
+  if (pattern == 2) hipLaunchKernelGGL((mfma_lds_loop_kernel<false, false, false>), grid, block, 0, s, iters, out, nullptr, 1u, 0);
+  else if (pattern == 3) hipLaunchKernelGGL((mfma_lds_loop_kernel<true, false, false>), grid, block, 0, s, iters, out, nullptr, 1u, 0);
   else hipLaunchKernelGGL(mfma_loop_kernel, grid, block, 0, s, pattern, iters, out);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
-// Pattern 3 of lce_probe_mfma with the pieces written to LDS loaded from `src` (device memory, `src_bytes` of it: a
-// power of two from 64 KiB to 1 GiB): 16 KiB per workgroup and k step, every workgroup walking the same window.
+// Pattern 3 of lce_probe_mfma with the pieces written to LDS loaded from `src` (device memory): 16 KiB per workgroup
+// and k step out of a window of `window_bytes` (a power of two from 64 KiB to 1 GiB).  windows == 1: every workgroup
+// walks the same window; windows == 64: every four workgroups of an XCD walk their own (src holds 64 * window_bytes).
 // barrier != 0: with a workgroup barrier after every fourth k step.
-int lce_probe_mfma_loads(int wgs, int iters, const void* src, uint64_t src_bytes, int barrier, float* out, void* stream) {
-  if (wgs <= 0 || iters <= 0 || (iters & 3) || !out || !src) return -3;
-  if (src_bytes < 65536 || (src_bytes & (src_bytes - 1)) || src_bytes > (1ull << 30)) return -3;
+int lce_probe_mfma_loads(int wgs, int iters, const void* src, uint64_t window_bytes, int windows, int barrier, float* out,
+                         void* stream) {
+  if (wgs <= 0 || iters <= 0 || (iters & 3) || !out || !src || (windows != 1 && windows != 64)) return -3;
+  if (window_bytes < 65536 || (window_bytes & (window_bytes - 1)) || window_bytes > (1ull << 30)) return -3;
   const dim3 grid((unsigned)wgs), block(256);
   hipStream_t s = (hipStream_t)stream;
   const char* p = reinterpret_cast<const char*>(src);
-  if (barrier) hipLaunchKernelGGL((mfma_lds_loop_kernel<true, true, true>), grid, block, 0, s, iters, out, p, (unsigned)src_bytes);
-  else hipLaunchKernelGGL((mfma_lds_loop_kernel<true, true, false>), grid, block, 0, s, iters, out, p, (unsigned)src_bytes);
+  const unsigned wb = (unsigned)window_bytes;
+  const int grouped = windows == 64;
+  if (barrier) hipLaunchKernelGGL((mfma_lds_loop_kernel<true, true, true>), grid, block, 0, s, iters, out, p, wb, grouped);
+  else hipLaunchKernelGGL((mfma_lds_loop_kernel<true, true, false>), grid, block, 0, s, iters, out, p, wb, grouped);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
