@@ -596,7 +596,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     a.x_dtype = lce::DT_BF16;
   }
   const bool split = splits(p);
-  const int64_t blk_bytes = a.Np * 2;  // times the slab width: one of the three blocks [hi ; lo ; hi] of a split dz
+  a.dz_rows = split ? 3 * a.Np : a.Np;  // rows per column group of the dz stage (BwdArgs::dz)
 
   for (int64_t i = 0; i < b.slabs; ++i) {
     a.v0 = i * b.vs;
@@ -636,9 +636,9 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
       continue;
     }
     // fp32 tensors as bf16 pairs (lce_gemm.h): x = [hi | hi | lo] against W = [hi ; lo ; hi] along a K axis of
-    // 3 H for the logits; dz comes back as three blocks [hi ; lo ; hi] of Np rows.
+    // 3 H for the logits; dz comes back as three blocks [hi ; lo ; hi] of Np rows in every column group.
     char* dz0 = (char*)a.dz;
-    const int64_t blk = blk_bytes * a.vs;
+    const int64_t blk = a.Np * 64 * 2;  // bytes from the first row of a block to that of the next
     if (ph & LCE_PHASE_BWD_DZ) {
       lce::BwdArgs z = a;
       z.H = 3 * p->H;

@@ -193,7 +193,7 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
 // `nseg` segments of `kseg` K tiles (r * nseg <= G, at least 16 K tiles each), whose fp32 sums meet in
 // 256 x 256 blocks of dw_part and are added, in segment order, by dw_tail_kernel.  With few tiles in all
 // (a small vocabulary slab times a small hidden size) every tile is a tail tile.  The K extent comes from
-// the row count on the device, so the plan is made there; a last segment that runs past the rows reads zeros.
+// the row count on the device, so the plan is made there; the segments cover the K tiles exactly.
 struct DwPlan {
   int tiles, full, tail_tiles, nseg, kseg, kt;
 };
@@ -214,10 +214,11 @@ LCE_DEV DwPlan dw_plan(const BwdArgs& a, int64_t rows) {
     p.nseg = 1;
     p.kseg = p.kt;
   } else {
-    const int seg = ((p.kt + s - 1) / s + 1) & ~1;  // even
+    // s segments that cover the K tiles exactly: an even number each, the last one takes what is left over
+    // (fewer than 2 s K tiles more than the others)
     p.tail_tiles = r;
-    p.kseg = seg;
-    p.nseg = (p.kt + seg - 1) / seg;
+    p.kseg = (p.kt / s) & ~1;
+    p.nseg = s;
   }
   return p;
 }
@@ -235,6 +236,7 @@ template <class T, bool WVH, int MODE> struct DwProblem {
   static constexpr bool kSwapAB = !WVH;  // (H, V) output: dz, the Q operand, feeds the A side (v along registers)
   static constexpr bool kVarK = true;    // whole tiles and segment items have different K extents
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
+  static constexpr bool kQGrouped = true;  // dz is staged in groups of 64 columns (BwdArgs::dz)
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows (the K extent): all of x, or the packed rows (see BwdArgs)
@@ -265,18 +267,25 @@ template <class T, bool WVH, int MODE> struct DwProblem {
     }
     tile_coords(tile, plan.tiles, tiles_p, tiles_q, 8, 8, tp, tq);
   }
-  LCE_DEV int item_ktiles(int local) const { return first + local < plan.full ? plan.kt : plan.kseg; }
+  LCE_DEV int item_ktiles(int local) const {
+    const int item = first + local;
+    if (item < plan.full) return plan.kt;
+    const int seg = (item - plan.full) % plan.nseg;
+    return seg == plan.nseg - 1 ? plan.kt - seg * plan.kseg : plan.kseg;
+  }
   LCE_DEV void origins(int local, const void*& p, const void*& q) const {
     int item, tp, tq, seg;
     decode(local, item, tp, tq, seg);
     const int64_t k0 = seg < 0 ? 0 : (int64_t)seg * plan.kseg * kBK;  // first token of the segment
     p = x + k0 * ldx + (int64_t)tp * kTile;
-    q = reinterpret_cast<const E*>(a.dz) + k0 * a.vs + (int64_t)tq * kTile;
+    q = reinterpret_cast<const E*>(a.dz) + ((int64_t)tq * (kTile / kBK) * a.dz_rows + k0) * kBK;
   }
-  // x rows past the last one read as zeros; dz is written for whole token tiles
+  // x rows past the last one read as zeros.  dz is written for whole token tiles of 256 rows, and the K tiles of
+  // the plan end with the pair of K tiles that holds the last row (dw_plan), so none of them reaches past
+  // the rows that were written -- except when there is no row at all: then dz reads as zeros too.
   LCE_DEV const void* p_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV const void* q_end() const {
-    return reinterpret_cast<const E*>(a.dz) + (rows + kTile - 1) / kTile * kTile * a.vs;
+    return reinterpret_cast<const E*>(a.dz) + (rows > 0 ? a.dz_rows * a.vs : 0);
   }
   LCE_DEV int k_valid(int) const { return (int)a.Np; }
   LCE_DEV void prefetch(int) {}
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdAr
   typedef typename elem_of<T>::type E;
   DwProblem<T, WVH, MODE> prob(a);
   Pipe3<T, E, false, E, false, DwProblem<T, WVH, MODE>> pipe(prob);
-  pipe.run(prob.ldx, a.vs, prob.plan.kt, lds);
+  pipe.run(prob.ldx, a.dz_rows, prob.plan.kt, lds);
 }
 
 // Second step for the tail tiles: kTailParts workgroups share tail tile b (16 of its rows each) -- they sum

@@ -5,10 +5,11 @@
 // (times 2^dz_shift, a power of two that keeps small probabilities in fp16's normal range)
 // (linear_cross_entropy/ops.py:309-314 and 415-422), rounded once to the
 // 16-bit compute type exactly where the reference casts dz before its dot
-// products (ops.py:314, 422).  The tile is transposed through LDS and written
-// to the row-major staging buffer dz[N][vs] of the current vocabulary slab as
-// full 128-byte lines.  The kernel is persistent (one workgroup per CU, operand
-// stream pipelined across tiles); fp32 operands are converted on the way into LDS.
+// products (ops.py:314, 422).  The staging buffer of the current vocabulary slab
+// is laid out in groups of 64 columns (BwdArgs::dz): a token's 64 columns of a
+// group are one 128-byte line, and dz leaves the compute unit as whole lines,
+// transposed through a small LDS area that the main loop does not use.
+// The kernel is persistent (one workgroup per CU, operand stream pipelined across tiles).
 #include "lce_gemm3.h"
 #include "lce_internal.h"
 
@@ -17,10 +18,15 @@ namespace lce {
 namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr int kPassCols = 64;                        // columns staged per pass
-constexpr int kSliceBytes = kWaveTile * kPassCols * 2;  // one wave's staging slice: 128 rows of 128 bytes
-constexpr int kLdsBytes = kMainloopLds;  // the epilogue stages through main-loop stage 1, idle by then
-static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must fit beside one stage");
+constexpr int kGroup = 64;               // columns per group of the stage
+constexpr int kPieceBytes = kBlk * kGroup * 2;   // 32 tokens x 64 columns: what a wave stages at a time
+constexpr int kWaveLds = 2 * kPieceBytes;        // two pieces per wave (the two column groups of its slice)
+constexpr int kLdsBytes = kMainloopLds + 4 * kWaveLds;  // the main loop's stages, then the epilogue's pieces
+static_assert(kLdsBytes <= 160 * 1024, "a compute unit has 160 KiB of LDS");
+#ifndef LCE_DZ_STORE_AUX
+#define LCE_DZ_STORE_AUX 2
+#endif
+constexpr int kDzStoreAux = LCE_DZ_STORE_AUX;  // cache policy of the dz stores: 2 = nt (streaming)
 
 // Turns the finished logit tile (tp, tq) into dz and writes it out.
 //
@@ -28,17 +34,23 @@ static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must
 // per token, four consecutive entries per register quad; lanes l and l+32 hold
 // the two halves of every run of 8 entries.  One v_permlane32_swap per pair of
 // register quads hands each lane a full run of 8 (16 bytes in the 16-bit
-// staging type).  A wave stages its own 128(token) x 128(v) sub-tile through a
-// private slice of `scratch` in two passes of 64 columns and reads it back as
-// whole 128-byte rows, so dz leaves the CU as full lines; no other wave is
-// involved, hence no workgroup barrier until the very end.  Staging rows are
-// 128 bytes with the 16-byte chunk index XOR-ed by (row & 7) ^ ((row >> 3) & 1),
-// the swizzle of the K-contiguous operand tiles, for the 16-byte writes (32
-// rows per instruction) and the row reads (8 rows per instruction).
+// staging type).  A wave stages 32 tokens x 64 columns at a time (a piece: the
+// tokens of one accumulator block, one column group) in its own LDS area and
+// reads the piece back as whole 128-byte lines, 8 consecutive tokens (1 KiB of
+// the stage) per store instruction; measured against storing the 16-byte runs
+// straight from the registers (32-byte sectors of 32 different lines per
+// instruction): 3 % of the kernel in favour of whole lines, 10 % with streaming
+// stores.  Lines of a piece have their 16-byte chunk index XOR-ed by
+// (line & 7) ^ ((line >> 3) & 1), the swizzle of the K-contiguous operand tiles,
+// for the 16-byte writes (32 lines per instruction) and the line reads (8 lines
+// per instruction).  The area lies behind the main loop's stages and only its
+// own wave touches it: no barrier, a wave that is done moves on by itself.
 //   * ignored tokens use lse = +inf, which makes every exp2 an exact +0;
-//   * the "- onehot" is applied by the one lane that owns the target column,
-//     from the fp32 value, onto the staged pass (one rounding, as in
-//     ops.py:313-314).
+//   * the "- onehot" is applied afterwards by the one lane that owns the target
+//     column: it waits for the wave's stores, then overwrites the staged
+//     softmax value with the rounding of the fp32 (p - 1) (one rounding, as in
+//     ops.py:313-314).  A wave meets a target in about one tile out of eight at
+//     a vocabulary of 131072, so the wait is rare.
 //
 // VTAIL is the variant for the one tile column that straddles the end of the
 // vocabulary: every run of 8 columns (a pair of register quads in lanes l, l+32)
@@ -47,12 +59,12 @@ static_assert(4 * kSliceBytes <= kLdsBytes - kStageBytes, "four wave slices must
 // are written as exact zeros.
 //
 // SPLIT (fp32 tensors carried as bf16 pairs, lce_gemm.h): dz is staged as hi = bf16(dz) and lo = bf16(dz - hi)
-// in three blocks of Np rows, [hi ; lo ; hi].  The staging sequence simply runs twice, once per part (this
+// in three blocks of Np rows per column group, [hi ; lo ; hi], each lane storing its 16-byte runs itself (this
 // path serves accuracy, not speed).
 // `pf_y`, `pf_lse`: label and lse of this lane's four tokens (DzProblem::prefetch), ignore_index / 0 for rows that do not exist.
 template <class T, bool ZREG, bool VTAIL, bool SPLIT>
 LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], const float (&pf_lse)[kNB],
-                              f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* scratch) {
+                              f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* pieces) {
   typedef typename elem_of<T>::type E;
   const int64_t v0 = a.v0 + (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
   const int tid = opaque_tid();
@@ -66,8 +78,25 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
   const int vrem = VTAIL ? (int)(left < 0 ? 0 : (left > kWaveTile ? kWaveTile : left)) : kWaveTile;
   const int nq = vrem >> 3, cut = vrem & 7;
   const int cut_mine = cut - 4 * half;  // elements of this lane's quad of the cut run that exist (<= 0: none)
-  char* mine = scratch + wave * kSliceBytes;
-  E* out = reinterpret_cast<E*>(a.dz) + (t0 + wq * kWaveTile) * a.vs + (int64_t)tp * kTile + wp * kWaveTile;
+  // This wave's 128 columns are two column groups (accumulator blocks 0, 1 and 2, 3); `row` = this lane's
+  // token row of block qb = 0 in the first of them.
+  const int64_t grp = a.dz_rows * kGroup;  // elements per column group
+  const int wpu = __builtin_amdgcn_readfirstlane(wp), wqu = __builtin_amdgcn_readfirstlane(wq);  // (uniform, for the scalar unit)
+  E* wave_base = reinterpret_cast<E*>(a.dz) + (int64_t)(tp * (kTile / kGroup) + wpu * (kWaveTile / kGroup)) * grp +
+                 (t0 + wqu * kWaveTile) * kGroup;
+  E* row = wave_base + (lane & 31) * kGroup;
+  const int64_t blk = a.Np * kGroup;  // SPLIT: elements between the three blocks of a column group
+  // Stores go through a buffer descriptor over this wave's part of the stage (scalar base, one 32-bit offset per
+  // lane, the block's offset as a scalar): no 64-bit vector address arithmetic.  All offsets stay below 2^31
+  // (dz_rows * 128 bytes for the second column group, plus two blocks of a bf16-pair stage).
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(wave_base, 0, 0x7fffffff, 0x00020000);
+  const unsigned lane_off = (unsigned)((lane & 31) * (kGroup * 2) + half * 16);
+  // staging: this lane's line of a piece when it writes (its token), and line / chunk when it reads back: 8 lines
+  // per instruction, 8 lanes each; the upper 32 lanes take their four lines in the order 5, 4, 7, 6 so that lanes
+  // l and l+32 always sit in lines of opposite parity (opposite bank halves)
+  char* mine = pieces + wave * kWaveLds;
+  const int wline = lane & 31, wsw = (wline & 7) ^ ((wline >> 3) & 1);
+  const int rline = (lane >> 3) + ((lane >> 5) ? 1 - 2 * ((lane >> 3) & 1) : 0), rchunk = lane & 7;
 
   // per-token scalars of this lane's four tokens
   float nlse[kNB], gain[kNB];
@@ -85,47 +114,37 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
     ykey[qb] = (valid && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == half) ? (int)rel : -1;
   }
 
-  const int64_t blk = a.Np * a.vs;  // SPLIT: elements between the three blocks of the stage
 #pragma unroll
-  for (int part = 0; part < (SPLIT ? 2 : 1); ++part) {
-  // (SPLIT: an opaque copy of the scale per part, so that the compiler recomputes the exponentials of part 1 instead of
-  // keeping all 256 of part 0 alive across the staging of that part, which spilled 2 KiB per lane)
-  float c1p = c1;
-  if (SPLIT) asm volatile("" : "+v"(c1p));
+  for (int qb = 0; qb < kNB; ++qb) {
 #pragma unroll
-  for (int ph = 0; ph < 2; ++ph) {
+    for (int pb = 0; pb < kNB; ++pb) {
+      const unsigned blk_off = (unsigned)((pb >> 1) * grp * 2) + qb * (kBlk * kGroup * 2);  // bytes, uniform
 #pragma unroll
-    for (int qb = 0; qb < kNB; ++qb) {
-      const int row = qb * kBlk + (lane & 31);
-      char* lrow = mine + row * (kPassCols * 2);
-      const int sw = (row & 7) ^ ((row >> 3) & 1);
+      for (int g = 0; g < 4; g += 2) {
+        float d[8];
 #pragma unroll
-      for (int pp = 0; pp < 2; ++pp) {
-        const int pb = 2 * ph + pp;
+        for (int h2 = 0; h2 < 2; ++h2) {
+          if (!VTAIL || pb * 4 + g + h2 < nq) {
 #pragma unroll
-        for (int g = 0; g < 4; g += 2) {
-          float d[8];
-#pragma unroll
-          for (int h2 = 0; h2 < 2; ++h2) {
-            if (!VTAIL || pb * 4 + g + h2 < nq) {
-#pragma unroll
-              for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
-                d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1p, nlse[qb]));
-                if (ZREG) d[i] *= gain[qb];
-              }
-            } else if (pb * 4 + g + h2 == nq && cut != 0) {
-#pragma unroll
-              for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
-                d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1p, nlse[qb]));
-                if (ZREG) d[i] *= gain[qb];
-                d[i] = (i - 4 * h2) < cut_mine ? d[i] : 0.f;
-              }
-            } else {
-#pragma unroll
-              for (int i = 4 * h2; i < 4 * h2 + 4; ++i) d[i] = 0.f;
+            for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
+              d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
+              if (ZREG) d[i] *= gain[qb];
             }
+          } else if (pb * 4 + g + h2 == nq && cut != 0) {
+#pragma unroll
+            for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
+              d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
+              if (ZREG) d[i] *= gain[qb];
+              d[i] = (i - 4 * h2) < cut_mine ? d[i] : 0.f;
+            }
+          } else {
+#pragma unroll
+            for (int i = 4 * h2; i < 4 * h2 + 4; ++i) d[i] = 0.f;
           }
-          if (SPLIT && part == 1) {
+        }
+#pragma unroll
+        for (int part = 0; part < (SPLIT ? 2 : 1); ++part) {
+          if (part == 1) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) d[i] = bf16_lo(d[i]);
           }
@@ -140,47 +159,62 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
           o[1] = s1[0];
           o[2] = s0[1];
           o[3] = s1[1];
-          const int chunk = pp * 4 + g + half;  // 16-byte chunk of the 64-column pass
-          *reinterpret_cast<u32x4_t*>(lrow + ((chunk ^ sw) << 4)) = o;
+          // streaming stores (aux 2 = nt): dz (1 GiB per slab) is read back from memory by the next kernels anyway,
+          // and a normal store would evict the W / x tiles the following main loop is about to reuse from L2
+          if constexpr (SPLIT) {
+            const unsigned voff = lane_off + (pb & 1) * (kBlk * 2) + g * 16;
+            const unsigned soff = blk_off + (part == 1 ? (unsigned)(blk * 2) : 0u);
+            __builtin_amdgcn_raw_buffer_store_b128(o, rsrc, (int)voff, (int)soff, kDzStoreAux);
+            if (part == 0) __builtin_amdgcn_raw_buffer_store_b128(o, rsrc, (int)voff, (int)(soff + (unsigned)(blk * 4)), kDzStoreAux);
+          } else {
+            const int chunk = (pb & 1) * 4 + g + half;  // 16-byte chunk of the token's line
+            *reinterpret_cast<u32x4_t*>(mine + (pb >> 1) * kPieceBytes + wline * (kGroup * 2) + ((chunk ^ wsw) << 4)) = o;
+          }
         }
       }
-      // the target column, if it falls into this pass: overwrite the staged value
-      // with the rounding of the fp32 (p - 1), as ops.py:313-314 rounds once
-      const int yl = ykey[qb] - ph * kPassCols;
-      if (yl >= 0 && yl < kPassCols) {
-        const int want = (yl >> 5) * 16 + ((yl >> 3) & 3) * 4 + (yl & 3);  // (pp, register) index
-        float zt = 0.f;
+    }
+    if constexpr (!SPLIT) {
+      // read the two pieces back as 128-byte lines and send them out
 #pragma unroll
-        for (int pp = 0; pp < 2; ++pp)
+      for (int gi = 0; gi < 2; ++gi)
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
-            if (want == pp * 16 + r) zt = acc[2 * ph + pp][qb][r];
-        float p = __builtin_amdgcn_exp2f(fmaf(zt, c1p, nlse[qb]));
-        if (ZREG) p *= gain[qb];
-        float tv = p - __builtin_bit_cast(float, (127 + a.dz_shift) << 23);  // the one, times 2^dz_shift
-        if (SPLIT && part == 1) tv = bf16_lo(tv);
-        *reinterpret_cast<unsigned short*>(lrow + (((yl >> 3) ^ sw) << 4) + (yl & 7) * 2) = to_bits<T>(tv);
+        for (int i = 0; i < 4; ++i) {
+          const int line = i * 8 + rline;
+          const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + gi * kPieceBytes + line * (kGroup * 2) +
+                                                              ((rchunk ^ (line & 7) ^ ((line >> 3) & 1)) << 4));
+          const unsigned soff = (unsigned)(gi * grp * 2) + qb * (kBlk * kGroup * 2);
+          __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, line * (kGroup * 2) + rchunk * 16, (int)soff, kDzStoreAux);
+        }
+    }
+    // The target column of this lane's token, if it lies in this wave's slice: the staged softmax value is
+    // replaced by the rounding of the fp32 (p - 1), once the wave's stores above have reached memory (the
+    // 16-byte piece that holds the column may have been another lane's store).  (These rare branches also keep
+    // the compiler from gathering the accumulator reads of all four blocks at the top, which spills.)
+    const int yl = ykey[qb];
+    if (yl >= 0) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      const int want = (yl >> 5) * 16 + ((yl >> 3) & 3) * 4 + (yl & 3);  // (block, register) index
+      float zt = 0.f;
+#pragma unroll
+      for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          // (a volatile read: the compiler would otherwise hoist the 64 accumulator reads above the branch)
+          float v;
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[pb][qb][r]));
+          if (want == pb * 16 + r) zt = v;
+        }
+      float p = __builtin_amdgcn_exp2f(fmaf(zt, c1, nlse[qb]));
+      if (ZREG) p *= gain[qb];
+      const float tv = p - __builtin_bit_cast(float, (127 + a.dz_shift) << 23);  // the one, times 2^dz_shift
+      E* at = row + (yl >> 6) * grp + qb * (kBlk * kGroup) + (yl & (kGroup - 1));
+      *reinterpret_cast<unsigned short*>(at) = to_bits<T>(tv);
+      if (SPLIT) {
+        *reinterpret_cast<unsigned short*>(at + 2 * blk) = to_bits<T>(tv);
+        *reinterpret_cast<unsigned short*>(at + blk) = to_bits<T>(bf16_lo(tv));
       }
-      // keep the register footprint small: an operand tile is in flight across this function
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // read the pass back as 128-byte rows and send it out
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      // 8 rows per instruction, 8 lanes each; the upper 32 lanes take their four rows in the order
-      // 5, 4, 7, 6 so that lanes l and l+32 always sit in rows of opposite parity (opposite bank halves)
-      const int row = i * 8 + (lane >> 3) + ((lane >> 5) ? 1 - 2 * ((lane >> 3) & 1) : 0), chunk = lane & 7;
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(mine + row * (kPassCols * 2) + ((chunk ^ (row & 7) ^ ((row >> 3) & 1)) << 4));
-      // streaming store: dz (1 GiB per slab) is read back from HBM by the next kernels anyway, and a
-      // normal store would evict the W / x tiles the following main loop is about to reuse from L2
-      E* dst = out + (int64_t)row * a.vs + ph * kPassCols + chunk * 8 + (SPLIT && part == 1 ? blk : 0);
-      __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(dst));
-      if (SPLIT && part == 0) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(dst + 2 * blk));
-      if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most 4 rows in registers at a time
     }
   }
-  }
-  __syncthreads();  // scratch is handed back to the main loop
 }
 
 // ZREG (z_regularization != 0) is a compile-time switch of the kernels rather than a
@@ -195,6 +229,7 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> stru
   static constexpr bool kKMask = KMASK;
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
+  static constexpr bool kQGrouped = false;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows: all of x, or the packed rows (see BwdArgs)
   const E* x;
@@ -246,7 +281,7 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> stru
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
     coords(tile, tp, tq);
-    dz_epilogue_impl<T, ZREG, VTAIL, SPLIT>(a, pf_y, pf_lse, acc, tp, tq, scratch);
+    dz_epilogue_impl<T, ZREG, VTAIL, SPLIT>(a, pf_y, pf_lse, acc, tp, tq, scratch + kStageBytes);  // (behind the main loop's stages)
   }
 };
 

@@ -162,6 +162,7 @@ template <class T, bool VTAIL, bool KMASK, bool WVH> struct FwdProblem {
   static constexpr bool kKMask = KMASK;
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
+  static constexpr bool kQGrouped = false;
   const FwdArgs& a;
   int64_t rows, ldx;
   const E* x;

@@ -69,8 +69,12 @@ template <class T> LCE_DEV unsigned short to_bits(float f) {
   typename elem_of<T>::type h = (typename elem_of<T>::type)f;
   return __builtin_bit_cast(unsigned short, h);
 }
+// Two floats -> one dword of the 16-bit type (a single v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32).
 template <class T> LCE_DEV unsigned int pack2(float lo, float hi) {
-  return (unsigned int)to_bits<T>(lo) | ((unsigned int)to_bits<T>(hi) << 16);
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef typename elem_of<T>::type e2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, e2_t));
 }
 // fp32 operands are carried as two bf16 numbers, v = hi + lo with hi = bf16(v) and lo = bf16(v - hi): 16
 // bits of mantissa instead of 8.  A product a*b is then taken as a_hi*b_hi + a_hi*b_lo + a_lo*b_hi (the

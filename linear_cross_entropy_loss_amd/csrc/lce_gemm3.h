@@ -84,6 +84,23 @@ template <class T, class SrcT, bool KC, bool KMASK> struct Stager3 {
     base = end = nullptr;
     range = 0;
   }
+  // The operand is stored in groups of 64 columns, [cols / 64][rows][64] with `rows` rows per group (the
+  // staged dz, see lce_bwd_dz.hip), instead of row-major.  KC (its columns are the K index): the 256 rows x
+  // 64 k of a K tile are one contiguous block of 128-byte rows, and the next K tile is the next group.
+  // Otherwise (its rows are the K index): the tile's 256 columns are four groups, each thread stays in one.
+  // The byte offsets of a tile's chunks (up to 3 groups + 64 rows) must fit 31 bits: rows < 5.5 million.
+  LCE_DEV void init_grouped(int64_t rows) {
+    init(kBK);
+    if (KC) {
+      k_stride = rows * (kBK * kEs);
+    } else {
+      const int t = threadIdx.x, c = t & 31, k = t >> 5;
+      voff = (unsigned)(((int64_t)(c >> 3) * rows + k) * (kBK * kEs) + (c & 7) * 16);
+      voff_cur = voff;
+      iter_stride = (unsigned)(8 * kBK * kEs);
+      k_stride = (int64_t)kBK * kBK * kEs;
+    }
+  }
   // Called whenever `base` moves.  `k_rem` = valid k elements from the start of
   // this K tile on.  Along K a K-contiguous operand runs on into the next row, so
   // its threads past the K extent are switched to an out-of-range offset; a
@@ -140,6 +157,8 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //        of P block i and Q block j, with Q along its registers and P along its lanes)
 //   void prefetch(int tile)                       called three K tiles before the tile's epilogue: the place to issue loads
 //        of per-row data the epilogue starts with (kept in members), so that their latency is not exposed there
+//   static constexpr bool kQGrouped               true if the Q operand is stored in groups of 64 columns (Stager3::init_grouped);
+//        run() then takes the rows per group in place of the Q row stride
 //   static constexpr bool kKMask                  false if `ktiles * 64 == k_valid` for every tile of the launch
 //   int  k_valid(int tile)                        K extent of that tile's contraction; the K tiles of the
 //        loop may run past it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
@@ -330,7 +349,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
     ktiles = ktiles_;
     const int wave = threadIdx.x >> 6;
     ps.init(ldp);
-    qs.init(ldq);
+    if constexpr (Problem::kQGrouped) qs.init_grouped(ldq); else qs.init(ldq);
     pr.init((wave & 1) * kWaveTile);
     qr.init((wave >> 1) * kWaveTile);
 

@@ -88,7 +88,12 @@ struct BwdArgs {
   // w_vh != 0: weight and dW are stored with the vocabulary as their row index, w[v * ldw + h], dw[v * lddw + h]
   // (and the buffer `w` holds ROWS [wv0, wv0 + Vw)); otherwise w[h * ldw + v], dw[h * lddw + v].
   int w_vh;
-  void* dz;         // [Np][vs] staged dz in the compute type (exact zeros outside N x vw)
+  // Staged dz in the compute type (exact zeros outside N x vw), stored in groups of 64 columns:
+  // element (row, v) of the slab sits at dz[((v / 64) * dz_rows + row) * 64 + v % 64], so that the 64-deep K tiles
+  // of the dx contraction (K = v) are contiguous blocks of 128-byte rows, and a token's 64 columns of a group are
+  // one 128-byte line.  dz_rows = Np, or 3 Np when dz is carried as bf16 pairs (`split` below).
+  void* dz;
+  int64_t dz_rows;
   float* dx_acc;    // [Np][Hp] fp32 running dx (null when there is a single slab)
   // dx: tiles of a last, mostly idle round of workgroups are cut along K instead (planned on the device,
   // see lce_bwd_dx.hip); the segments' partial sums meet in dx_part, dx_tail_blocks() blocks of 256 x 256
@@ -108,9 +113,9 @@ struct BwdArgs {
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
   int live;         // bwd_dz: bands of W that the XCDs keep in flight together (lce_gemm.h, tile_coords)
-  // fp32 tensors carried as bf16 pairs (lce_gemm.h): dz is staged as three blocks of Np rows,
-  // [hi ; lo ; hi], `dz` pointing at the first; only bwd_dz looks at this flag (the dx and dW launches get
-  // plain 16-bit problems over these blocks).
+  // fp32 tensors carried as bf16 pairs (lce_gemm.h): every column group of the stage holds three blocks of Np
+  // rows, [hi ; lo ; hi]; only bwd_dz looks at this flag (the dx and dW launches get plain 16-bit problems over
+  // these blocks: dx with `dz` pointing at the first row of a block, dW with 3 Np token rows).
   int split;
   // Packed rows (tokens with an ignored label dropped; n_rows == null: the call works on all rows).
   // *n_rows (device) rows are worked on.  When *n_rows != N they are the rows of xc (row stride ldxc) and
