@@ -237,6 +237,7 @@ template <class T, bool WVH, int MODE> struct DwProblem {
   static constexpr bool kVarK = true;    // whole tiles and segment items have different K extents
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
   static constexpr bool kQGrouped = true;  // dz is staged in groups of 64 columns (BwdArgs::dz)
+  static constexpr bool kColumnEpilogue = false;
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows (the K extent): all of x, or the packed rows (see BwdArgs)

@@ -160,6 +160,7 @@ template <class T, bool KMASK, bool WVH, int MODE> struct DxProblem {
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = MODE == kDxTails;  // segment items have their own K extent
   static constexpr bool kQGrouped = true;          // dz is staged in groups of 64 columns (BwdArgs::dz)
+  static constexpr bool kColumnEpilogue = false;
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
   int64_t rows;  // token rows: all, or the packed ones (see BwdArgs)

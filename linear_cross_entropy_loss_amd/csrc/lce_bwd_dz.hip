@@ -230,6 +230,7 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> stru
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
   static constexpr bool kQGrouped = false;
+  static constexpr bool kColumnEpilogue = false;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows: all of x, or the packed rows (see BwdArgs)
   const E* x;

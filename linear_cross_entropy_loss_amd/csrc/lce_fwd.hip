@@ -35,7 +35,8 @@ LCE_DEV float fast_log(float v) { return __builtin_amdgcn_logf(v) * kLn2; }
 // halves), so every run but at most one is inside or outside the vocabulary as a
 // whole, uniformly over the wave, and is taken or skipped with a scalar branch;
 // the one run that V cuts through is handled element by element.
-template <class T, bool VTAIL>
+// MON: the monitoring partials (slice max, sum softmax*z, sum z^2) are formed as well.
+template <class T, bool VTAIL, bool MON>
 LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
   const int64_t v0 = (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;  // t0: inside the chunk of rows of this launch
   const int tid = opaque_tid();
@@ -58,7 +59,7 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
     if (VTAIL && vrem == 0) {  // nothing of this slice exists
       if (lane < 32) {
         a.part_lse[o] = -INFINITY;
-        if (a.monitoring) {
+        if (MON) {
           a.part_max[o] = -INFINITY;
           a.part_pz[o] = 0.f;
           a.part_sq[o] = 0.f;
@@ -87,7 +88,7 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
     m *= a.scale;  // logit_scale > 0, so max commutes with the scaling
     const float mo = m * kLog2e;
     float s = 0.f, pz = 0.f, sq = 0.f;
-    if (a.monitoring) {
+    if (MON) {
 #pragma unroll
       for (int pb = 0; pb < kNB; ++pb)
 #pragma unroll
@@ -132,7 +133,7 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
     s += __shfl_xor(s, 32);
     if (lane < 32) {
       a.part_lse[o] = m + fast_log(s);
-      if (a.monitoring) {
+      if (MON) {
         a.part_max[o] = m;
         a.part_pz[o] = pz / s;
         a.part_sq[o] = sq;
@@ -151,18 +152,140 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
   }
 }
 
+
+// The same reduction for the kernels whose last K tile is multiplied column by column (Pipe3::step_last_columns;
+// full tiles, no monitoring): one block column of the accumulator at a time -- 32 tokens along the lanes, this
+// wave's 128 vocabulary entries of each token in 4 x 16 registers of lanes l and l + 32 -- cut into 16 slots of
+// straight-line code that run behind the matrix instructions of the next column.  A lane folds its 64 values
+// in two chunks of 32 (slots 8c .. 8c + 7 of chunk c) into a running (max, sum of exp2) pair, so that only 32
+// accumulator values are in vector registers at a time, and meets the other half of the slice in lane ^ 32.
+struct FwdColumnState {
+  float v[32];   // the chunk being summed
+  float m, s;    // running max (unscaled logits) and sum of exp2(scaled logit - scaled max)
+  float mo;      // scaled max of the chunk being summed
+  float e[4], f; // exponentials of the last slot, not yet added; factor for the sum at a chunk change
+};
+// The logit of the target column, written by the one lane that holds it (rare: a wave holds the target of
+// one token in a thousand at a vocabulary of 131072).  `yl`: the column inside this wave's 128-wide slice if
+// this lane's half holds it, else -1.
+LCE_DEV void fwd_store_target(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int64_t tok, int qb, int yl) {
+  if (yl >= 0) {
+    const int want = (yl >> 5) * 16 + ((yl >> 3) & 3) * 4 + (yl & 3);  // (block, register) index
+    float zt = 0.f;
+#pragma unroll
+    for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        // (a volatile read: the compiler would otherwise hoist the 64 accumulator reads above the branch)
+        float v;
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[pb][qb][r]));
+        if (want == pb * 16 + r) zt = v;
+      }
+    a.tgt[tok] = zt * a.scale;
+  }
+}
+
+// Slot 0..15 of block column QB: the running (max, sum) of this lane's 64 values.
+template <int QB>
+LCE_DEV void fwd_slot_sum(const FwdArgs& a, FwdColumnState& st, f32x16_t (&acc)[kNB][kNB], int slot) {
+  const float c1 = a.scale * kLog2e;
+  const int c = slot >> 3, sub = slot & 7;  // chunk c: accumulator blocks 2c, 2c + 1, slots 8c .. 8c + 7
+  if (sub == 0) {
+#pragma unroll
+    for (int r = 0; r < 32; ++r) st.v[r] = acc[2 * c + (r >> 4)][QB][r & 15];
+    float cm = st.v[0];
+#pragma unroll
+    for (int r = 1; r < 32; ++r) cm = fmaxf(cm, st.v[r]);
+    const float mn = c == 0 ? cm : fmaxf(st.m, cm);
+    st.mo = mn * c1;  // logit_scale > 0, so max commutes with the scaling
+    if (c == 0) st.s = 0.f; else st.f = fast_exp2(fmaf(st.m, c1, -st.mo));  // factor that moves the sum to the new max
+    st.m = mn;
+  }
+  // (the exponentials of a slot are added up in the next one, when they are there)
+  if (slot > 0) st.s += (st.e[0] + st.e[1]) + (st.e[2] + st.e[3]);
+  if (sub == 0 && c > 0) st.s *= st.f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) st.e[r] = fast_exp2(fmaf(st.v[4 * sub + r], c1, -st.mo));
+  if (slot == 15) st.s += (st.e[0] + st.e[1]) + (st.e[2] + st.e[3]);
+}
+// After slot 15: the other half of the slice.  Leaves the slice's max (unscaled) in st.m and its sum of exp2 in st.s.
+LCE_DEV void fwd_merge_halves(const FwdArgs& a, FwdColumnState& st) {
+  const float c1 = a.scale * kLog2e;
+  // after the swaps both lanes of a pair hold the lower lane's value in [0] and the upper lane's in [1]
+  const unsigned mb = __builtin_bit_cast(unsigned, st.m), sb = __builtin_bit_cast(unsigned, st.s);
+  const auto mm = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
+  const auto ss = __builtin_amdgcn_permlane32_swap(sb, sb, false, false);
+  // (elements copied to scalars first: a bit cast applied to a vector element reads element 0 whichever is named)
+  const unsigned m0u = mm[0], m1u = mm[1], s0u = ss[0], s1u = ss[1];
+  const float m0 = __builtin_bit_cast(float, m0u), m1 = __builtin_bit_cast(float, m1u);
+  const float s0 = __builtin_bit_cast(float, s0u), s1 = __builtin_bit_cast(float, s1u);
+  const float mt = fmaxf(m0, m1), mo = mt * c1;
+  st.s = s0 * fast_exp2(fmaf(m0, c1, -mo)) + s1 * fast_exp2(fmaf(m1, c1, -mo));
+  st.m = mt;
+}
+template <class T, int QB>
+LCE_DEV void fwd_epilogue_slot(const FwdArgs& a, FwdColumnState& st, f32x16_t (&acc)[kNB][kNB], int tp, int tq, int slot) {
+  fwd_slot_sum<QB>(a, st, acc, slot);
+  if (slot == 15) {
+    fwd_merge_halves(a, st);
+    const float lse = fmaf(st.m, a.scale, fast_log(st.s));
+    // one store per token: the upper lanes get an offset that the range check of the buffer store drops
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t slice = ((int64_t)tp * kTile + (wave & 1) * kWaveTile) / kChunkV;
+    float* base = a.part_lse + slice * a.nc + (int64_t)tq * kTile + (wave >> 1) * kWaveTile + QB * kBlk;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(base, 0, kBlk * 4, 0x00020000);
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, lse), rsrc, lane < 32 ? lane * 4 : (int)0x80000000, 0, 0);
+  }
+}
+
+// Full tiles with monitoring: the same (max, sum) arithmetic, so that the loss does not depend on the monitoring
+// flag bit for bit, then the slice's sum softmax*z and sum z^2 in a second pass over the column.
+template <class T, int QB>
+LCE_DEV void fwd_epilogue_column_mon(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, int64_t tok, int yl) {
+  FwdColumnState st;
+#pragma unroll
+  for (int slot = 0; slot < 16; ++slot) fwd_slot_sum<QB>(a, st, acc, slot);
+  fwd_merge_halves(a, st);
+  const float c1 = a.scale * kLog2e, mo = st.m * c1;
+  float pz = 0.f, sq = 0.f;
+#pragma unroll
+  for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float e = fast_exp2(fmaf(acc[pb][QB][r], c1, -mo));
+      const float z = acc[pb][QB][r] * a.scale;
+      pz = fmaf(e, z, pz);
+      sq = fmaf(z, z, sq);
+    }
+  pz += __shfl_xor(pz, 32);
+  sq += __shfl_xor(sq, 32);
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int64_t slice = ((int64_t)tp * kTile + (wave & 1) * kWaveTile) / kChunkV;
+  const int64_t o = slice * a.nc + (int64_t)tq * kTile + (wave >> 1) * kWaveTile + QB * kBlk + (lane & 31);
+  if (lane < 32) {
+    a.part_lse[o] = fmaf(st.m, a.scale, fast_log(st.s));
+    a.part_max[o] = st.m * a.scale;
+    a.part_pz[o] = pz / st.s;
+    a.part_sq[o] = sq;
+  }
+  fwd_store_target(a, acc, tok, QB, yl);
+}
+
 // Persistent workgroups, operand stream pipelined across output tiles.  The
 // launch covers `tiles_p` tile columns of the vocabulary window [v0, v0 + vw)
 // starting at its column tile `tp0` (all full columns, or the one straddling V
 // for the VTAIL variant).  The token rows are those of x, or -- when the tokens with ignored
 // labels were packed away -- the first `rows` rows of the packed copy (the count lives on the device).
 // WVH: the weight is stored (V, H) row-major, so that the P operand runs along K in memory like x does.
-template <class T, bool VTAIL, bool KMASK, bool WVH> struct FwdProblem {
+template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON> struct FwdProblem {
   typedef typename elem_of<T>::type E;
   static constexpr bool kKMask = KMASK;
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
   static constexpr bool kQGrouped = false;
+  static constexpr bool kColumnEpilogue = !VTAIL && !MON;
   const FwdArgs& a;
   int64_t rows, ldx;
   const E* x;
@@ -195,20 +318,71 @@ template <class T, bool VTAIL, bool KMASK, bool WVH> struct FwdProblem {
   }
   LCE_DEV const void* q_end() const { return matrix_end<E>(x, rows, ldx, a.H); }
   LCE_DEV int k_valid(int) const { return (int)a.H; }
-  LCE_DEV void prefetch(int) {}
+  // Column epilogue: the labels of this lane's four tokens are fetched three K tiles ahead.
+  int64_t pf_y[kNB];
+  int etp, etq;
+  LCE_DEV void prefetch(int tile) {
+    if constexpr (kColumnEpilogue) {
+      int tp, tq;
+      coords(tile, tp, tq);
+      const int lane = threadIdx.x & 63, wq = threadIdx.x >> 7;
+#pragma unroll
+      for (int qb = 0; qb < kNB; ++qb) {
+        const int64_t tok = a.row0 + (int64_t)tq * kTile + wq * kWaveTile + qb * kBlk + (lane & 31);
+        pf_y[qb] = tok < rows ? a.y[tok] : a.ignore_index;
+      }
+    }
+  }
+  LCE_DEV void epilogue_begin(int tile) {
+    coords(tile, etp, etq);
+    etp += (int)(a.v0 / kTile);
+  }
+  FwdColumnState est;
+  template <int J> LCE_DEV void epilogue_slot(int, f32x16_t (&acc)[kNB][kNB], int slot, char*) {
+    fwd_epilogue_slot<T, J>(a, est, acc, etp, etq, slot);
+  }
+  LCE_DEV void epilogue_end(int, f32x16_t (&acc)[kNB][kNB], char*) const {
+    const int tid = opaque_tid();
+    const int lane = tid & 63, wave = tid >> 6;
+    const int64_t slice_v0 = (int64_t)etp * kTile + (wave & 1) * kWaveTile;
+#pragma unroll
+    for (int qb = 0; qb < kNB; ++qb) {
+      const int64_t tok = a.row0 + (int64_t)etq * kTile + (wave >> 1) * kWaveTile + qb * kBlk + (lane & 31);
+      const int64_t yy = pf_y[qb], rel = yy - slice_v0;
+      const bool here = yy != a.ignore_index && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == (lane >> 5);
+      fwd_store_target(a, acc, tok, qb, here ? (int)rel : -1);
+    }
+  }
+  template <int QB> LCE_DEV void column_mon(f32x16_t (&acc)[kNB][kNB], int tp, int tq) const {
+    const int tid = opaque_tid();
+    const int lane = tid & 63, wave = tid >> 6;
+    const int64_t slice_v0 = (int64_t)tp * kTile + (wave & 1) * kWaveTile;
+    const int64_t tok = a.row0 + (int64_t)tq * kTile + (wave >> 1) * kWaveTile + QB * kBlk + (lane & 31);
+    const int64_t yy = tok < rows ? a.y[tok] : a.ignore_index, rel = yy - slice_v0;
+    const bool here = yy != a.ignore_index && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == (lane >> 5);
+    fwd_epilogue_column_mon<T, QB>(a, acc, tp, tq, tok, here ? (int)rel : -1);
+  }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     coords(tile, tp, tq);
-    fwd_epilogue<T, VTAIL>(a, rows, acc, (int)(a.v0 / kTile) + tp, tq);
+    tp += (int)(a.v0 / kTile);
+    if constexpr (VTAIL) {
+      fwd_epilogue<T, VTAIL, MON>(a, rows, acc, tp, tq);
+    } else {
+      column_mon<0>(acc, tp, tq);
+      column_mon<1>(acc, tp, tq);
+      column_mon<2>(acc, tp, tq);
+      column_mon<3>(acc, tp, tq);
+    }
   }
 };
 
-template <class T, bool VTAIL, bool KMASK, bool WVH>
+template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON>
 __global__ __launch_bounds__(kThreads) void fwd_tiles_persistent_kernel(const FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  FwdProblem<T, VTAIL, KMASK, WVH> prob(a);
-  Pipe3<T, E, WVH, E, true, FwdProblem<T, VTAIL, KMASK, WVH>> pipe(prob);
+  FwdProblem<T, VTAIL, KMASK, WVH, MON> prob(a);
+  Pipe3<T, E, WVH, E, true, FwdProblem<T, VTAIL, KMASK, WVH, MON>> pipe(prob);
   pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
@@ -361,9 +535,9 @@ __global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
   }
 }
 
-template <class T, bool VTAIL, bool KMASK, bool WVH>
+template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON>
 hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = fwd_tiles_persistent_kernel<T, VTAIL, KMASK, WVH>;
+  auto kern = fwd_tiles_persistent_kernel<T, VTAIL, KMASK, WVH, MON>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
   if (e != hipSuccess) return e;
@@ -373,26 +547,30 @@ hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
 }
 
 // All full tile columns of the vocabulary, then the column that straddles V.
-template <class T, bool WVH> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
+template <class T, bool WVH, bool MON> hipError_t launch_persistent(const FwdArgs& a, hipStream_t s) {
   const int64_t left = a.Np - a.row0;  // token tiles of this chunk at most
   const int64_t tq = (left < a.nc ? left : a.nc) / kTile, full = a.vw / kTile;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = exact_k ? launch_one<T, false, false, WVH>(a, full * tq, s)
-                           : launch_one<T, false, true, WVH>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, false, false, WVH, MON>(a, full * tq, s)
+                           : launch_one<T, false, true, WVH, MON>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (a.vw % kTile) return launch_one<T, true, true, WVH>(a, tq, s);
+  if (a.vw % kTile) return launch_one<T, true, true, WVH, MON>(a, tq, s);
   return hipSuccess;
+}
+
+template <class T, bool WVH> hipError_t launch_layout(const FwdArgs& a, hipStream_t s) {
+  return a.monitoring ? launch_persistent<T, WVH, true>(a, s) : launch_persistent<T, WVH, false>(a, s);
 }
 
 }  // namespace
 
 hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s) {
   if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16)
-    return a.w_vh ? launch_persistent<BF16, true>(a, s) : launch_persistent<BF16, false>(a, s);
+    return a.w_vh ? launch_layout<BF16, true>(a, s) : launch_layout<BF16, false>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16)
-    return a.w_vh ? launch_persistent<F16, true>(a, s) : launch_persistent<F16, false>(a, s);
+    return a.w_vh ? launch_layout<F16, true>(a, s) : launch_layout<F16, false>(a, s);
   // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as the bf16 packed copy)
   return hipErrorInvalidValue;
 }

@@ -36,6 +36,8 @@ struct StageRegs {
   u32x4_t v[8];
 };
 
+#define LCE_SG_VALU 0x002
+#define LCE_SG_TRANS 0x400
 #define LCE_SG_MFMA 0x008
 #define LCE_SG_VMEM_RD 0x020
 #define LCE_SG_DS_RD 0x100
@@ -162,6 +164,16 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //   static constexpr bool kKMask                  false if `ktiles * 64 == k_valid` for every tile of the launch
 //   int  k_valid(int tile)                        K extent of that tile's contraction; the K tiles of the
 //        loop may run past it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
+//   static constexpr bool kColumnEpilogue          true if the epilogue works through the accumulator one block column
+//        (Q block: 32 lanes' worth of Q rows, all 128 P rows of the wave) at a time, in 16 slots of straight-line
+//        vector ALU code per column:
+//          void epilogue_begin(int tile)                  per-tile scalars, kept in members
+//          template <int J> void epilogue_slot(int tile, acc, int slot, char* extra)   slot 0..15 of column J
+//          (acc[0..3][J]); no branches, no barriers; state between slots in members
+//          void epilogue_end(int tile, acc, char* extra)  whatever is rare and branchy, after the last column
+//        The last K tile of an output tile is then multiplied column by column, and slot k of column j runs
+//        behind the k-th matrix instruction of column j + 1 (step_last_columns).  `extra`: LDS behind the two stages
+//        (the launch must provide it), which the main loop never touches.  Otherwise:
 //   void epilogue(int tile, acc, char* scratch)
 //        consumes the finished accumulator; may use `scratch`, 96 KiB of LDS
 //        that the pipeline does not touch until the next barrier it issues
@@ -344,6 +356,67 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
     __builtin_amdgcn_sched_barrier(0);
   }
 
+
+  // The last K tile of an output tile, for a problem whose epilogue works column by column
+  // (Problem::kColumnEpilogue), with that epilogue.  The 64 matrix instructions of the K tile are issued one
+  // block column of the accumulator after the other (all four k-steps of column 0, then of column 1, ...):
+  // column j is final when column j + 1 starts, and its epilogue -- vector ALU work that would otherwise run
+  // with the matrix pipe idle -- is cut into 16 slots, one behind each matrix instruction of column j + 1.  Only
+  // the last column's epilogue runs on its own.  The order is fixed in the source, slot by slot (a scheduling
+  // barrier after each): left to the compiler, with or without scheduling groups, the matrix instructions end
+  // up in a row ahead of the epilogue.  The K tile's 16 P fragments stay in registers once read (64 VGPRs, where the
+  // steady-state loop double-buffers 8 + 8 fragments), the Q fragments come one k-step ahead of their use.
+  // Everything else is as in step<1, false, false, true>: the staging set (K tile 0 of the next output tile) goes to
+  // LDS stage 0 (one chunk per slot of column 0) and is refilled with its K tile 1 (one chunk per slot of column
+  // 1); one workgroup barrier.  Each accumulator block still sums its k-steps in the same order, so the result
+  // is bit-identical to the row-by-row order.
+  template <int J>
+  LCE_DEV void last_column(f32x16_t (&acc)[kNB][kNB], PRegs& sp, QRegs& sq, s16x8_t (&pa)[4][kNB], s16x8_t (&qk)[2],
+                           int tile) {
+    const char* cur = lds + kStageBytes;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int n = 4 * J + ks, nn = n + 1;  // Q fragment of k-step n = 4 * column + ks lives in buffer n & 1
+      // one k-step ahead: the Q fragment of the next k-step (of the next column after the last) and, in column 0,
+      // the P fragments of the next k-step, which then stay for the other columns
+      if (nn < 16) qk[nn & 1] = qr.read(cur + kTileBytes, nn >> 2, nn & 3);
+      if (J == 0 && ks < 3) {
+#pragma unroll
+        for (int b = 0; b < kNB; ++b) pa[ks + 1][b] = pr.read(cur, b, ks + 1);
+      }
+#pragma unroll
+      for (int i = 0; i < kNB; ++i) {
+        const int slot = 4 * ks + i;
+        acc[i][J] = Problem::kSwapAB ? mfma32<T>(qk[n & 1], pa[ks][i], acc[i][J])
+                                     : mfma32<T>(pa[ks][i], qk[n & 1], acc[i][J]);
+        if (J == 0) store_chunks(sp, sq, lds, slot, slot + 1);
+        if (J == 1) load_chunks(sp, sq, slot, slot + 1);
+        if constexpr (J > 0) prob.template epilogue_slot<J - 1>(tile, acc, slot, lds + kMainloopLds);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  LCE_DEV void step_last_columns(f32x16_t (&acc)[kNB][kNB], PRegs& sp, QRegs& sq, int tile) {
+    s16x8_t pa[4][kNB], qk[2];  // the K tile's P fragments [k-step][block]; two Q fragments
+#pragma unroll
+    for (int b = 0; b < kNB; ++b) pa[0][b] = pf[0][b];
+    qk[0] = qf[0][0];
+    prob.epilogue_begin(tile);
+    last_column<0>(acc, sp, sq, pa, qk, tile);
+    last_column<1>(acc, sp, sq, pa, qk, tile);
+    stream_advance();
+    last_column<2>(acc, sp, sq, pa, qk, tile);
+    last_column<3>(acc, sp, sq, pa, qk, tile);
+    // the barrier: every wave's part of the next K tile is in LDS stage 0, and no wave reads this stage any more
+    __syncthreads();
+#pragma unroll
+    for (int slot = 0; slot < 16; ++slot) {
+      prob.template epilogue_slot<3>(tile, acc, slot, lds + kMainloopLds);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    prob.epilogue_end(tile, acc, lds + kMainloopLds);
+  }
+
   LCE_DEV void run(int64_t ldp, int64_t ldq, int ktiles_, char* lds_) {
     lds = lds_;
     ktiles = ktiles_;
@@ -379,8 +452,12 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
       prob.prefetch(tile);  // three K tiles ahead of the epilogue
       step<1, false, true, false>(acc, sp, sq);
       step<0, false, false, false>(acc, sp, sq);
-      step<1, false, false, true>(acc, sp, sq);
-      prob.epilogue(tile, acc, lds + kStageBytes);
+      if constexpr (Problem::kColumnEpilogue) {
+        step_last_columns(acc, sp, sq, tile);
+      } else {
+        step<1, false, false, true>(acc, sp, sq);
+        prob.epilogue(tile, acc, lds + kStageBytes);
+      }
     }
   }
 };
