@@ -169,58 +169,79 @@ def host_cpu_model():
     return "unknown"
 
 
-def cpu_baseline(cfg, torch, rows=2048):
-    """Eager fp32 linear + F.cross_entropy fwd+bwd on all host cores, on a bounded row sample of the same workload.
+def cpu_baseline(cfg, torch, chunk=2048, budget_s=75.0):
+    """Eager fp32 linear + F.cross_entropy fwd+bwd on all host cores over the WHOLE workload, as an N-chunked eager
+    loop: `chunk` rows at a time (the N x V fp32 logits and their gradient, 16 GiB at the default shape, never exist
+    at once), every chunk's gradients accumulated -- the same mathematics as one unchunked step.
 
-    Inputs by the workload's own recipe (x ~ N(0,1), W truncated normal with std 1/sqrt(H), the workload's labels
-    and ignored fraction) upcast to fp32; 1 warm-up + 3 timed steps, median.  The whole workload would need the
-    N x V fp32 logits and their gradient on the host (16 GiB at the default shape), so the first `rows` tokens
-    are timed at full H and V and the rate is what is reported: the cost per token does not depend on N.
+    Inputs by the workload's own recipe (x ~ N(0,1), W truncated normal with std 1/sqrt(H), the workload's labels and
+    ignored fraction) in fp32; a warm-up over one chunk, then up to three timed steps (median), fewer when a step
+    takes so long that three would exceed `budget_s` seconds; a workload whose single step would exceed it (config
+    5: about 600 s) is timed on its first chunks only and says so.
     """
-    from oracle import eager_fp32_step
+    from oracle import eager_fp32_step_chunked
 
-    H, V = cfg["H"], cfg["V"]
-    Ns = min(cfg["N"], rows)
+    N, H, V = cfg["N"], cfg["H"], cfg["V"]
     # all host cores of this job: the box's share (OMP_NUM_THREADS there) where that is smaller than what the OS shows
     torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS") or (os.cpu_count() or 1))))
     g = torch.Generator().manual_seed(cfg["seed"])
-    x = torch.randn(Ns, H, generator=g)
     std = 1.0 / math.sqrt(H)
     w = torch.empty(H, V)
     torch.nn.init.trunc_normal_(w, mean=0.0, std=std, a=-3 * std, b=3 * std, generator=g)
-    if cfg.get("zipf"):
-        p = torch.arange(1, V + 1, dtype=torch.float64) ** -1.1
-        y = torch.searchsorted(torch.cumsum(p, 0) / p.sum(), torch.rand(Ns, generator=g, dtype=torch.float64)).clamp_(max=V - 1)
-    else:
-        y = torch.randint(0, V, (Ns,), generator=g)
-    if cfg["ignore"] > 0:
-        y[torch.rand(Ns, generator=g) < cfg["ignore"]] = -1
     threads = torch.get_num_threads()
-    eager_fp32_step(x, y, w, -1, cfg["z_reg"], cfg["scale"])  # warm-up
-    ts = []
-    for _ in range(3):
+
+    def inputs(n):
+        x = torch.randn(n, H, generator=g)
+        if cfg.get("zipf"):
+            p = torch.arange(1, V + 1, dtype=torch.float64) ** -1.1
+            y = torch.searchsorted(torch.cumsum(p, 0) / p.sum(), torch.rand(n, generator=g, dtype=torch.float64)).clamp_(max=V - 1)
+        else:
+            y = torch.randint(0, V, (n,), generator=g)
+        if cfg["ignore"] > 0:
+            y[torch.rand(n, generator=g) < cfg["ignore"]] = -1
+        return x, y
+
+    def timed(x, y):
         t0 = time.perf_counter()
-        eager_fp32_step(x, y, w, -1, cfg["z_reg"], cfg["scale"])
-        ts.append(time.perf_counter() - t0)
-    t = sorted(ts)[1]
-    return dict(value=8.0 * Ns * H * V / t / 1e12, unit=f"TFLOP/s (8*N*H*V convention, on a {Ns}-token sample)",
+        eager_fp32_step_chunked(x, y, w, -1, cfg["z_reg"], cfg["scale"], chunk=chunk)
+        return time.perf_counter() - t0
+
+    xw, yw = inputs(min(N, chunk))
+    t_chunk = timed(xw, yw)  # warm-up (one chunk), also the estimate of a step
+    est = t_chunk * math.ceil(N / chunk)
+    if est <= budget_s:
+        Ns = N
+        x, y = inputs(N)
+        reps = max(1, min(3, int(budget_s / est)))
+    else:  # bounded sample: as many whole chunks as fit about a third of the budget
+        Ns = min(N, chunk * max(1, int(budget_s / 3 / t_chunk)))
+        x, y = inputs(Ns)
+        reps = 1
+    ts = sorted(timed(x, y) for _ in range(reps))
+    t = ts[(reps - 1) // 2]
+    whole = Ns == N
+    return dict(value=8.0 * Ns * H * V / t / 1e12, unit="TFLOP/s",
                 cores=threads, kind="port", host_cpu=host_cpu_model(), os_cpu_count=os.cpu_count(),
                 torch_num_threads=threads,
-                sample=f"first {Ns} of {cfg['N']} tokens at full H={H}, V={V}, inputs by the workload's recipe; eager "
-                       f"fp32 matmul + F.cross_entropy fwd+bwd; 1 warm-up + 3 timed, median; {t * 1e3:.0f} ms per "
-                       f"sample step",
-                ms_per_sample_step=t * 1e3)
+                sample=(f"the whole workload: all {N} tokens at H={H}, V={V} in {math.ceil(N / chunk)} chunks of {chunk} rows"
+                        if whole else
+                        f"the first {Ns} of {N} tokens at full H={H}, V={V} in chunks of {chunk} rows (one step of the "
+                        f"whole workload would take about {est:.0f} s)") +
+                       f", inputs by the workload's recipe; eager fp32 matmul + F.cross_entropy fwd+bwd with gradients "
+                       f"accumulated over the chunks; warm-up over one chunk, {reps} timed step(s), median; "
+                       f"8*N*H*V FLOP convention",
+                ms_per_step=t * 1e3 * (N / Ns), ms_per_step_is_measured=whole, timed_steps=reps,
+                tokens_timed=Ns)
 
 
 def sources_sha16():
-    """Hash of the operator's kernel sources (the measurement probes are a library of their own and do not count):
-    profiles/hbm_traffic.json carries the one its counters were collected on."""
+    """Hash of the operator's kernel sources: profiles/hbm_traffic.json carries the one its counters were collected on."""
     import hashlib
 
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "linear_cross_entropy_loss_amd", "csrc")
     for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".h")) and name != "lce_probe.hip":
+        if name.endswith((".hip", ".h")):
             with open(os.path.join(csrc, name), "rb") as f:
                 h.update(name.encode() + b"\0" + f.read())
     return h.hexdigest()[:16]
@@ -283,142 +304,6 @@ def c4_sweep(args, torch):
     }
 
 
-def _events_ms(fn, torch, reps):
-    fn()
-    torch.cuda.synchronize()
-    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    s.record()
-    for _ in range(reps):
-        fn()
-    e.record()
-    torch.cuda.synchronize()
-    return s.elapsed_time(e) / reps
-
-
-def _load_probe_lib():
-    from linear_cross_entropy_loss_amd.build import PROBE_LIB_PATH
-
-    if not PROBE_LIB_PATH.exists():
-        raise RuntimeError(f"{PROBE_LIB_PATH} is missing: run `python -m linear_cross_entropy_loss_amd.build`")
-    lib = ctypes.CDLL(str(PROBE_LIB_PATH))
-    vp = ctypes.c_void_p
-    lib.lce_probe_mfma.restype = ctypes.c_int
-    lib.lce_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp]
-    lib.lce_probe_mfma_loads.restype = ctypes.c_int
-    lib.lce_probe_mfma_loads.argtypes = [ctypes.c_int, ctypes.c_int, vp, ctypes.c_uint64, ctypes.c_int, ctypes.c_int, vp, vp]
-    lib.lce_probe_flush.restype = ctypes.c_int
-    lib.lce_probe_flush.argtypes = [ctypes.c_int, vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, vp]
-    return lib
-
-
-def probe_ceiling(torch):
-    """What bounds the tile kernels on this part: (1) a register-only loop of the same MFMA instruction over
-    the same 128 x 128 wave tile, on constant and on random operands, with the tile kernels' LDS reads and
-    writes added, with their operand loads from L2 added as well, with their one barrier per K tile, and with a
-    quarter of the loads missing L2 (still no epilogues), on all and on half of the compute units;
-    (2) the vendor GEMM (torch.matmul -> hipBLASLt) on the four contractions of the default workload; (3) the
-    operator's forward tile kernel on all and on half of the compute units (a chip-level power limit shows as a
-    higher rate per compute unit when fewer of them run)."""
-    from linear_cross_entropy_loss_amd import _lib
-
-    probe = _load_probe_lib()
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    out = {"probe": "ceiling", "compute_units": cus, "peak_bf16_tflops_published": PEAK_TFLOPS["bf16"], "mfma_loop": [],
-           "vendor_gemm": [], "fwd_tiles": []}
-    buf = torch.empty(cus * 256 * 4, dtype=torch.float32, device="cuda")
-    iters = 200000
-    # operand windows of the loads patterns: 2 MiB of random bf16 in [-2, 2) each.  One window walked by all workgroups
-    # stays in every L2; with 64 of them (128 MiB: resident in the Infinity Cache, 16 MiB per XCD: not in its L2), one per
-    # four workgroups of an XCD, a quarter of the requests goes over the fabric, as in the tile kernels
-    window = (torch.rand(64 << 20, device="cuda") * 4 - 2).to(torch.bfloat16)
-    for wgs in (cus, cus // 2):
-        for pattern, name in ((0, "constant operands"), (1, "random bf16 operands"),
-                              (2, "random, fragments re-read from LDS"), (3, "random, LDS reads + LDS writes"),
-                              (4, "random, LDS traffic + operand loads"),
-                              (5, "random, LDS traffic + loads + barrier"),
-                              (6, "same, a quarter of the loads over fabric")):
-            def run():
-                if pattern >= 4:
-                    rc = probe.lce_probe_mfma_loads(wgs, iters, ctypes.c_void_p(window.data_ptr()), 2 << 20,
-                                                    64 if pattern == 6 else 1, int(pattern >= 5),
-                                                    ctypes.c_void_p(buf.data_ptr()), stream)
-                else:
-                    rc = probe.lce_probe_mfma(pattern, wgs, iters, ctypes.c_void_p(buf.data_ptr()), stream)
-                assert rc == 0
-            ms = _events_ms(run, torch, 3)
-            flops = wgs * 4.0 * iters * 16 * 32768
-            out["mfma_loop"].append(dict(operands=name, workgroups=wgs, waves_per_simd=1, ms=ms,
-                                         tflops=flops / ms / 1e9, tflops_per_cu=flops / ms / 1e9 / wgs))
-    del window
-    N, H, V = 16384, 2048, 131072
-    g = torch.Generator(device="cuda").manual_seed(2)
-    x = torch.randn(N, H, device="cuda", generator=g).to(torch.bfloat16)
-    w = (torch.randn(H, V // 4, device="cuda", generator=g) / math.sqrt(H)).to(torch.bfloat16)
-    dz = (torch.randn(N, V // 4, device="cuda", generator=g) * 1e-3).to(torch.bfloat16)
-    for name, a, b in (("logits of one slab  x[N,H] @ W[H,V/4]", x, w), ("dx of one slab  dz[N,V/4] @ W^T", dz, w.t()),
-                       ("dW of one slab  x^T @ dz[N,V/4]", x.t(), dz)):
-        ms = _events_ms(lambda: torch.matmul(a, b), torch, 10)
-        out["vendor_gemm"].append(dict(gemm=name, ms=ms, tflops=2.0 * N * H * (V // 4) / ms / 1e9))
-    del dz
-    wf = (torch.randn(H, V, device="cuda", generator=g) / math.sqrt(H)).to(torch.bfloat16)
-    ms = _events_ms(lambda: torch.matmul(x, wf), torch, 5)
-    out["vendor_gemm"].append(dict(gemm="all logits  x[N,H] @ W[H,V]", ms=ms, tflops=2.0 * N * H * V / ms / 1e9))
-    # the operator's own forward tile kernel, all compute units against half of them
-    lib = _lib.load()
-    y = torch.randint(0, V, (N,), device="cuda", generator=g)
-    lse = torch.empty(N, device="cuda")
-    out5 = torch.empty(5, device="cuda")
-    nv = torch.empty(1, dtype=torch.int64, device="cuda")
-    P = lambda t: ctypes.c_void_p(t.data_ptr())
-    for cap in (0, cus // 2):
-        p = _lib.make_problem(N, H, V, H, V, H, V, x.dtype, wf.dtype, x.dtype, wf.dtype, -1, 1.0, 0.0, 4096, False,
-                              _lib.PHASE_FWD_TILES, _lib.PACK_NEVER, cap)
-        fwd_b, _ = _lib.workspace_bytes(p)
-        ws = torch.empty(fwd_b, dtype=torch.uint8, device="cuda")
-
-        def run():
-            rc = lib.lce_forward(ctypes.byref(p), P(x), P(wf), P(y), P(lse), P(out5), P(nv), P(ws), fwd_b, stream)
-            assert rc == 0
-        ms = _events_ms(run, torch, 5)
-        n = cap or cus
-        out["fwd_tiles"].append(dict(workgroups=n, ms=ms, tflops=2.0 * N * H * V / ms / 1e9,
-                                     tflops_per_cu=2.0 * N * H * V / ms / 1e9 / n))
-    return out
-
-
-def probe_flush(torch):
-    """Cost of flushing 256 x 256 fp32 blocks of partial sums into a matrix in memory, the traffic a backward
-    would generate that fed every dz tile straight into the dx and dW contractions: a compute unit cannot hold
-    an H-wide accumulator (256 x H fp32 = 2 MiB at H = 2048 against 512 KiB of registers), so each
-    256-token x 256-column dz tile would add H/256 blocks to dW and H/256 blocks to dx."""
-    probe = _load_probe_lib()
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    H, Vs = 2048, 32768  # one slab of dW in fp32: 256 MiB
-    dst = torch.zeros(H, Vs, dtype=torch.float32, device="cuda")
-    tiles = 64
-    out = {"probe": "flush", "compute_units": cus, "target": f"fp32 [{H}][{Vs}]", "block": "256 x 256 fp32 = 256 KiB",
-           "modes": []}
-    for atomic, name in ((1, "fp32 atomic add (global_atomic_add_f32)"), (0, "plain 16-byte load + add + store (no other writer)")):
-        def run():
-            rc = probe.lce_probe_flush(atomic, ctypes.c_void_p(dst.data_ptr()), H, Vs, tiles, cus, stream)
-            assert rc == 0
-        ms = _events_ms(run, torch, 3)
-        payload = cus * tiles * 256 * 256 * 4
-        out["modes"].append(dict(mode=name, ms=ms, blocks=cus * tiles, us_per_block_per_cu=ms * 1e3 / tiles,
-                                 payload_TB_per_s=payload / ms / 1e9))
-    # what the default workload would flush per step: R/256 x V/256 dz tiles, each 2 * H/256 blocks
-    N, V = 16384, 131072
-    dz_tiles = (N // 256) * (V // 256)
-    blocks = dz_tiles * 2 * (H // 256)
-    out["fused_backward_at_default_shape"] = dict(
-        dz_tiles=dz_tiles, blocks_flushed=blocks, payload_GiB=blocks * 256 * 256 * 4 / 2 ** 30,
-        ms_at_measured_rate={m["mode"]: blocks * 256 * 256 * 4 / (m["payload_TB_per_s"] * 1e9) for m in out["modes"]},
-        note="to be compared with the 19 ms the whole staged backward takes (dz through a 16-bit buffer in HBM)")
-    return out
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -426,9 +311,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_bf16_N16384_H2048_V131072", choices=sorted(WORKLOADS) + ["c4_sweep"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--probe", choices=["ceiling", "flush"],
-                    help="run a measurement probe instead of the benchmark and print its JSON: 'ceiling' (register-only "
-                         "MFMA loop, vendor GEMM, half of the compute units), 'flush' (partial-sum blocks into memory)")
+    ap.add_argument("--probe", choices=["ceiling", "flush", "overlap"],
+                    help="run a measurement probe instead of the benchmark and print its JSON (built on demand, "
+                         "linear_cross_entropy_loss_amd/probes): 'ceiling' (register-only MFMA loop, vendor GEMM, half of "
+                         "the compute units), 'flush' (partial-sum blocks into memory), 'overlap' (epilogue arithmetic "
+                         "behind matrix instructions)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic, to scale "
                          "FETCH_SIZE / WRITE_SIZE counters collected with rocprofv3 --pmc)")
@@ -451,7 +338,9 @@ def main():
         build(force=True)
 
     if args.probe:
-        print(json.dumps(probe_ceiling(torch) if args.probe == "ceiling" else probe_flush(torch)))
+        from linear_cross_entropy_loss_amd import probes
+
+        print(json.dumps(probes.run(args.probe, torch)))
         return
     if args.workload == "c4_sweep":
         print(json.dumps(c4_sweep(args, torch)))
@@ -553,6 +442,9 @@ def main():
         "peak_hbm_bytes_incl_grads": int(peak_bytes),
         "peak_hbm_bytes_extra": int(peak_bytes - out_bytes),
         "scratch_budget_bytes": int(cfg["n_chunk"] * V * 4),
+        # device memory the library's code object holds on every GPU it runs on, outside the allocator's statistics:
+        # the fixed scratch array of lce_forward_static (not used by this benchmark)
+        "static_scratch_bytes_per_gpu": int(_lib.STATIC_SCRATCH_BYTES),
         "kernels": phases,
         "roofline": roofline,
     }

@@ -15,7 +15,8 @@
  *     (H, V) row-major with row stride ldw (linear_cross_entropy/ops.py:913);
  *     y is N contiguous int64 labels (ops.py:210), each ignore_index or in
  *     [0, V); any other value makes the returned loss NaN.
- *   - Shapes: any N, H, V, n_chunk >= 1 (N, V <= 2^30, H <= 2^20).  The
+ *   - Shapes: any N, H, V, n_chunk >= 1 (N <= 2^22 -- 2^20 for fp32
+ *     activations --, V <= 2^30, H <= 2^20).  The
  *     reference's divisibility rules (N % 512, H % 256, V % 4096,
  *     ops.py:689-691, 905-907) are lifted; shapes that obey them run at full
  *     speed, others pay for partly empty tiles.
@@ -131,8 +132,7 @@ enum {
  * scales with the number of labelled tokens; the pre-pass costs a few small
  * launches (about 0.04 ms per forward + backward), which a small problem does
  * not earn back.  LCE_PACK_AUTO packs when 8*N*H*V >= 2^41 FLOPs; results are
- * the same either way up to the summation order of dW and the loss, and lse of
- * an ignored row (see lce_forward).  Use the same value in lce_workspace_bytes,
+ * the same either way up to the summation order of dW and the loss.  Use the same value in lce_workspace_bytes,
  * lce_forward and lce_backward of one problem.
  */
 enum {
@@ -201,8 +201,8 @@ int lce_backward_plan(const lce_problem* p, int64_t* slabs, int64_t* slab_width)
  * 793-794, 802), without ever writing logits to memory.
  *
  *   lse     out, N floats: logsumexp of the scaled logits of every row whose
- *           label is not ignore_index (when rows are packed and monitoring
- *           == 0 the other rows are not computed at all and get 0)
+ *           label is not ignore_index; 0 for the other rows, whether rows are
+ *           packed (such rows are then not computed at all) or not
  *   out5    out, 5 floats: loss, z_reg, logit_max, logit_entropy, logit_norm
  *           (the 5-tuple of ops.py:802 with the meanings of ops.py:9-17; the
  *           last three are 0 when monitoring == 0)
@@ -222,8 +222,15 @@ int lce_forward(const lce_problem* p, const void* x, const void* w, const int64_
  * holds until the process ends.  The call allocates and frees nothing.
  *
  *   - A problem whose lce_workspace_bytes forward size exceeds
- *     LCE_STATIC_SCRATCH_BYTES is refused with LCE_ESTATIC (e.g. N = 4096 rows
- *     at V = 131072, H = 2048 fits; N = 16384 does not): use lce_forward.
+ *     LCE_STATIC_SCRATCH_BYTES is refused with LCE_ESTATIC: use lce_forward.
+ *     At V = 131072, H = 2048: N = 4096 rows need 32.1 MiB with monitoring
+ *     == 0 and fit; with monitoring != 0 they need 64.02 MiB (four partial
+ *     buffers of 16 MiB plus the per-token items) and do not, N = 2048 does;
+ *     N = 16384 does not fit either way.
+ *   - The array is part of the library's code object: every process holds
+ *     LCE_STATIC_SCRATCH_BYTES of device memory on every GPU it runs the
+ *     library on, whether or not this entry point is ever called, outside any
+ *     allocator's statistics.
  *   - All calls on one GPU share that GPU's array: calls that overlap in time
  *     on one GPU (two streams, two threads) race.  Calls on one stream, or
  *     otherwise ordered, are fine; nothing is carried from one call to the next.

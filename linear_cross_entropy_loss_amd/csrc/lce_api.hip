@@ -29,6 +29,9 @@ int check(const lce_problem* p, bool backward) {
   if (p->N <= 0 || p->H <= 0 || p->V <= 0 || p->n_chunk <= 0) return LCE_EINVAL_SHAPE;
   // Any N, H, V; only the row strides are constrained (below).
   if (p->N > (int64_t)1 << 30 || p->V > (int64_t)1 << 30 || p->H > (int64_t)1 << 20) return LCE_EINVAL_SHAPE;
+  // The dz stage is addressed in column groups of all token rows (BwdArgs::dz) through 32-bit byte offsets that
+  // span up to four groups: 4 * rows * 128 bytes must stay below 2^31 (three times the rows for bf16 pairs).
+  if (p->N > ((int64_t)1 << 22) / (p->x_dtype == LCE_F32 ? 4 : 1)) return LCE_EINVAL_SHAPE;
   const int xd = p->x_dtype, wd = p->w_dtype;
   const bool ok = (is16(xd) && (wd == xd || wd == LCE_F32)) || (xd == LCE_F32 && wd == LCE_F32);
   if (!ok) return LCE_EINVAL_DTYPE;
@@ -138,7 +141,8 @@ FwdPlan plan_fwd(const lce_problem* p) {
   // memory by all eight XCDs; over a long launch they drift apart and stop sharing what they fetch.  Launches
   // of 32768 columns bring them back in step (measured at N = 16384, H = 8192, V = 131072: 24.6 ms against 27.3
   // in one launch; no difference at H = 2048, where x stays in the cache).
-  if ((size_t)f.nc * (size_t)p->H * 2 > ((size_t)128 << 20) && f.vs > 32768) f.vs = 32768;
+  // (fp32 activations reach the tile kernels as bf16 pairs, three times as wide)
+  if ((size_t)f.nc * (size_t)(splits(p) ? 3 * p->H : p->H) * 2 > ((size_t)128 << 20) && f.vs > 32768) f.vs = 32768;
   if (p->w_dtype == LCE_F32) {
     // slab copies of at most 256 MiB (at least one tile column)
     const int64_t hw = splits(p) ? 3 * p->H : p->H;  // rows of the copy
@@ -461,7 +465,8 @@ const char* lce_strerror(int status) {
   switch (status) {
     case LCE_OK: return "ok";
     case LCE_EINVAL_SHAPE:
-      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N, V <= 2^30, H <= 2^20; "
+      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N <= 2^22 (2^20 for fp32 activations), "
+             "V <= 2^30, H <= 2^20; "
              "ceil(N/256) * ceil(V/256) <= 2^28)";
     case LCE_EINVAL_DTYPE:
       return "unsupported dtype combination (x: bf16/f16/f32; w: x dtype or f32; grads: same dtype or f32)";
@@ -550,7 +555,9 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
   a.ignore_index = p->ignore_index;
   a.scale = p->logit_scale; a.z_reg = p->z_reg;
   a.dx = dx; a.dw = dw;
-  // fp16 staging of dz: times 2^10, unless z_reg is so large that (1 + 2 * z_reg * lse) * 2^10 could leave fp16's range
+  // fp16 staging of dz: times 2^10, unless z_reg is so large that the factor 1 + 2 * z_reg * lse on top of it would
+  // leave fp16's range for ordinary logits (with the factor 2^10 in place bwd_dz clamps that factor to +-63, which
+  // |lse| < 992 never reaches at z_reg <= 1/32)
   a.dz_shift = p->x_dtype == LCE_F16 && p->z_reg <= 0.03125f ? 10 : 0;
   a.dz = base + b.dz;
   a.dx_acc = b.slabs > 1 || splits(p) ? (float*)(base + b.dx_acc) : nullptr;

@@ -110,6 +110,8 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
     // (the power-of-two factor of the staged dz rides along in the exponent)
     nlse[qb] = valid ? fmaf(-l, kLog2e, (float)a.dz_shift) : -INFINITY;
     gain[qb] = 1.f + 2.f * a.z_reg * l;
+    // (with the staging factor 2^10 of fp16 in place: |dz| * 2^10 <= 63 * 2^10 stays finite in fp16 whatever lse is)
+    if (a.dz_shift != 0) gain[qb] = fminf(fmaxf(gain[qb], -63.f), 63.f);
     // target column inside this wave's slice, only in the lane half that holds it
     ykey[qb] = (valid && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == half) ? (int)rel : -1;
   }

@@ -333,7 +333,7 @@ template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON> struct FwdProblem
       }
     }
   }
-  LCE_DEV void epilogue_begin(int tile) {
+  LCE_DEV void epilogue_begin(int tile, char*) {
     coords(tile, etp, etq);
     etp += (int)(a.v0 / kTile);
   }
@@ -396,7 +396,8 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
   const int64_t tok = a.row0 + tokl;  // < Np; rows that do not exist only keep the block sums aligned
   const int64_t rows = a.n_rows ? packed_rows(a.n_rows, a.N) : a.N;
   const bool exists = tok < rows;
-  // packed rows: lse goes back to the token's own place; tokens that were dropped get 0
+  // packed rows: lse goes back to the token's own place; tokens that were dropped get 0 (as every token with an
+  // ignored label does, below)
   if (a.perm != nullptr && g == 1 && tok < a.N && a.y0[tok] == a.ignore_index) a.lse[tok] = 0.f;
   const int nslices = (int)(a.Vp / kChunkV);
 
@@ -433,7 +434,10 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
       if (sh_s[i][r] != 0.f) St += sh_s[i][r] * fast_exp2((sh_m[i][r] - Mt) * kLog2e);
     const float lse = Mt + fast_log(St);
     sh_lse[r] = lse;
-    if (exists) a.lse[a.perm != nullptr ? packed_token(a.perm, tok, a.N) : tok] = lse;
+    // lse[i] of a token with an ignored label is 0, whether its row was computed (all rows are when they are not
+    // packed) or not: a caller sees one thing.  (sh_lse keeps the value: logit_entropy is taken over valid rows only,
+    // and the backward never looks at the lse of such a token.)
+    if (exists) a.lse[a.perm != nullptr ? packed_token(a.perm, tok, a.N) : tok] = a.y[tok] != a.ignore_index ? lse : 0.f;
   }
   __syncthreads();
   const float lse = sh_lse[r];

@@ -167,7 +167,7 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //   static constexpr bool kColumnEpilogue          true if the epilogue works through the accumulator one block column
 //        (Q block: 32 lanes' worth of Q rows, all 128 P rows of the wave) at a time, in 16 slots of straight-line
 //        vector ALU code per column:
-//          void epilogue_begin(int tile)                  per-tile scalars, kept in members
+//          void epilogue_begin(int tile, char* extra)     per-tile scalars, kept in members
 //          template <int J> void epilogue_slot(int tile, acc, int slot, char* extra)   slot 0..15 of column J
 //          (acc[0..3][J]); no branches, no barriers; state between slots in members
 //          void epilogue_end(int tile, acc, char* extra)  whatever is rare and branchy, after the last column
@@ -401,7 +401,7 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
 #pragma unroll
     for (int b = 0; b < kNB; ++b) pa[0][b] = pf[0][b];
     qk[0] = qf[0][0];
-    prob.epilogue_begin(tile);
+    prob.epilogue_begin(tile, lds + kMainloopLds);
     last_column<0>(acc, sp, sq, pa, qk, tile);
     last_column<1>(acc, sp, sq, pa, qk, tile);
     stream_advance();

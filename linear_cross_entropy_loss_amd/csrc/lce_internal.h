@@ -107,8 +107,9 @@ struct BwdArgs {
   // type, and the dx / dW kernels fold 2^-dz_shift into their final factor.  bf16 has fp32's exponent range and
   // needs none (0); in fp16 the softmax probabilities of a large vocabulary (of order 1/V) would fall below the
   // normal range (6.1e-5) and lose precision bit by bit -- with 10 they stay normal down to 6e-8, while
-  // |dz| * 2^10 stays below fp16's maximum for any gain = 1 + 2 * z_reg * lse below 63 (the host takes 0 instead
-  // when z_reg is large enough for that to matter).
+  // |dz| * 2^10 stays below fp16's maximum for any gain = 1 + 2 * z_reg * lse below 63: bwd_dz clamps the gain to
+  // +-63 when the factor is in place, and the host takes 0 instead when z_reg > 1/32, where logits of ordinary size
+  // (|lse| < 992 at 1/32) would already reach that.
   int dz_shift;
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels

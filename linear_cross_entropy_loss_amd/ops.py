@@ -19,6 +19,7 @@ from __future__ import annotations
 import contextvars
 import ctypes
 import math
+import warnings
 
 import torch
 
@@ -54,7 +55,23 @@ def _row_multiple(dtype):
     return 4 if dtype == torch.float32 else 8
 
 
-def _aligned_rows(t):
+_copy_warned = set()
+
+
+def _warn_copy_once(what, t, why):
+    """One warning per kind of copy: a weight that cannot be read in place is copied on every call (forward and
+    backward), which costs its size in memory and a pass over it in time."""
+    if what in _copy_warned or torch.compiler.is_compiling():
+        return
+    _copy_warned.add(what)
+    warnings.warn(
+        f"linear_cross_entropy: the {what} of shape {tuple(t.shape)}, strides {tuple(t.stride())}, {t.dtype} cannot be "
+        f"read in place ({why}) and is copied on every call ({t.numel() * t.element_size() / 2**20:.0f} MiB)",
+        stacklevel=3,
+    )
+
+
+def _aligned_rows(t, what=None):
     """`t` itself when the kernels can read it in place, else a copy whose row stride is padded with zeros.
 
     The kernels take any number of rows and columns, but rows must start on 16-byte boundaries.  Only a
@@ -64,6 +81,9 @@ def _aligned_rows(t):
     m = _row_multiple(t.dtype)
     if t.stride(-1) == 1 and t.stride(0) % m == 0 and t.stride(0) >= t.shape[1] and t.data_ptr() % 16 == 0:
         return t
+    if what is not None:
+        _warn_copy_once(what, t, f"rows must be contiguous and start on 16-byte boundaries: row strides that are "
+                                 f"multiples of {m} elements")
     rows, cols = t.shape
     padded = torch.zeros((rows, -(-cols // m) * m), dtype=t.dtype, device=t.device)
     padded[:, :cols] = t
@@ -89,8 +109,11 @@ def _weight_rows(At, layout):
     """The matrix the kernels read: (H, V) rows for W_HV, (V, H) rows for W_VH (no copy unless misaligned)."""
     if layout == _lib.W_VH:
         w = At.t()
-        return w if w.data_ptr() % 16 == 0 else w.clone(memory_format=torch.contiguous_format)
-    return _aligned_rows(At)
+        if w.data_ptr() % 16 == 0:
+            return w
+        _warn_copy_once("weight", At, "its first element is not on a 16-byte boundary")
+        return w.clone(memory_format=torch.contiguous_format)
+    return _aligned_rows(At, "weight")
 
 
 def _empty_rows(rows, cols, dtype, device):

@@ -1,4 +1,5 @@
-// Measurement probes (liblce_probe_gfx950.so; not part of the operator, loaded only by `bench.py --probe`).
+// Measurement probes (liblce_probe_gfx950.so; not part of the operator: built on demand by
+// `python -m linear_cross_entropy_loss_amd.build --probes` and loaded only by `bench.py --probe`).
 //
 //   lce_probe_mfma    what the matrix pipes of this part sustain with no data movement at all: every wave
 //                     keeps 4 A and 4 B fragments in registers and issues v_mfma_f32_32x32x16_bf16 over a
@@ -11,6 +12,9 @@
 //                     and k step are fetched with buffer loads (64 KiB per workgroup and 64-deep K tile, the window
 //                     shared by all workgroups so that it is served by the L2s) and are what the LDS writes store;
 //                     optionally with the one workgroup barrier per K tile that the tile kernels need.
+//   lce_probe_overlap how much of an epilogue's vector ALU work (fma, exp2, add per logit) hides behind matrix
+//                     instructions of the same wave: the register-only loop with k such triples behind every
+//                     MFMA, against the MFMAs alone and the triples alone.
 //   lce_probe_flush   what adding 256 x 256 fp32 blocks of partial sums into a matrix in memory costs, with
 //                     atomics or as plain read-modify-write: the traffic a backward that fed dz straight into
 //                     the dx and dW contractions would generate once per dz tile (its H-wide accumulators do
@@ -195,6 +199,68 @@ __global__ __launch_bounds__(256) void flush_kernel(float* dst, int64_t rows, in
   }
 }
 
+// mode 0: 16 MFMAs per iteration (random operands in registers); 1: KV (fma, exp2, add) triples per iteration and no
+// MFMA; 2: both, KV / 16 triples behind each MFMA.  One wave per SIMD, as in the tile kernels.
+template <int MODE, int KV>
+__global__ __launch_bounds__(256) void overlap_kernel(int iters, float* out) {
+  s16x8_t a[4], b[4];
+  const unsigned tid = blockIdx.x * 256u + threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      a[i][e] = random_bf16(tid * 64u + i * 8u + e);
+      b[i][e] = random_bf16(tid * 64u + 32u + i * 8u + e);
+    }
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  float v[16], s[16];
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    v[q] = -1.f - 0.001f * (tid & 63) - q;
+    s[q] = 0.f;
+  }
+  const float c = 0.999f + 1e-6f * (tid & 3);
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (MODE != 1)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[i]),
+                                                              __builtin_bit_cast(bf16x8_t, b[j]), acc[i][j], 0, 0, 0);
+        if (MODE != 0) {
+#pragma unroll
+          for (int u = 0; u < KV / 16; ++u) {
+            const int q = (i * 4 + j + u * 5) & 15;
+            s[q] += __builtin_amdgcn_exp2f(fmaf(v[q], c, -0.5f));
+            v[q] = v[q] * 0.99999f;  // (keeps the inputs changing)
+          }
+        }
+        if (MODE == 2) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x402, 4 * (KV / 16), 0);
+        }
+      }
+    asm volatile("" ::: "memory");
+  }
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) t += acc[i][j][r];
+#pragma unroll
+  for (int q = 0; q < 16; ++q) t += s[q] + v[q];
+  out[tid] = t;
+}
+
 }  // namespace
 
 extern "C" {
@@ -240,6 +306,22 @@ int lce_probe_flush(int atomic, float* dst, int64_t rows, int64_t ld, int tiles,
   } else {
     hipLaunchKernelGGL(flush_kernel<false>, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, dst, rows, ld, tiles);
   }
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+// Launches `wgs` workgroups of 4 waves running `iters` iterations of: mode 0, 16 MFMAs; mode 1, 16 * per_mfma
+// (fma, exp2, add) triples; mode 2, both, per_mfma triples behind each MFMA.  per_mfma: 1, 2 or 4.  out: wgs * 256 floats.
+int lce_probe_overlap(int mode, int per_mfma, int wgs, int iters, float* out, void* stream) {
+  if (mode < 0 || mode > 2 || wgs <= 0 || iters <= 0 || !out) return -3;
+  const dim3 grid((unsigned)wgs), block(256);
+  hipStream_t s = (hipStream_t)stream;
+#define LCE_OVL(M, K) hipLaunchKernelGGL((overlap_kernel<M, K>), grid, block, 0, s, iters, out)
+  if (mode == 0) LCE_OVL(0, 16);
+  else if (per_mfma == 1) { if (mode == 1) LCE_OVL(1, 16); else LCE_OVL(2, 16); }
+  else if (per_mfma == 2) { if (mode == 1) LCE_OVL(1, 32); else LCE_OVL(2, 32); }
+  else if (per_mfma == 4) { if (mode == 1) LCE_OVL(1, 64); else LCE_OVL(2, 64); }
+  else return -3;
+#undef LCE_OVL
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 

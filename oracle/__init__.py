@@ -10,4 +10,5 @@ from .lce_oracle import (  # noqa: F401
     lce_forward_backward_fp64,
     lce_bruteforce,
     eager_fp32_step,
+    eager_fp32_step_chunked,
 )

@@ -21,6 +21,9 @@ checkout):
   evaluated in row chunks).
 * ``eager_fp32_step``       -- ``bench_fusions.py:30-33`` (the eager torch
   provider used as the baseline).
+* ``eager_fp32_step_chunked`` -- the same step as an N-chunked eager loop
+  (``bench_fusions.py:71-83`` without the checkpointing), for workloads whose
+  N x V fp32 logits do not fit the host.
 
 Pinning status: every function here is pinned by ``tests/test_oracle.py``
 against library routines (``F.cross_entropy`` + autograd in fp64), central
@@ -165,3 +168,31 @@ def eager_fp32_step(x, y, w, ignore_index=-100, z_regularization=0.0, logit_scal
         loss = loss + z_regularization * torch.logsumexp(z, -1)[y1 != ignore_index].pow(2).mean()
     loss.backward()
     return loss.detach(), x32.grad, w32.grad
+
+
+def eager_fp32_step_chunked(x, y, w, ignore_index=-100, z_regularization=0.0, logit_scale=1.0, chunk=2048):
+    """The same step over all tokens, `chunk` rows at a time, so that only chunk x V logits exist at once:
+    the mathematically identical N-chunked eager loop (the pattern of bench_fusions.py:71-83, without the
+    checkpointing).  Every chunk's loss terms are summed and divided by the number of valid labels of the whole
+    batch, its backward adds into the same dW, and its rows of dx are its own.  Returns (loss, dx, dw) in fp32.
+    """
+    import torch.nn.functional as F
+
+    x2 = x.reshape(-1, x.shape[-1])
+    y1 = y.reshape(-1)
+    R = (y1 != ignore_index).sum()
+    w32 = w.float().detach().requires_grad_(True)
+    dx = torch.empty(x2.shape, dtype=torch.float32)
+    loss = torch.zeros((), dtype=torch.float32)
+    for r0 in range(0, x2.shape[0], chunk):
+        xc = x2[r0:r0 + chunk].float().detach().requires_grad_(True)
+        yc = y1[r0:r0 + chunk]
+        z = (xc @ w32) * logit_scale
+        part = F.cross_entropy(z, yc, ignore_index=ignore_index, reduction="sum")
+        if z_regularization > 0:
+            part = part + z_regularization * torch.logsumexp(z, -1)[yc != ignore_index].pow(2).sum()
+        part = part / R
+        part.backward()
+        dx[r0:r0 + chunk] = xc.grad
+        loss += part.detach()
+    return loss, dx, w32.grad

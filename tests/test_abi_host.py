@@ -434,3 +434,25 @@ def test_vocabulary_major_weight_layout_is_checked_and_detected():
     assert ops._weight_layout(torch.zeros(1000, 100, dtype=torch.bfloat16).t(), torch.bfloat16) == _lib.W_HV  # H % 8
     assert ops._weight_layout(torch.zeros(1000, 264, dtype=torch.bfloat16)[:, :256].t(), torch.bfloat16) == _lib.W_VH
     assert ops._weight_layout(torch.zeros(1000, 256, dtype=torch.float32).t(), torch.float16) == _lib.W_VH  # master weight
+
+
+def test_a_weight_that_cannot_be_read_in_place_is_copied_with_one_warning():
+    """A weight the kernels cannot read in place (here: (V, H) storage with H % 8 != 0, handed over transposed) is
+    copied on every call; the host says so once, naming shape, strides and size, and stays silent afterwards.
+    A weight that is read in place raises nothing."""
+    import warnings
+
+    from linear_cross_entropy_loss_amd import ops
+
+    ops._copy_warned.clear()
+    good = torch.zeros(64, 1000, dtype=torch.bfloat16)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        assert ops._weight_rows(good, ops._weight_layout(good, torch.bfloat16)) is good
+    bad = torch.zeros(1000, 100, dtype=torch.bfloat16).t()  # (H, V) = (100, 1000) view of a (V, H) matrix
+    with pytest.warns(UserWarning, match=r"weight of shape \(100, 1000\).*copied on every call"):
+        w = ops._weight_rows(bad, ops._weight_layout(bad, torch.bfloat16))
+    assert w.stride(1) == 1 and w.stride(0) % 8 == 0 and torch.equal(w, bad)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        ops._weight_rows(bad, ops._weight_layout(bad, torch.bfloat16))  # the second copy is silent

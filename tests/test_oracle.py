@@ -189,3 +189,24 @@ def test_eager_fp32_step_is_the_same_function_in_single_precision(zreg, scale, i
         loss0, dx0, _ = eager_fp32_step(x, y, w, ignore_index, 0.0, scale)
         assert abs(loss0.item() - loss.item()) > 1e-3 * abs(loss.item())
         assert (dx0 - dx).abs().max() > 1e-3 * dx.abs().max()
+
+
+@pytest.mark.parametrize("zreg,scale,ignore_index,chunk", [(0.0, 1.0, -1, 16), (1e-2, 0.5, -1, 7), (0.3, 2.0, 5, 48), (0.0, 1.0, -1, 1000)])
+def test_chunked_eager_fp32_step_equals_the_unchunked_one(zreg, scale, ignore_index, chunk):
+    """The N-chunked form of the CPU baseline (what bench.py times on the whole workload): same loss and gradients
+    as the unchunked step up to fp32 summation order and as the fp64 closed forms, for chunk sizes that divide the
+    token count, that do not, and that exceed it; a chunk whose labels are all ignored contributes exact zeros."""
+    from oracle import eager_fp32_step, eager_fp32_step_chunked
+
+    x, y, w = _rand(48, 24, 40, seed=23, ignore_frac=0.3, ignore_index=ignore_index)
+    y[:7] = ignore_index  # the first chunk of 7 holds no valid label
+    ref = lce_forward_backward_fp64(x, y, w, ignore_index, zreg, scale)
+    loss1, dx1, dw1 = eager_fp32_step(x, y, w, ignore_index, zreg, scale)
+    loss, dx, dw = eager_fp32_step_chunked(x, y, w, ignore_index, zreg, scale, chunk=chunk)
+    assert loss.dtype == torch.float32 and dx.dtype == torch.float32 and dw.dtype == torch.float32
+    assert abs(loss.item() - loss1.item()) <= 1e-5 * abs(loss1.item())
+    assert abs(loss.item() - ref.loss.item()) <= 1e-5 * abs(ref.loss.item())
+    for got, one, want in ((dx, dx1, ref.dx), (dw, dw1, ref.dw)):
+        assert torch.allclose(got, one, rtol=1e-4, atol=1e-6 * one.abs().max().item())
+        assert torch.allclose(got.double(), want, rtol=1e-4, atol=1e-6 * want.abs().max().item())
+    assert (dx[y == ignore_index] == 0).all()

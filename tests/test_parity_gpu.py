@@ -356,6 +356,8 @@ def test_many_tokens_go_through_the_forward_in_chunks(mon):
     keep = y != -1
     assert nv.item() == int(keep.sum().item())
     assert torch.allclose(lse[keep].double(), ref.lse[keep], rtol=2e-4, atol=2e-4)
+    # a token with an ignored label has lse == 0, whether its row was computed (rows not packed) or not
+    assert (lse[~keep].view(torch.int32) == 0).all()
     assert torch.equal(out5[0], out[0])
 
 
@@ -370,6 +372,23 @@ def test_fp16_with_a_large_z_regularisation(z_reg):
     ref = _oracle(x, y, w, -1, z_reg, 1.0, grad_output=64.0)
     assert torch.isfinite(dx).all() and torch.isfinite(dw).all()
     assert ref.lse.abs().max().item() > 8
+    assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item())
+    for got, want in ((dx, ref.dx), (dw, ref.dw)):
+        emax, el2 = rel_errors(got, want)
+        assert emax <= GRAD_TOL and el2 <= GRAD_TOL, (emax, el2)
+
+
+def test_fp16_z_regularisation_with_lse_near_a_thousand_stays_finite():
+    """fp16 stages dz times 2^10 with the factor 1 + 2 * z_reg * lse on top: at z_reg = 0.03 and logits around 1e3
+    that factor is about 60, the staged values reach 6e4 -- inside fp16's range (the kernel clamps the factor to
+    63, which lse < 1033 does not reach here), so the gradients stay finite and match the fp64 oracle."""
+    print("fp16 z_reg=0.03, lse near 1000", flush=True)
+    x, y, w = make_inputs(512, 256, 4096, torch.float16, seed=93, ignore_frac=0.1)
+    scale = 205.0
+    out, dx, dw = _run(x, y, w, -1, 0.03, scale, 512, False, grad_output=1.0 / 64)
+    ref = _oracle(x, y, w, -1, 0.03, scale, grad_output=1.0 / 64)
+    assert 800 < ref.lse.abs().max().item() < 1030
+    assert torch.isfinite(out[0]) and torch.isfinite(dx).all() and torch.isfinite(dw).all()
     assert abs(out[0].item() - ref.loss.item()) <= LOSS_RTOL * abs(ref.loss.item())
     for got, want in ((dx, ref.dx), (dw, ref.dw)):
         emax, el2 = rel_errors(got, want)
