@@ -15,7 +15,7 @@
  *     (H, V) row-major with row stride ldw (linear_cross_entropy/ops.py:913);
  *     y is N contiguous int64 labels (ops.py:210), each ignore_index or in
  *     [0, V); any other value makes the returned loss NaN.
- *   - Shapes: any N, H, V, n_chunk >= 1 (N <= 2^22 -- 2^20 for fp32
+ *   - Shapes: any N, H, V, n_chunk >= 1 (N <= 2^30 -- 2^20 for fp32
  *     activations --, V <= 2^30, H <= 2^20).  The
  *     reference's divisibility rules (N % 512, H % 256, V % 4096,
  *     ops.py:689-691, 905-907) are lifted; shapes that obey them run at full

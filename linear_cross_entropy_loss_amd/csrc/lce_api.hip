@@ -29,9 +29,9 @@ int check(const lce_problem* p, bool backward) {
   if (p->N <= 0 || p->H <= 0 || p->V <= 0 || p->n_chunk <= 0) return LCE_EINVAL_SHAPE;
   // Any N, H, V; only the row strides are constrained (below).
   if (p->N > (int64_t)1 << 30 || p->V > (int64_t)1 << 30 || p->H > (int64_t)1 << 20) return LCE_EINVAL_SHAPE;
-  // The dz stage is addressed in column groups of all token rows (BwdArgs::dz) through 32-bit byte offsets that
-  // span up to four groups: 4 * rows * 128 bytes must stay below 2^31 (three times the rows for bf16 pairs).
-  if (p->N > ((int64_t)1 << 22) / (p->x_dtype == LCE_F32 ? 4 : 1)) return LCE_EINVAL_SHAPE;
+  // bf16 pairs: bwd_dz reaches the three parts of its stage through 32-bit byte offsets (two parts of at least
+  // Np * 256 * 2 bytes each)
+  if (p->x_dtype == LCE_F32 && p->N > (int64_t)1 << 20) return LCE_EINVAL_SHAPE;
   const int xd = p->x_dtype, wd = p->w_dtype;
   const bool ok = (is16(xd) && (wd == xd || wd == LCE_F32)) || (xd == LCE_F32 && wd == LCE_F32);
   if (!ok) return LCE_EINVAL_DTYPE;
@@ -465,7 +465,7 @@ const char* lce_strerror(int status) {
   switch (status) {
     case LCE_OK: return "ok";
     case LCE_EINVAL_SHAPE:
-      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N <= 2^22 (2^20 for fp32 activations), "
+      return "shape outside the supported set (need N, H, V, N_chunk_size >= 1; N <= 2^30 (2^20 for fp32 activations), "
              "V <= 2^30, H <= 2^20; "
              "ceil(N/256) * ceil(V/256) <= 2^28)";
     case LCE_EINVAL_DTYPE:
@@ -603,7 +603,7 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     a.x_dtype = lce::DT_BF16;
   }
   const bool split = splits(p);
-  a.dz_rows = split ? 3 * a.Np : a.Np;  // rows per column group of the dz stage (BwdArgs::dz)
+  a.dz_rows = split ? 3 * a.Np : a.Np;  // rows of the dz stage (BwdArgs::dz)
 
   for (int64_t i = 0; i < b.slabs; ++i) {
     a.v0 = i * b.vs;
@@ -643,9 +643,9 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
       continue;
     }
     // fp32 tensors as bf16 pairs (lce_gemm.h): x = [hi | hi | lo] against W = [hi ; lo ; hi] along a K axis of
-    // 3 H for the logits; dz comes back as three blocks [hi ; lo ; hi] of Np rows in every column group.
+    // 3 H for the logits; dz comes back as three parts [hi ; lo ; hi] of Np rows.
     char* dz0 = (char*)a.dz;
-    const int64_t blk = a.Np * 64 * 2;  // bytes from the first row of a block to that of the next
+    const int64_t blk = a.Np * a.vs * 2;  // bytes from the first row of a part to that of the next
     if (ph & LCE_PHASE_BWD_DZ) {
       lce::BwdArgs z = a;
       z.H = 3 * p->H;

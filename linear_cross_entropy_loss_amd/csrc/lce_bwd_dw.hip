@@ -236,7 +236,7 @@ template <class T, bool WVH, int MODE> struct DwProblem {
   static constexpr bool kSwapAB = !WVH;  // (H, V) output: dz, the Q operand, feeds the A side (v along registers)
   static constexpr bool kVarK = true;    // whole tiles and segment items have different K extents
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
-  static constexpr bool kQGrouped = true;  // dz is staged in groups of 64 columns (BwdArgs::dz)
+  static constexpr bool kQBlocked = true;  // dz is staged in blocks of 256 rows x 64 columns (BwdArgs::dz)
   static constexpr bool kColumnEpilogue = false;
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
@@ -279,7 +279,13 @@ template <class T, bool WVH, int MODE> struct DwProblem {
     decode(local, item, tp, tq, seg);
     const int64_t k0 = seg < 0 ? 0 : (int64_t)seg * plan.kseg * kBK;  // first token of the segment
     p = x + k0 * ldx + (int64_t)tp * kTile;
-    q = reinterpret_cast<const E*>(a.dz) + ((int64_t)tq * (kTile / kBK) * a.dz_rows + k0) * kBK;
+    q = reinterpret_cast<const E*>(a.dz) + dz_block_offset(k0 / kTile, (int64_t)tq * (kTile / kBK), a.vs) + (k0 % kTile) * kBK;
+  }
+  // (segments start at even numbers of K tiles: in the first or the third quarter of a row of blocks)
+  LCE_DEV int q_phase(int local) const {
+    int item, tp, tq, seg;
+    decode(local, item, tp, tq, seg);
+    return seg < 0 ? 0 : (seg * plan.kseg) & 3;
   }
   // x rows past the last one read as zeros.  dz is written for whole token tiles of 256 rows, and the K tiles of
   // the plan end with the pair of K tiles that holds the last row (dw_plan), so none of them reaches past
@@ -308,7 +314,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdAr
   typedef typename elem_of<T>::type E;
   DwProblem<T, WVH, MODE> prob(a);
   Pipe3<T, E, false, E, false, DwProblem<T, WVH, MODE>> pipe(prob);
-  pipe.run(prob.ldx, a.dz_rows, prob.plan.kt, lds);
+  pipe.run(prob.ldx, a.vs / kBK, prob.plan.kt, lds);
 }
 
 // Second step for the tail tiles: kTailParts workgroups share tail tile b (16 of its rows each) -- they sum

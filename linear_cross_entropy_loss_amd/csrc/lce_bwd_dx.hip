@@ -159,7 +159,7 @@ template <class T, bool KMASK, bool WVH, int MODE> struct DxProblem {
   static constexpr bool kKMask = KMASK;
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = MODE == kDxTails;  // segment items have their own K extent
-  static constexpr bool kQGrouped = true;          // dz is staged in groups of 64 columns (BwdArgs::dz)
+  static constexpr bool kQBlocked = true;          // dz is staged in blocks of 256 rows x 64 columns (BwdArgs::dz)
   static constexpr bool kColumnEpilogue = false;
   typedef typename elem_of<T>::type E;
   const BwdArgs& a;
@@ -195,12 +195,14 @@ template <class T, bool KMASK, bool WVH, int MODE> struct DxProblem {
     const int64_t k0 = k0_of(seg);
     p = WVH ? reinterpret_cast<const E*>(a.w) + ((a.v0 - a.wv0) + k0) * a.ldw + (int64_t)tp * kTile
             : reinterpret_cast<const E*>(a.w) + (int64_t)tp * kTile * a.ldw + (a.v0 - a.wv0) + k0;
-    q = reinterpret_cast<const E*>(a.dz) + ((k0 / kBK) * a.dz_rows + (int64_t)tq * kTile) * kBK;  // (k0 is a multiple of 64)
+    q = reinterpret_cast<const E*>(a.dz) + dz_block_offset(tq, k0 / kBK, a.vs);  // (k0 is a multiple of 64)
   }
   LCE_DEV const void* p_end() const {
     return WVH ? matrix_end<E>(a.w, a.Vw, a.ldw, a.H) : matrix_end<E>(a.w, a.H, a.ldw, a.Vw);
   }
-  // (only whole token tiles that were written are read; K tiles past the slab lie past the last column group)
+  // (only whole token tiles that were written are read.  K tiles past the slab -- the last segment of a split tail
+  // tile may have some -- lie in the next row of blocks, or past the stage: the K mask gives those threads an
+  // out-of-range offset, the other operand's are zeros)
   LCE_DEV const void* q_end() const { return reinterpret_cast<const E*>(a.dz) + a.dz_rows * a.vs; }
   LCE_DEV int k_valid(int local) const {
     int item, tp, tq, seg;
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dx_persistent_kernel(const BwdAr
   typedef typename elem_of<T>::type E;
   DxProblem<T, KMASK, WVH, MODE> prob(a);
   Pipe3<T, E, !WVH, E, true, DxProblem<T, KMASK, WVH, MODE>> pipe(prob);
-  pipe.run(a.ldw, a.dz_rows, MODE == kDxTails ? prob.plan.kseg : (int)(a.vs / kBK), lds);
+  pipe.run(a.ldw, a.vs / kBK, MODE == kDxTails ? prob.plan.kseg : (int)(a.vs / kBK), lds);
 }
 
 // Second step for the tail tiles: kTailParts workgroups share tail tile b (16 rows each) -- they sum its

@@ -59,7 +59,7 @@ constexpr int kDzStoreAux = LCE_DZ_STORE_AUX;  // cache policy of the dz stores:
 // are written as exact zeros.
 //
 // SPLIT (fp32 tensors carried as bf16 pairs, lce_gemm.h): dz is staged as hi = bf16(dz) and lo = bf16(dz - hi)
-// in three blocks of Np rows per column group, [hi ; lo ; hi], each lane storing its 16-byte runs itself (this
+// in three parts of Np rows, [hi ; lo ; hi], each lane storing its 16-byte runs itself (this
 // path serves accuracy, not speed).
 // `pf_y`, `pf_lse`: label and lse of this lane's four tokens (DzProblem::prefetch), ignore_index / 0 for rows that do not exist.
 template <class T, bool ZREG, bool VTAIL, bool SPLIT>
@@ -78,17 +78,17 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
   const int vrem = VTAIL ? (int)(left < 0 ? 0 : (left > kWaveTile ? kWaveTile : left)) : kWaveTile;
   const int nq = vrem >> 3, cut = vrem & 7;
   const int cut_mine = cut - 4 * half;  // elements of this lane's quad of the cut run that exist (<= 0: none)
-  // This wave's 128 columns are two column groups (accumulator blocks 0, 1 and 2, 3); `row` = this lane's
-  // token row of block qb = 0 in the first of them.
-  const int64_t grp = a.dz_rows * kGroup;  // elements per column group
+  // This wave's 128 columns are two column groups (accumulator blocks 0, 1 and 2, 3), neighbouring blocks of the
+  // stage; `row` = this lane's token row of block qb = 0 in the first of them.
+  constexpr int64_t grp = kDzBlockElems;  // elements from a block of the stage to the next column group's
   const int wpu = __builtin_amdgcn_readfirstlane(wp), wqu = __builtin_amdgcn_readfirstlane(wq);  // (uniform, for the scalar unit)
-  E* wave_base = reinterpret_cast<E*>(a.dz) + (int64_t)(tp * (kTile / kGroup) + wpu * (kWaveTile / kGroup)) * grp +
-                 (t0 + wqu * kWaveTile) * kGroup;
+  E* wave_base = reinterpret_cast<E*>(a.dz) + dz_block_offset(tq, tp * (kTile / kGroup) + wpu * (kWaveTile / kGroup), a.vs) +
+                 wqu * kWaveTile * kGroup;
   E* row = wave_base + (lane & 31) * kGroup;
-  const int64_t blk = a.Np * kGroup;  // SPLIT: elements between the three blocks of a column group
+  const int64_t blk = a.Np * a.vs;  // SPLIT: elements between the three parts of the stage
   // Stores go through a buffer descriptor over this wave's part of the stage (scalar base, one 32-bit offset per
   // lane, the block's offset as a scalar): no 64-bit vector address arithmetic.  All offsets stay below 2^31
-  // (dz_rows * 128 bytes for the second column group, plus two blocks of a bf16-pair stage).
+  // (one block for the second column group, plus two parts of a bf16-pair stage).
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(wave_base, 0, 0x7fffffff, 0x00020000);
   const unsigned lane_off = (unsigned)((lane & 31) * (kGroup * 2) + half * 16);
   // staging: this lane's line of a piece when it writes (its token), and line / chunk when it reads back: 8 lines
@@ -231,7 +231,7 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> stru
   static constexpr bool kKMask = KMASK;
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
-  static constexpr bool kQGrouped = false;
+  static constexpr bool kQBlocked = false;
   static constexpr bool kColumnEpilogue = false;
   const BwdArgs& a;
   int64_t rows, ldx;  // token rows: all of x, or the packed rows (see BwdArgs)

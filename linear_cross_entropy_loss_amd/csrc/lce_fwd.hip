@@ -284,7 +284,7 @@ template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON> struct FwdProblem
   static constexpr bool kKMask = KMASK;
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
-  static constexpr bool kQGrouped = false;
+  static constexpr bool kQBlocked = false;
   static constexpr bool kColumnEpilogue = !VTAIL && !MON;
   const FwdArgs& a;
   int64_t rows, ldx;

@@ -86,18 +86,18 @@ template <class T, class SrcT, bool KC, bool KMASK> struct Stager3 {
     base = end = nullptr;
     range = 0;
   }
-  // The operand is stored in groups of 64 columns, [cols / 64][rows][64] with `rows` rows per group (the
-  // staged dz, see lce_bwd_dz.hip), instead of row-major.  KC (its columns are the K index): the 256 rows x
-  // 64 k of a K tile are one contiguous block of 128-byte rows, and the next K tile is the next group.
-  // Otherwise (its rows are the K index): the tile's 256 columns are four groups, each thread stays in one.
-  // The byte offsets of a tile's chunks (up to 3 groups + 64 rows) must fit 31 bits: rows < 5.5 million.
-  LCE_DEV void init_grouped(int64_t rows) {
+  // The operand is stored in blocks of 256 rows x 64 columns, [rows / 256][cols / 64][256][64] (the staged dz, see
+  // BwdArgs::dz), instead of row-major.  KC (its columns are the K index): the 256 rows x 64 k of a K tile are one
+  // contiguous block of 128-byte rows, and the next K tile is the next block.  Otherwise (its rows are the K
+  // index): the tile's 256 columns are four consecutive blocks, each thread stays in one; a K tile is 64 rows of
+  // them, and after four K tiles the stream moves on to the next row of blocks (Pipe3::stream_advance).
+  LCE_DEV void init_blocked() {
     init(kBK);
     if (KC) {
-      k_stride = rows * (kBK * kEs);
+      k_stride = kTile * (kBK * kEs);
     } else {
       const int t = threadIdx.x, c = t & 31, k = t >> 5;
-      voff = (unsigned)(((int64_t)(c >> 3) * rows + k) * (kBK * kEs) + (c & 7) * 16);
+      voff = (unsigned)((c >> 3) * (kTile * kBK * kEs) + k * (kBK * kEs) + (c & 7) * 16);
       voff_cur = voff;
       iter_stride = (unsigned)(8 * kBK * kEs);
       k_stride = (int64_t)kBK * kBK * kEs;
@@ -159,8 +159,10 @@ template <class S> LCE_DEV const void* matrix_end(const void* base, int64_t rows
 //        of P block i and Q block j, with Q along its registers and P along its lanes)
 //   void prefetch(int tile)                       called three K tiles before the tile's epilogue: the place to issue loads
 //        of per-row data the epilogue starts with (kept in members), so that their latency is not exposed there
-//   static constexpr bool kQGrouped               true if the Q operand is stored in groups of 64 columns (Stager3::init_grouped);
-//        run() then takes the rows per group in place of the Q row stride
+//   static constexpr bool kQBlocked               true if the Q operand is stored in blocks of 256 rows x 64 columns
+//        (Stager3::init_blocked); run() then takes the column groups per row of blocks in place of the Q row stride, and
+//   int  q_phase(int tile)                        (rows are the K index) says which of the four K tiles of a row of blocks
+//        the tile's first K tile is
 //   static constexpr bool kKMask                  false if `ktiles * 64 == k_valid` for every tile of the launch
 //   int  k_valid(int tile)                        K extent of that tile's contraction; the K tiles of the
 //        loop may run past it (`ktiles * 64 >= k_valid`), the excess contributes exact zeros
@@ -194,6 +196,9 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
   int ktiles;
   int load_tile;  // output tile the fetch stream is in
   int k_rem;      // valid k elements left from the K tile the stream points at
+  int q_phase;    // blocked Q operand with rows as its K index: K tile of the current row of blocks, 0..3
+  int64_t q_jump; // and the bytes from the last K tile of a row of blocks to the first of the next
+  static constexpr bool kQRowBlocks = Problem::kQBlocked && !Q_KC;
 
   static constexpr int kPReads = P_KC ? 4 : 8;  // LDS read instructions per k-step
   static constexpr int kQReads = Q_KC ? 4 : 8;
@@ -223,12 +228,18 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
       qs.end = qs.base;
     }
     k_rem = prob.k_valid(tile);
+    if constexpr (kQRowBlocks) q_phase = tile < prob.num_tiles() ? prob.q_phase(tile) : 0;
     ps.retarget(k_rem);
     qs.retarget(k_rem);
   }
   LCE_DEV void stream_advance() {
     ps.base += ps.k_stride;
-    qs.base += qs.k_stride;
+    if constexpr (kQRowBlocks) {
+      qs.base += q_phase == 3 ? q_jump : qs.k_stride;
+      q_phase = (q_phase + 1) & 3;
+    } else {
+      qs.base += qs.k_stride;
+    }
     k_rem -= kBK;
     ps.retarget(k_rem);
     qs.retarget(k_rem);
@@ -422,7 +433,14 @@ template <class T, class PSrc, bool P_KC, class QSrc, bool Q_KC, class Problem> 
     ktiles = ktiles_;
     const int wave = threadIdx.x >> 6;
     ps.init(ldp);
-    if constexpr (Problem::kQGrouped) qs.init_grouped(ldq); else qs.init(ldq);
+    if constexpr (Problem::kQBlocked) {
+      qs.init_blocked();
+      // (ldq: column groups per row of blocks) what takes a stream whose K index is the rows from the last K tile of
+      // a row of blocks to the first of the next
+      q_jump = ldq * (kTile * kBK * QStager::kEs) - 3 * qs.k_stride;
+    } else {
+      qs.init(ldq);
+    }
     pr.init((wave & 1) * kWaveTile);
     qr.init((wave >> 1) * kWaveTile);
 

@@ -88,10 +88,11 @@ struct BwdArgs {
   // w_vh != 0: weight and dW are stored with the vocabulary as their row index, w[v * ldw + h], dw[v * lddw + h]
   // (and the buffer `w` holds ROWS [wv0, wv0 + Vw)); otherwise w[h * ldw + v], dw[h * lddw + v].
   int w_vh;
-  // Staged dz in the compute type (exact zeros outside N x vw), stored in groups of 64 columns:
-  // element (row, v) of the slab sits at dz[((v / 64) * dz_rows + row) * 64 + v % 64], so that the 64-deep K tiles
-  // of the dx contraction (K = v) are contiguous blocks of 128-byte rows, and a token's 64 columns of a group are
-  // one 128-byte line.  dz_rows = Np, or 3 Np when dz is carried as bf16 pairs (`split` below).
+  // Staged dz in the compute type (exact zeros outside N x vw), stored in blocks of 256 rows x 64 columns,
+  // [rows / 256][vs / 64][256][64] (dz_block_offset below): the 64-deep K tiles of the dx contraction (K = v) are
+  // consecutive 32 KiB blocks, the K tiles of the dW contraction (K = tokens) quarters of four neighbouring blocks,
+  // and a token's 64 columns of a group are one 128-byte line.  dz_rows = Np rows, or 3 Np when dz is carried as
+  // bf16 pairs (`split` below).
   void* dz;
   int64_t dz_rows;
   float* dx_acc;    // [Np][Hp] fp32 running dx (null when there is a single slab)
@@ -114,9 +115,9 @@ struct BwdArgs {
   int first, last;  // slab position
   int num_cus;      // compute units of the device: grid size of the persistent kernels
   int live;         // bwd_dz: bands of W that the XCDs keep in flight together (lce_gemm.h, tile_coords)
-  // fp32 tensors carried as bf16 pairs (lce_gemm.h): every column group of the stage holds three blocks of Np
-  // rows, [hi ; lo ; hi]; only bwd_dz looks at this flag (the dx and dW launches get plain 16-bit problems over
-  // these blocks: dx with `dz` pointing at the first row of a block, dW with 3 Np token rows).
+  // fp32 tensors carried as bf16 pairs (lce_gemm.h): the stage holds three parts of Np rows each, [hi ; lo ; hi];
+  // only bwd_dz looks at this flag (the dx and dW launches get plain 16-bit problems over these parts: dx with `dz`
+  // pointing at the first row of a part, dW with 3 Np token rows).
   int split;
   // Packed rows (tokens with an ignored label dropped; n_rows == null: the call works on all rows).
   // *n_rows (device) rows are worked on.  When *n_rows != N they are the rows of xc (row stride ldxc) and
@@ -130,6 +131,12 @@ struct BwdArgs {
   void* dxc;
   int64_t lddxc;
 };
+
+// Element offset of block (row tile, column group) of a dz stage that is `vs` columns wide.
+constexpr int kDzBlockElems = 256 * 64;
+__host__ __device__ inline int64_t dz_block_offset(int64_t row_tile, int64_t group, int64_t vs) {
+  return (row_tile * (vs / 64) + group) * kDzBlockElems;
+}
 
 // Factor applied to dx and dW after their fp32 accumulation: grad_out * logit_scale / n_valid
 // (linear_cross_entropy/ops.py:332, 443-447, 810), times the power of two that undoes the scaling of the staged
