@@ -280,8 +280,8 @@ __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
 
 template <class T, bool KMASK, bool WVH, int MODE> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
   auto kern = bwd_dx_persistent_kernel<T, KMASK, WVH, MODE>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
+  static LdsOptIn optin;
+  hipError_t e = optin.ensure(reinterpret_cast<const void*>(kern), kMainloopLds);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(a.dx_grid), dim3(kThreads), kMainloopLds, s, a);
   return hipGetLastError();

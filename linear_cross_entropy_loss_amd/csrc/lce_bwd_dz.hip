@@ -300,8 +300,8 @@ __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdAr
 template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH>
 hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
   auto kern = bwd_dz_persistent_kernel<T, ZREG, VTAIL, KMASK, SPLIT, WVH>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  static LdsOptIn optin;
+  hipError_t e = optin.ensure(reinterpret_cast<const void*>(kern), kLdsBytes);
   if (e != hipSuccess) return e;
   const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kLdsBytes, s, a);

@@ -153,18 +153,6 @@ LCE_DEV void fwd_epilogue(const FwdArgs& a, int64_t rows, f32x16_t (&acc)[kNB][k
 }
 
 
-// The same reduction for the kernels whose last K tile is multiplied column by column (Pipe3::step_last_columns;
-// full tiles, no monitoring): one block column of the accumulator at a time -- 32 tokens along the lanes, this
-// wave's 128 vocabulary entries of each token in 4 x 16 registers of lanes l and l + 32 -- cut into 16 slots of
-// straight-line code that run behind the matrix instructions of the next column.  A lane folds its 64 values
-// in two chunks of 32 (slots 8c .. 8c + 7 of chunk c) into a running (max, sum of exp2) pair, so that only 32
-// accumulator values are in vector registers at a time, and meets the other half of the slice in lane ^ 32.
-struct FwdColumnState {
-  float v[32];   // the chunk being summed
-  float m, s;    // running max (unscaled logits) and sum of exp2(scaled logit - scaled max)
-  float mo;      // scaled max of the chunk being summed
-  float e[4], f; // exponentials of the last slot, not yet added; factor for the sum at a chunk change
-};
 // The logit of the target column, written by the one lane that holds it (rare: a wave holds the target of
 // one token in a thousand at a vocabulary of 131072).  `yl`: the column inside this wave's 128-wide slice if
 // this lane's half holds it, else -1.
@@ -185,11 +173,38 @@ LCE_DEV void fwd_store_target(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int64
   }
 }
 
-// Slot 0..15 of block column QB: the running (max, sum) of this lane's 64 values.
-template <int QB>
+// The same reduction for the kernels whose last K tile is multiplied column by column (Pipe3::step_last_columns:
+// all but the tile column that straddles V): one block column of the accumulator at a time -- 32 tokens along the lanes, this
+// wave's 128 vocabulary entries of each token in 4 x 16 registers of lanes l and l + 32 -- cut into 16 slots of
+// straight-line code that run behind the matrix instructions of the next column.  A lane folds its 64 values
+// in two chunks of 32 (slots 8c .. 8c + 7 of chunk c) into a running (max, sum of exp2) pair, so that only 32
+// accumulator values are in vector registers at a time, and meets the other half of the slice in lane ^ 32.
+struct FwdColumnState {
+  float v[32];   // the chunk being summed
+  float m, s;    // running max (unscaled logits) and sum of exp2(scaled logit - scaled max)
+  float mo;      // scaled max of the chunk being summed
+  float e[4], f; // exponentials of the last slot, not yet added; factor for the sum at a chunk change
+  float pz, sq;  // monitoring: sum exp2(..) * scaled logit (moves with the max like s) and sum of squared scaled logits
+};
+// Slot 0..15 of block column QB: the running (max, sum) of this lane's 64 values -- and, MON, the two monitoring
+// sums, which leave the arithmetic on (max, sum) as it is, so that the loss does not depend on the monitoring flag
+// bit for bit.  The exponentials of a slot are added up in the next one, when they are there.
+template <int QB, bool MON>
 LCE_DEV void fwd_slot_sum(const FwdArgs& a, FwdColumnState& st, f32x16_t (&acc)[kNB][kNB], int slot) {
   const float c1 = a.scale * kLog2e;
   const int c = slot >> 3, sub = slot & 7;  // chunk c: accumulator blocks 2c, 2c + 1, slots 8c .. 8c + 7
+  if (slot > 0) {
+    st.s += (st.e[0] + st.e[1]) + (st.e[2] + st.e[3]);
+    if (MON) {
+      const int prev = 4 * ((slot - 1) & 7);  // (the chunk of the previous slot is still in st.v)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float z = st.v[prev + r] * a.scale;
+        st.pz = fmaf(st.e[r], z, st.pz);
+        st.sq = fmaf(z, z, st.sq);
+      }
+    }
+  }
   if (sub == 0) {
 #pragma unroll
     for (int r = 0; r < 32; ++r) st.v[r] = acc[2 * c + (r >> 4)][QB][r & 15];
@@ -198,17 +213,33 @@ LCE_DEV void fwd_slot_sum(const FwdArgs& a, FwdColumnState& st, f32x16_t (&acc)[
     for (int r = 1; r < 32; ++r) cm = fmaxf(cm, st.v[r]);
     const float mn = c == 0 ? cm : fmaxf(st.m, cm);
     st.mo = mn * c1;  // logit_scale > 0, so max commutes with the scaling
-    if (c == 0) st.s = 0.f; else st.f = fast_exp2(fmaf(st.m, c1, -st.mo));  // factor that moves the sum to the new max
+    if (c == 0) {
+      st.s = 0.f;
+      if (MON) st.pz = st.sq = 0.f;
+    } else {
+      st.f = fast_exp2(fmaf(st.m, c1, -st.mo));  // moves the sums to the new max
+      st.s *= st.f;
+      if (MON) st.pz *= st.f;
+    }
     st.m = mn;
   }
-  // (the exponentials of a slot are added up in the next one, when they are there)
-  if (slot > 0) st.s += (st.e[0] + st.e[1]) + (st.e[2] + st.e[3]);
-  if (sub == 0 && c > 0) st.s *= st.f;
 #pragma unroll
   for (int r = 0; r < 4; ++r) st.e[r] = fast_exp2(fmaf(st.v[4 * sub + r], c1, -st.mo));
-  if (slot == 15) st.s += (st.e[0] + st.e[1]) + (st.e[2] + st.e[3]);
+  if (slot == 15) {
+    st.s += (st.e[0] + st.e[1]) + (st.e[2] + st.e[3]);
+    if (MON) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float z = st.v[28 + r] * a.scale;
+        st.pz = fmaf(st.e[r], z, st.pz);
+        st.sq = fmaf(z, z, st.sq);
+      }
+    }
+  }
 }
-// After slot 15: the other half of the slice.  Leaves the slice's max (unscaled) in st.m and its sum of exp2 in st.s.
+// After slot 15: the other half of the slice.  Leaves the slice's max (unscaled) in st.m, its sum of exp2 in st.s
+// and, MON, the slice's monitoring sums in st.pz, st.sq.
+template <bool MON>
 LCE_DEV void fwd_merge_halves(const FwdArgs& a, FwdColumnState& st) {
   const float c1 = a.scale * kLog2e;
   // after the swaps both lanes of a pair hold the lower lane's value in [0] and the upper lane's in [1]
@@ -220,57 +251,40 @@ LCE_DEV void fwd_merge_halves(const FwdArgs& a, FwdColumnState& st) {
   const float m0 = __builtin_bit_cast(float, m0u), m1 = __builtin_bit_cast(float, m1u);
   const float s0 = __builtin_bit_cast(float, s0u), s1 = __builtin_bit_cast(float, s1u);
   const float mt = fmaxf(m0, m1), mo = mt * c1;
-  st.s = s0 * fast_exp2(fmaf(m0, c1, -mo)) + s1 * fast_exp2(fmaf(m1, c1, -mo));
+  const float f0 = fast_exp2(fmaf(m0, c1, -mo)), f1 = fast_exp2(fmaf(m1, c1, -mo));
+  st.s = s0 * f0 + s1 * f1;
   st.m = mt;
+  if (MON) {
+    const unsigned pb = __builtin_bit_cast(unsigned, st.pz), qb = __builtin_bit_cast(unsigned, st.sq);
+    const auto pp = __builtin_amdgcn_permlane32_swap(pb, pb, false, false);
+    const auto qq = __builtin_amdgcn_permlane32_swap(qb, qb, false, false);
+    const unsigned p0u = pp[0], p1u = pp[1], q0u = qq[0], q1u = qq[1];
+    st.pz = __builtin_bit_cast(float, p0u) * f0 + __builtin_bit_cast(float, p1u) * f1;
+    st.sq = __builtin_bit_cast(float, q0u) + __builtin_bit_cast(float, q1u);
+  }
 }
-template <class T, int QB>
+template <class T, int QB, bool MON>
 LCE_DEV void fwd_epilogue_slot(const FwdArgs& a, FwdColumnState& st, f32x16_t (&acc)[kNB][kNB], int tp, int tq, int slot) {
-  fwd_slot_sum<QB>(a, st, acc, slot);
+  fwd_slot_sum<QB, MON>(a, st, acc, slot);
   if (slot == 15) {
-    fwd_merge_halves(a, st);
-    const float lse = fmaf(st.m, a.scale, fast_log(st.s));
-    // one store per token: the upper lanes get an offset that the range check of the buffer store drops
+    fwd_merge_halves<MON>(a, st);
+    // one store per token and partial: the upper lanes get an offset that the range check of the buffer store drops
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t slice = ((int64_t)tp * kTile + (wave & 1) * kWaveTile) / kChunkV;
-    float* base = a.part_lse + slice * a.nc + (int64_t)tq * kTile + (wave >> 1) * kWaveTile + QB * kBlk;
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(base, 0, kBlk * 4, 0x00020000);
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, lse), rsrc, lane < 32 ? lane * 4 : (int)0x80000000, 0, 0);
-  }
-}
-
-// Full tiles with monitoring: the same (max, sum) arithmetic, so that the loss does not depend on the monitoring
-// flag bit for bit, then the slice's sum softmax*z and sum z^2 in a second pass over the column.
-template <class T, int QB>
-LCE_DEV void fwd_epilogue_column_mon(const FwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq, int64_t tok, int yl) {
-  FwdColumnState st;
-#pragma unroll
-  for (int slot = 0; slot < 16; ++slot) fwd_slot_sum<QB>(a, st, acc, slot);
-  fwd_merge_halves(a, st);
-  const float c1 = a.scale * kLog2e, mo = st.m * c1;
-  float pz = 0.f, sq = 0.f;
-#pragma unroll
-  for (int pb = 0; pb < kNB; ++pb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float e = fast_exp2(fmaf(acc[pb][QB][r], c1, -mo));
-      const float z = acc[pb][QB][r] * a.scale;
-      pz = fmaf(e, z, pz);
-      sq = fmaf(z, z, sq);
+    const int64_t o = slice * a.nc + (int64_t)tq * kTile + (wave >> 1) * kWaveTile + QB * kBlk;
+    const int voff = lane < 32 ? lane * 4 : (int)0x80000000;
+    auto store = [&](float* base, float v) {
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(base + o, 0, kBlk * 4, 0x00020000);
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rsrc, voff, 0, 0);
+    };
+    store(a.part_lse, fmaf(st.m, a.scale, fast_log(st.s)));
+    if (MON) {
+      store(a.part_max, st.m * a.scale);
+      store(a.part_pz, st.pz / st.s);
+      store(a.part_sq, st.sq);
     }
-  pz += __shfl_xor(pz, 32);
-  sq += __shfl_xor(sq, 32);
-  const int tid = opaque_tid();
-  const int lane = tid & 63, wave = tid >> 6;
-  const int64_t slice = ((int64_t)tp * kTile + (wave & 1) * kWaveTile) / kChunkV;
-  const int64_t o = slice * a.nc + (int64_t)tq * kTile + (wave >> 1) * kWaveTile + QB * kBlk + (lane & 31);
-  if (lane < 32) {
-    a.part_lse[o] = fmaf(st.m, a.scale, fast_log(st.s));
-    a.part_max[o] = st.m * a.scale;
-    a.part_pz[o] = pz / st.s;
-    a.part_sq[o] = sq;
   }
-  fwd_store_target(a, acc, tok, QB, yl);
 }
 
 // Persistent workgroups, operand stream pipelined across output tiles.  The
@@ -285,7 +299,7 @@ template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON> struct FwdProblem
   static constexpr bool kSwapAB = false;
   static constexpr bool kVarK = false;
   static constexpr bool kQBlocked = false;
-  static constexpr bool kColumnEpilogue = !VTAIL && !MON;
+  static constexpr bool kColumnEpilogue = !VTAIL;
   const FwdArgs& a;
   int64_t rows, ldx;
   const E* x;
@@ -339,7 +353,7 @@ template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON> struct FwdProblem
   }
   FwdColumnState est;
   template <int J> LCE_DEV void epilogue_slot(int, f32x16_t (&acc)[kNB][kNB], int slot, char*) {
-    fwd_epilogue_slot<T, J>(a, est, acc, etp, etq, slot);
+    fwd_epilogue_slot<T, J, MON>(a, est, acc, etp, etq, slot);
   }
   LCE_DEV void epilogue_end(int, f32x16_t (&acc)[kNB][kNB], char*) const {
     const int tid = opaque_tid();
@@ -353,27 +367,10 @@ template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON> struct FwdProblem
       fwd_store_target(a, acc, tok, qb, here ? (int)rel : -1);
     }
   }
-  template <int QB> LCE_DEV void column_mon(f32x16_t (&acc)[kNB][kNB], int tp, int tq) const {
-    const int tid = opaque_tid();
-    const int lane = tid & 63, wave = tid >> 6;
-    const int64_t slice_v0 = (int64_t)tp * kTile + (wave & 1) * kWaveTile;
-    const int64_t tok = a.row0 + (int64_t)tq * kTile + (wave >> 1) * kWaveTile + QB * kBlk + (lane & 31);
-    const int64_t yy = tok < rows ? a.y[tok] : a.ignore_index, rel = yy - slice_v0;
-    const bool here = yy != a.ignore_index && rel >= 0 && rel < kWaveTile && ((rel >> 2) & 1) == (lane >> 5);
-    fwd_epilogue_column_mon<T, QB>(a, acc, tp, tq, tok, here ? (int)rel : -1);
-  }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char*) const {
     int tp, tq;
     coords(tile, tp, tq);
-    tp += (int)(a.v0 / kTile);
-    if constexpr (VTAIL) {
-      fwd_epilogue<T, VTAIL, MON>(a, rows, acc, tp, tq);
-    } else {
-      column_mon<0>(acc, tp, tq);
-      column_mon<1>(acc, tp, tq);
-      column_mon<2>(acc, tp, tq);
-      column_mon<3>(acc, tp, tq);
-    }
+    fwd_epilogue<T, VTAIL, MON>(a, rows, acc, (int)(a.v0 / kTile) + tp, tq);
   }
 };
 
@@ -542,8 +539,8 @@ __global__ __launch_bounds__(256) void fwd_final_kernel(const FwdArgs a) {
 template <class T, bool VTAIL, bool KMASK, bool WVH, bool MON>
 hipError_t launch_one(const FwdArgs& a, int64_t tiles, hipStream_t s) {
   auto kern = fwd_tiles_persistent_kernel<T, VTAIL, KMASK, WVH, MON>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMainloopLds);
+  static LdsOptIn optin;
+  hipError_t e = optin.ensure(reinterpret_cast<const void*>(kern), kMainloopLds);
   if (e != hipSuccess) return e;
   const int grid = (int)(tiles < a.num_cus ? tiles : a.num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), kMainloopLds, s, a);

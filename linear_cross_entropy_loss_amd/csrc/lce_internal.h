@@ -5,9 +5,27 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace lce {
 
 enum { DT_BF16 = 0, DT_F16 = 1, DT_F32 = 2 };
+
+// The tile kernels use more dynamic LDS than a kernel gets by default and have to opt in
+// (hipFuncAttributeMaxDynamicSharedMemorySize): once per kernel and device, not before every launch.  One object
+// per kernel (a function-local static of its launcher); thread-safe.
+struct LdsOptIn {
+  std::atomic<uint64_t> done{0};  // bit d: set on device d (devices from 64 on are set every time)
+  hipError_t ensure(const void* kernel, int bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1)) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && dev >= 0 && dev < 64) done.fetch_or((uint64_t)1 << dev, std::memory_order_release);
+    return e;
+  }
+};
 
 // Columns of logits covered by one forward partial (one wave's slice of a tile).
 constexpr int kChunkV = 128;
