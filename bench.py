@@ -68,7 +68,59 @@ def make_gpu_inputs(cfg, torch):
     return x, y, w
 
 
-def time_phases(cfg, x, y, w, torch, reps=5):
+def time_phases_one_pass(cfg, x, y, w, prob, chunks, torch, reps):
+    """time_phases for lce_forward_backward's single pass over the logits (`w`: the rows the kernels read)."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    lib = _lib.load()
+    N, H, V = cfg["N"], cfg["H"], cfg["V"]
+    dev = x.device
+    ws = torch.empty(_lib.forward_backward_workspace_bytes(prob(0)), dtype=torch.uint8, device=dev)
+    lse = torch.empty(N, dtype=torch.float32, device=dev)
+    out5 = torch.empty(5, dtype=torch.float32, device=dev)
+    nv = torch.empty(1, dtype=torch.int64, device=dev)
+    g = torch.ones(1, dtype=torch.float32, device=dev)
+    dx = torch.empty_like(x)
+    dw = torch.empty_like(w)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def call(ph):
+        p = prob(ph)
+        rc = lib.lce_forward_backward(ctypes.byref(p), P(x), P(w), P(y), P(g), P(lse), P(out5), P(nv), P(dx), P(dw),
+                                      P(ws), ws.numel(), stream)
+        _lib.raise_for_status(rc, "lce_forward_backward")
+
+    call(0)
+    torch.cuda.synchronize()
+    rows = int(nv.item()) if 8.0 * N * H * V >= 2.0 ** 41 else N
+    out = {}
+    for name, ph, flops, nbytes in (
+        ("fwd_stage", _lib.PHASE_FWD_TILES, 2.0 * rows * H * V / chunks, 0.0),
+        # 2 bytes read and 2 written per logit: bound by memory traffic, not by matrix instructions
+        ("stage_scale", _lib.PHASE_BWD_DZ, 0.0, 4.0 * rows * V / chunks),
+        ("bwd_dx", _lib.PHASE_BWD_DX, 2.0 * rows * H * V / chunks, 0.0),
+        # (with more than one chunk: the tile kernel adding into the fp32 plane, and after the last chunk the pass that stores dW)
+        ("bwd_dw", _lib.PHASE_BWD_DW, 2.0 * rows * H * V / chunks, 0.0),
+        ("pack", _lib.PHASE_PACK, 0.0, 0.0),
+    ):
+        call(ph)
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            call(ph)
+        e.record()
+        torch.cuda.synchronize()
+        launches = 1 if name == "pack" else chunks
+        per_launch_ms = s.elapsed_time(e) / reps / launches
+        out[name] = dict(ms_per_launch=per_launch_ms, launches_per_step=launches, flops_per_launch=flops,
+                         tflops=flops / per_launch_ms / 1e9)
+        if nbytes:
+            out[name].update(bytes_per_launch=nbytes, gb_per_s=nbytes / per_launch_ms / 1e6)
+    return out
+
+
+def time_phases(cfg, x, y, w, torch, reps=5, one_pass=True):
     """Average duration (ms) of each heavy kernel, bracketed by events on the launch stream, through the C ABI."""
     from linear_cross_entropy_loss_amd import _lib
 
@@ -85,6 +137,9 @@ def time_phases(cfg, x, y, w, torch, reps=5):
                                  -1, cfg["scale"], cfg["z_reg"], cfg["n_chunk"], cfg["monitoring"], phases, 0, 0,
                                  _lib.W_VH if vh else _lib.W_HV)
 
+    chunks, _ = _lib.forward_backward_plan(prob(0))
+    if chunks > 0 and not cfg["monitoring"] and one_pass:
+        return time_phases_one_pass(cfg, x, y, w, prob, chunks, torch, reps)
     fwd_b, bwd_b = _lib.workspace_bytes(prob(0))
     # one workspace per call: a call restricted to one kernel relies on what the full call left in it
     ws_f = torch.empty(fwd_b, dtype=torch.uint8, device=dev)
@@ -311,6 +366,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_bf16_N16384_H2048_V131072", choices=sorted(WORKLOADS) + ["c4_sweep"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--two-pass", action="store_true",
+                    help="loss-only forward and a backward that recomputes the logit tiles (lce_forward, lce_backward: "
+                         "8*H*V FLOPs per token), instead of the default, gradients from the forward's one evaluation of "
+                         "the logits where the problem allows it (lce_forward_backward: 6*H*V)")
+    ap.add_argument("--library", metavar="SO",
+                    help="load this build of liblce_gfx950.so instead of the one in the package (to time two builds "
+                         "on the same box)")
     ap.add_argument("--probe", choices=["ceiling", "flush", "overlap"],
                     help="run a measurement probe instead of the benchmark and print its JSON (built on demand, "
                          "linear_cross_entropy_loss_amd/probes): 'ceiling' (register-only MFMA loop, vendor GEMM, half of "
@@ -330,8 +392,14 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs an AMD GPU (torch.cuda.is_available() is False)", file=sys.stderr)
         sys.exit(1)
-    from linear_cross_entropy_loss_amd import _lib, linear_cross_entropy
+    from linear_cross_entropy_loss_amd import _lib, linear_cross_entropy, ops
 
+    if args.two_pass:
+        ops.one_pass.set(False)
+    if args.library:
+        from pathlib import Path
+
+        _lib.LIB_PATH = Path(args.library).resolve()
     if not _lib.LIB_PATH.exists():  # normally built beforehand and shipped with the tree
         from linear_cross_entropy_loss_amd.build import build
 
@@ -386,13 +454,23 @@ def main():
     flops = (2.0 * (N if cfg["monitoring"] else rows) + 6.0 * rows) * H * V
     tflops = flops / ms / 1e9
     peak = PEAK_TFLOPS[cfg["dtype"]]
+    # which route the steps above took (ops.LinearXentImplementation.forward decides the same way)
+    route = "two_pass"
+    if not args.two_pass and not cfg["monitoring"] and cfg["dtype"] != "f32" and cfg.get("w_dtype", cfg["dtype"]) == cfg["dtype"]:
+        wr = w.detach().t() if cfg.get("w_vh") else w.detach()
+        pr = _lib.make_problem(N, H, V, x.stride(0), wr.stride(0), H, wr.stride(0), x.dtype, wr.dtype, x.dtype, wr.dtype, -1,
+                               cfg["scale"], cfg["z_reg"], cfg["n_chunk"], False, 0, 0, 0,
+                               _lib.W_VH if cfg.get("w_vh") else _lib.W_HV)
+        if _lib.forward_backward_plan(pr)[0] > 0:
+            route = "one_pass"
+    flops_executed = flops if route == "two_pass" else 6.0 * rows * H * V
 
     ms_median = median_step_ms(step, torch, reps=20, flush=False)
     ms_median_flushed = median_step_ms(step, torch, reps=20, flush=True)
     x.grad = None
     w.grad = None
 
-    phases = time_phases(cfg, x.detach(), y, w.detach(), torch)
+    phases = time_phases(cfg, x.detach(), y, w.detach(), torch, one_pass=route == "one_pass")
     dom = max(phases, key=lambda k: phases[k]["ms_per_launch"] * phases[k]["launches_per_step"])
     d = phases[dom]
     roofline = dict(bound="mfma", kernel=dom, achieved=d["tflops"], peak=peak, unit="TFLOP/s",
@@ -427,8 +505,13 @@ def main():
                          "304.4 ms = 115.6 TFLOP/s on the 8NHV convention",
         "dtype": cfg["dtype"],
         "data": "synthetic",
-        "flops_note": "value counts the FLOPs executed: tokens with an ignored label are dropped before the tile "
-                      "kernels, so 8*H*V is multiplied by the tokens computed, not by N",
+        "flops_note": "value is on the metric's convention, 8*H*V FLOPs per token (logits, logits again, dx, dW), times the "
+                      "tokens computed: tokens with an ignored label are dropped before the tile kernels.  On the "
+                      "one_pass route the logits are evaluated once and 6*H*V FLOPs per token are executed "
+                      "(tflops_executed, pct_mfma_peak_executed); on the two_pass route value is what is executed",
+        "route": route,
+        "tflops_executed": flops_executed / ms / 1e9,
+        "pct_mfma_peak_executed": 100.0 * flops_executed / ms / 1e9 / peak,
         "tokens_computed": rows,
         "tflops_8NHV_convention": 8.0 * N * H * V / ms / 1e9,
         "pct_mfma_peak_8NHV_convention": 100.0 * 8.0 * N * H * V / ms / 1e9 / PEAK_TFLOPS[cfg["dtype"]],

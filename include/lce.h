@@ -261,6 +261,57 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
                  const float* lse, const int64_t* n_valid, const float* grad_out,
                  void* dx, void* dw, void* ws, size_t ws_bytes, void* stream);
 
+/*
+ * Forward and backward in one call, from ONE evaluation of the logits.
+ * Replaces LinearXentImplementation.forward as the reference runs it when a
+ * gradient is wanted (ops.py:687-802): there the loop over N_chunk_size-row
+ * groups computes the logits of a group once, keeps them in memory (ops.py:700)
+ * and launches the dx / dA programs on them before the next group
+ * (ops.py:721-791).  Same inputs and outputs as lce_forward followed by
+ * lce_backward; the gradients differ from theirs by rounding only (the staged
+ * dz is rounded to the 16-bit compute type twice instead of once, see below).
+ *
+ * The tokens go through in chunks of `chunk_rows` rows (lce_forward_backward_plan)
+ * against the whole vocabulary.  Per chunk: the logit kernel writes the forward's
+ * per-slice partials and, in the 16-bit compute type, e = exp(z - slice max)
+ * for every logit (chunk_rows * V * 2 bytes); the row merge gives lse; one pass
+ * over the stage turns e into dz; dx of the chunk is complete after one
+ * contraction; dW is summed over the chunks in an fp32 plane of H * V * 4 bytes
+ * (the reference's fp32 At_grad, ops.py:692; no plane with a single chunk).
+ * The chunk is the longest for which all of it stays within n_chunk * V * 4
+ * bytes.  8*N*H*V FLOPs become 6*N*H*V.
+ *
+ * Problems this route does not cover take the two calls above, one after the
+ * other on the same workspace, inside this entry point: fp32 activations, a
+ * weight whose dtype differs from x's, monitoring != 0, and shapes whose plane
+ * leaves no room for a chunk within the bound (lce_forward_backward_plan then
+ * reports 0 chunks).  `phases` selects kernels of either route; on the one-pass
+ * route LCE_PHASE_FWD_TILES is the logit kernel and LCE_PHASE_BWD_DZ the pass
+ * that turns e into dz.
+ *
+ *   grad_out   device pointer to 1 float: upstream gradient of the loss
+ *              (the reference multiplies it in afterwards, ops.py:810)
+ *   dx, dw     as for lce_backward; with both NULL this is lce_forward
+ *   ws         lce_forward_backward_workspace_bytes(p) bytes
+ */
+int lce_forward_backward_workspace_bytes(const lce_problem* p, size_t* bytes);
+int lce_forward_backward_plan(const lce_problem* p, int64_t* chunks, int64_t* chunk_rows);
+int lce_forward_backward(const lce_problem* p, const void* x, const void* w, const int64_t* y,
+                         const float* grad_out, float* lse, float* out5, int64_t* n_valid,
+                         void* dx, void* dw, void* ws, size_t ws_bytes, void* stream);
+
+/*
+ * t[r][c] *= *factor for r < rows, c < cols, in place, the product formed in
+ * fp32; `factor` is a device pointer to 1 float, and when it holds 1 the call
+ * reads and writes nothing else.  Replaces the x_grad.mul_(grad_output) /
+ * At_grad.mul_(grad_output) of LinearXentImplementation.backward (ops.py:810)
+ * for gradients that lce_forward_backward produced with a grad_out of 1
+ * (a caller that only learns the upstream gradient later, as autograd does).
+ * Row stride `ld` in elements: a multiple of 8 (16-bit) or 4 (fp32), rows on
+ * 16-byte boundaries.
+ */
+int lce_scale(void* t, int dtype, int64_t rows, int64_t cols, int64_t ld, const float* factor, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

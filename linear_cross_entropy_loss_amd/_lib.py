@@ -27,6 +27,10 @@ EXPORTS = (
     "lce_forward",
     "lce_forward_static",
     "lce_backward",
+    "lce_forward_backward_workspace_bytes",
+    "lce_forward_backward_plan",
+    "lce_forward_backward",
+    "lce_scale",
 )
 
 _DTYPES = {torch.bfloat16: LCE_BF16, torch.float16: LCE_F16, torch.float32: LCE_F32}
@@ -95,6 +99,14 @@ def load():
     lib.lce_forward_static.argtypes = [P, vp, vp, vp, vp, vp, vp, vp]
     lib.lce_backward.restype = ctypes.c_int
     lib.lce_backward.argtypes = [P, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+    lib.lce_forward_backward_workspace_bytes.restype = ctypes.c_int
+    lib.lce_forward_backward_workspace_bytes.argtypes = [P, ctypes.POINTER(sz)]
+    lib.lce_forward_backward_plan.restype = ctypes.c_int
+    lib.lce_forward_backward_plan.argtypes = [P, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]
+    lib.lce_forward_backward.restype = ctypes.c_int
+    lib.lce_forward_backward.argtypes = [P, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+    lib.lce_scale.restype = ctypes.c_int
+    lib.lce_scale.argtypes = [vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, vp, vp]
     _lib = lib
     return lib
 
@@ -149,3 +161,21 @@ def backward_plan(prob: LceProblem) -> tuple[int, int]:
     n, w = ctypes.c_int64(0), ctypes.c_int64(0)
     raise_for_status(lib.lce_backward_plan(ctypes.byref(prob), ctypes.byref(n), ctypes.byref(w)), "lce_backward_plan")
     return int(n.value), int(w.value)
+
+
+def forward_backward_workspace_bytes(prob: LceProblem) -> int:
+    lib = load()
+    b = ctypes.c_size_t(0)
+    raise_for_status(lib.lce_forward_backward_workspace_bytes(ctypes.byref(prob), ctypes.byref(b)),
+                     "lce_forward_backward_workspace_bytes")
+    return int(b.value)
+
+
+def forward_backward_plan(prob: LceProblem) -> tuple[int, int]:
+    """(chunks of token rows, rows per chunk) of lce_forward_backward's single pass over the logits for `prob`;
+    (0, 0) when the call would run lce_forward and lce_backward one after the other instead."""
+    lib = load()
+    n, r = ctypes.c_int64(0), ctypes.c_int64(0)
+    raise_for_status(lib.lce_forward_backward_plan(ctypes.byref(prob), ctypes.byref(n), ctypes.byref(r)),
+                     "lce_forward_backward_plan")
+    return int(n.value), int(r.value)

@@ -16,7 +16,7 @@ CSRC = PKG_DIR / "csrc"
 LIB_NAME = "liblce_gfx950.so"
 LIB_PATH = PKG_DIR / LIB_NAME
 
-SOURCES = ["lce_api.hip", "lce_fwd.hip", "lce_bwd_dz.hip", "lce_bwd_dx.hip", "lce_bwd_dw.hip", "lce_convert.hip", "lce_compact.hip"]
+SOURCES = ["lce_api.hip", "lce_fwd.hip", "lce_bwd_dz.hip", "lce_bwd_dx.hip", "lce_bwd_dw.hip", "lce_convert.hip", "lce_compact.hip", "lce_fuse.hip"]
 # Measurement probes (`bench.py --probe`): sources and library of their own, built on demand only.
 PROBE_DIR = PKG_DIR / "probes"
 PROBE_LIB_NAME = "liblce_probe_gfx950.so"

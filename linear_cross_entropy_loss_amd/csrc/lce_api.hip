@@ -315,6 +315,74 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   return LCE_EWORKSPACE;
 }
 
+// lce_forward_backward: the logits are computed once.  The tokens go through in chunks of `nc` rows against the
+// whole vocabulary: logit kernel (partials of the loss, and e = exp(z - slice max) into the stage), row merge
+// (lse), the pass that turns e into dz, then dx of the chunk (complete: K = the vocabulary) and the chunk's
+// term of dW, which is summed over the chunks in an fp32 plane (the reference's fp32 At_grad, ops.py:692).
+// Everything counts towards the bound n_chunk * V * 4 (the reference's logits chunk, ops.py:700): the chunk is
+// the longest that fits.  Problems outside the set below -- and those whose plane alone does not fit -- take the
+// two-pass route (forward, then a backward that recomputes the logits).
+struct FusedPlan {
+  bool ok;
+  bool pack;
+  int64_t nc;
+  int chunks;
+  PackPlan k;
+  size_t chunk_rows, lse_rows, tgt, blk, part_lse, part_max, stage, plane, part, total;
+  bool parts_on;
+};
+
+bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) {
+  memset(f, 0, sizeof(*f));
+  const bool x16 = p->x_dtype == LCE_BF16 || p->x_dtype == LCE_F16;
+  if (!x16 || p->w_dtype != p->x_dtype || p->monitoring) return false;
+  const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V), Hp = (size_t)lce::padded_hidden(p->H);
+  const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
+  // (packed rows of dx go to their tokens through 32-bit offsets into dx)
+  f->pack = packs_rows(p) && (size_t)p->N * (size_t)p->lddx * dxes < ((size_t)1 << 31);
+  f->k = plan_pack(p, 0, false);
+  size_t o = f->pack ? f->k.end : f->k.xc;  // the labels are always counted; the copy of x only exists for packed rows
+  f->chunk_rows = o; o += align_up(1024 * 8);
+  f->lse_rows = o; o += align_up(Np * 4);
+  f->tgt = o; o += align_up(Np * 4);
+  f->blk = o; o += align_up(Np / lce::kMergeRows * 8 * sizeof(double));
+  const size_t fixed = o;
+  const size_t bound = (size_t)p->n_chunk * (size_t)p->V * 4;
+  const size_t reserve = align_up((size_t)p->N * 4) + 4096;  // what the caller holds besides the workspace: lse and a few scalars
+  auto total_for = [&](int64_t nc, int chunks, FusedPlan* out) -> size_t {
+    size_t t = fixed;
+    const size_t part = align_up(Vp / lce::kChunkV * (size_t)nc * 4);
+    out->part_lse = t; t += part;
+    out->part_max = t; t += part;
+    out->stage = t; t += align_up((size_t)nc * Vp * 2);
+    // split-K partial sums of dx (and, with a single chunk, of dW): one buffer
+    size_t pb = want_dx ? dx_part_bytes((size_t)nc, Hp, (int64_t)Vp, (int64_t)Vp) : 0;
+    if (chunks == 1 && want_dw) {
+      const size_t w = dw_part_bytes((size_t)nc, Hp, (int64_t)Vp, (int64_t)Vp);
+      if (w > pb) pb = w;
+    }
+    out->part = t; t += pb;
+    out->parts_on = pb != 0;
+    out->plane = t;
+    if (chunks > 1 && want_dw) t += align_up(Hp * Vp * 4);
+    out->total = t;
+    return t;
+  };
+  // one chunk if it fits; else the fewest chunks of equal length that do
+  const int64_t tiles = (int64_t)(Np / 256);
+  for (int chunks = 1; chunks <= tiles && chunks <= 1024; ++chunks) {
+    const int64_t nc = (tiles + chunks - 1) / chunks * 256;
+    if ((nc * (chunks - 1)) >= (int64_t)Np) continue;  // the same chunk length as with one chunk fewer
+    if (total_for(nc, chunks, f) + reserve <= bound) {
+      f->nc = nc;
+      f->chunks = (int)(((int64_t)Np + nc - 1) / nc);
+      f->ok = true;
+      return true;
+    }
+  }
+  return false;
+}
+
 bool misaligned(const void* p) { return ((uintptr_t)p & 15) != 0; }
 
 // Scratch of lce_forward_static: a fixed array in device memory, one copy per GPU the library runs on,
@@ -451,6 +519,143 @@ int forward_impl(const lce_problem* p, const void* x, const void* w, const int64
   if (ph & LCE_PHASE_FWD_REDUCE) {
     e = lce::launch_fwd_final(a, s);
     if (e != hipSuccess) return hip_fail(e, "fwd_final");
+  }
+  return LCE_OK;
+}
+
+// Body of lce_forward_backward for a problem that plan_fused accepts.
+int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const void* w, const int64_t* y,
+               const float* grad_out, float* lse, float* out5, int64_t* n_valid, void* dx, void* dw, void* ws,
+               void* stream) {
+  hipStream_t s = (hipStream_t)stream;
+  char* base = (char*)ws;
+  const PackPlan& k = f.k;
+  const int64_t Np = lce::padded_tokens(p->N), Vp = lce::padded_vocab(p->V);
+  const int64_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
+  int num_cus = 0;
+  int rc = current_num_cus(&num_cus, p->max_workgroups);
+  if (rc != LCE_OK) return rc;
+  int64_t* n_rows = (int64_t*)(base + k.n_rows);
+  int* perm = (int*)(base + k.perm);
+  int64_t* yc = (int64_t*)(base + k.yc);
+  int64_t* chunk_rows = (int64_t*)(base + f.chunk_rows);
+
+  // row merge and final sums: the forward's own kernels
+  lce::FwdArgs fa;
+  memset(&fa, 0, sizeof(fa));
+  fa.x = x; fa.w = w; fa.y = y;
+  fa.N = p->N; fa.H = p->H; fa.V = p->V; fa.ldx = p->ldx; fa.ldw = p->ldw;
+  fa.Np = Np; fa.Vp = Vp;
+  fa.x_dtype = p->x_dtype; fa.w_dtype = p->w_dtype;
+  fa.ignore_index = p->ignore_index;
+  fa.scale = p->logit_scale; fa.z_reg = p->z_reg; fa.monitoring = 0;
+  fa.lse = lse; fa.out5 = out5; fa.n_valid = n_valid;
+  fa.part_lse = (float*)(base + f.part_lse);
+  fa.tgt = (float*)(base + f.tgt);
+  fa.blk = (float*)(base + f.blk);
+  fa.lse_rows = (float*)(base + f.lse_rows);
+  fa.num_cus = num_cus;
+  fa.nc = f.nc;
+  if (f.pack) {
+    fa.n_rows = n_rows; fa.perm = perm; fa.y0 = y; fa.y = yc;
+  }
+
+  // (a call restricted to some kernels works on what a full call left in the workspace)
+  const int ph = p->phases ? p->phases : ~0;
+  // the count of valid labels comes first (the gradients' factor needs it), with it the packing
+  hipError_t e = hipSuccess;
+  if (ph & LCE_PHASE_PACK) {
+    e = lce::launch_compact_labels(y, p->N, p->ignore_index, (int*)(base + k.cnt), n_rows, perm, yc, s);
+    if (e != hipSuccess) return hip_fail(e, "compact_labels");
+  }
+  if (f.pack && (ph & LCE_PHASE_PACK)) {
+    e = lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, perm, n_rows, p->N, base + k.xc, k.ldxc * 2, nullptr, nullptr,
+                                num_cus, s, true);
+    if (e != hipSuccess) return hip_fail(e, "gather_rows");
+    e = lce::launch_chunk_rows(n_rows, p->N, f.nc, f.chunks, chunk_rows, s);
+    if (e != hipSuccess) return hip_fail(e, "chunk_rows");
+  }
+
+  lce::BwdArgs b;
+  memset(&b, 0, sizeof(b));
+  b.w = w; b.n_valid = n_rows; b.grad_out = grad_out;
+  b.H = p->H; b.V = p->V; b.Hp = lce::padded_hidden(p->H);
+  b.ldw = p->ldw; b.lddx = p->lddx; b.lddw = p->lddw;
+  b.x_dtype = p->x_dtype; b.w_dtype = p->w_dtype; b.dx_dtype = p->dx_dtype; b.dw_dtype = p->dw_dtype;
+  b.w_vh = p->w_layout == LCE_W_VH;
+  b.ignore_index = p->ignore_index;
+  b.scale = p->logit_scale; b.z_reg = p->z_reg;
+  b.dw = dw;
+  b.dz_shift = p->x_dtype == LCE_F16 && p->z_reg <= 0.03125f ? 10 : 0;  // (as in lce_backward)
+  b.dz = base + f.stage;
+  b.v0 = 0; b.vw = p->V; b.vs = Vp; b.wv0 = 0; b.Vw = p->V;
+  b.first = 1; b.last = 1;
+  b.num_cus = num_cus; b.dx_grid = num_cus; b.dw_grid = num_cus;
+  b.live = lce::live_bands(lce::padded_k(p->H) * 2);
+  b.part_lse = (float*)(base + f.part_lse);
+  b.part_max = (float*)(base + f.part_max);
+  b.nc = f.nc;
+  b.dx_part = f.parts_on && dx ? (float*)(base + f.part) : nullptr;
+  b.dw_part = f.parts_on && dw && f.chunks == 1 ? (float*)(base + f.part) : nullptr;
+  b.dw_plane = f.chunks > 1 ? (float*)(base + f.plane) : nullptr;
+
+  for (int c = 0; c < f.chunks; ++c) {
+    const int64_t row0 = (int64_t)c * f.nc;
+    lce::BwdArgs a = b;
+    a.Np = Np - row0 < f.nc ? Np - row0 : f.nc;
+    a.dz_rows = a.Np;
+    a.lse = (const float*)(base + f.lse_rows) + row0;
+    a.tgt = (float*)(base + f.tgt) + row0;
+    if (f.pack) {
+      a.N = p->N;
+      a.n_rows = chunk_rows + c;
+      a.perm = perm + row0;
+      a.perm_always = 1;
+      a.x = a.xc = base + k.xc + (size_t)row0 * (size_t)k.ldxc * 2;
+      a.ldx = a.ldxc = k.ldxc;
+      a.y = yc + row0;
+      a.dx = dx;
+    } else {
+      a.N = p->N - row0 < f.nc ? p->N - row0 : f.nc;
+      a.x = a.xc = (const char*)x + (size_t)row0 * (size_t)p->ldx * 2;
+      a.ldx = a.ldxc = p->ldx;
+      a.y = y + row0;
+      a.dx = dx ? (char*)dx + (size_t)row0 * (size_t)p->lddx * dxes : nullptr;
+    }
+    a.dw_acc = f.chunks == 1 ? 0 : (c == 0 ? 1 : 2);
+    a.last_chunk = c == f.chunks - 1;
+    if (ph & LCE_PHASE_FWD_TILES) {
+      e = lce::launch_fwd_stage(a, s);
+      if (e != hipSuccess) return hip_fail(e, "fwd_stage");
+    }
+    if (ph & LCE_PHASE_FWD_REDUCE) {
+      lce::FwdArgs r = fa;
+      r.row0 = row0;
+      e = lce::launch_fwd_rows(r, s);
+      if (e != hipSuccess) return hip_fail(e, "fwd_rows");
+    }
+    if ((dx || dw) && (ph & LCE_PHASE_BWD_DZ)) {
+      e = lce::launch_stage_scale(a, s);
+      if (e != hipSuccess) return hip_fail(e, "stage_scale");
+    }
+    if (dx && (ph & LCE_PHASE_BWD_DX)) {
+      e = lce::launch_bwd_dx(a, s);
+      if (e != hipSuccess) return hip_fail(e, "bwd_dx");
+    }
+    if (dw && (ph & LCE_PHASE_BWD_DW)) {
+      e = lce::launch_bwd_dw(a, s);
+      if (e != hipSuccess) return hip_fail(e, "bwd_dw");
+    }
+  }
+  if (ph & LCE_PHASE_FWD_REDUCE) {
+    e = lce::launch_fwd_final(fa, s);
+    if (e != hipSuccess) return hip_fail(e, "fwd_final");
+  }
+  if (f.pack && dx && (ph & LCE_PHASE_BWD_DX)) {
+    // tokens that were dropped get exact zeros (nothing to do if none was)
+    e = lce::launch_scatter_rows(nullptr, 0, perm, n_rows, p->N, y, p->ignore_index, dx, p->lddx * dxes, p->H * dxes,
+                                 num_cus, s);
+    if (e != hipSuccess) return hip_fail(e, "scatter_rows");
   }
   return LCE_OK;
 }
@@ -687,6 +892,60 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
     if (e != hipSuccess) return hip_fail(e, "scatter_rows");
   }
   return LCE_OK;
+}
+
+int lce_scale(void* t, int dtype, int64_t rows, int64_t cols, int64_t ld, const float* factor, void* stream) {
+  if (dtype != LCE_BF16 && dtype != LCE_F16 && dtype != LCE_F32) return LCE_EINVAL_DTYPE;
+  if (rows < 0 || cols < 0 || ld < cols || ld % (dtype == LCE_F32 ? 4 : 8) || !factor) return LCE_EINVAL_ARG;
+  if (rows == 0 || cols == 0) return LCE_OK;
+  if (!t || misaligned(t)) return LCE_EINVAL_ARG;
+  int num_cus = 0;
+  int rc = current_num_cus(&num_cus, 0);
+  if (rc != LCE_OK) return rc;
+  hipError_t e = lce::launch_scale_rows(t, dtype, rows, cols, ld, factor, num_cus, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "scale_rows");
+  return LCE_OK;
+}
+
+int lce_forward_backward_workspace_bytes(const lce_problem* p, size_t* bytes) {
+  int rc = check(p, true);
+  if (rc != LCE_OK) return rc;
+  if (!bytes) return LCE_EINVAL_ARG;
+  FusedPlan f;
+  if (plan_fused(p, true, true, &f)) { *bytes = f.total; return LCE_OK; }
+  size_t fw = 0, bw = 0;
+  rc = lce_workspace_bytes(p, &fw, &bw);
+  if (rc != LCE_OK) return rc;
+  *bytes = fw > bw ? fw : bw;
+  return LCE_OK;
+}
+
+int lce_forward_backward_plan(const lce_problem* p, int64_t* chunks, int64_t* chunk_rows) {
+  int rc = check(p, true);
+  if (rc != LCE_OK) return rc;
+  FusedPlan f;
+  const bool ok = plan_fused(p, true, true, &f);
+  if (chunks) *chunks = ok ? f.chunks : 0;
+  if (chunk_rows) *chunk_rows = ok ? f.nc : 0;
+  return LCE_OK;
+}
+
+int lce_forward_backward(const lce_problem* p, const void* x, const void* w, const int64_t* y,
+                         const float* grad_out, float* lse, float* out5, int64_t* n_valid, void* dx,
+                         void* dw, void* ws, size_t ws_bytes, void* stream) {
+  int rc = check(p, true);
+  if (rc != LCE_OK) return rc;
+  if (!x || !w || !y || !grad_out || !lse || !out5 || !n_valid) return LCE_EINVAL_ARG;
+  if (misaligned(x) || misaligned(w) || misaligned(dx) || misaligned(dw)) return LCE_EINVAL_ARG;
+  FusedPlan f;
+  if ((dx || dw) && plan_fused(p, true, true, &f)) {
+    if (!ws || ws_bytes < f.total || misaligned(ws)) return LCE_EWORKSPACE;
+    return fused_impl(p, f, x, w, y, grad_out, lse, out5, n_valid, dx, dw, ws, stream);
+  }
+  // two passes over the logits, on the same workspace one after the other
+  rc = forward_impl(p, x, w, y, lse, out5, n_valid, ws, ws_bytes, stream);
+  if (rc != LCE_OK || (!dx && !dw)) return rc;
+  return lce_backward(p, x, w, y, lse, n_valid, grad_out, dx, dw, ws, ws_bytes, stream);
 }
 
 }  // extern "C"

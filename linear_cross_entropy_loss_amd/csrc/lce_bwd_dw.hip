@@ -188,6 +188,45 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
   }
 }
 
+// dW summed over chunks of token rows (BwdArgs::dw_plane): the tile's block of the plane holds the accumulator
+// as the registers do -- quad (rb, cbk, rq) of thread t at float 4 * (((rb * 4 + cbk) * 4 + rq) * 256 + t) -- so
+// that every load and store of a wave covers 1 KiB of consecutive addresses.  LOAD: the block is added to the
+// accumulator before the sums go (back) to the block.  After the last chunk dw_plane_out_kernel scales the sums
+// and stores dW.
+// The four quads of an accumulator block are fetched together before any is used.
+template <bool LOAD>
+LCE_DEV void dw_plane_io(float* blk, f32x16_t (&acc)[kNB][kNB]) {
+  // one descriptor over the block, the thread's 16 bytes as the vector offset, the quad as a scalar offset: no
+  // 64-bit address per quad
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(blk, 0, kTile * kTile * 4, 0x00020000);
+  const int voff = opaque_tid() * 16;
+#pragma unroll
+  for (int rb = 0; rb < kNB; ++rb)
+#pragma unroll
+    for (int cb = 0; cb < kNB; ++cb) {
+      u32x4_t old[4];
+      if (LOAD) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq)
+          old[rq] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, ((rb * 4 + cb) * 4 + rq) * 4096, 0);
+      }
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        f32x4_t v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          // (a volatile read: the compiler would otherwise read all 256 accumulator registers before the first load)
+          float t;
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[rb][cb][rq * 4 + j]));
+          v[j] = t;
+        }
+        if (LOAD) v += __builtin_bit_cast(f32x4_t, old[rq]);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), rsrc, voff, ((rb * 4 + cb) * 4 + rq) * 4096, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // (the quads of one accumulator block in registers at a time: an operand tile is in flight)
+    }
+}
+
 // How one launch divides its work: as for dx (lce_bwd_dx.hip).  The T = (vs/256) x (Hp/256) output tiles
 // go to G persistent workgroups in rounds; a last round with r <= G/2 tiles is cut along K = tokens into
 // `nseg` segments of `kseg` K tiles (r * nseg <= G, at least 16 K tiles each), whose fp32 sums meet in
@@ -232,7 +271,8 @@ LCE_DEV DwPlan dw_plan(const BwdArgs& a, int64_t rows) {
 //   kDwTails     the K segments of the tail tiles only (their launch follows that of the whole tiles)
 enum { kDwAll = 0, kDwStaged = 1, kDwTails = 2, kDwStaged32 = 3 };
 
-template <class T, bool WVH, int MODE> struct DwProblem {
+// ACC: what the plane of sums over chunks of token rows has to do with a tile (BwdArgs::dw_acc; whole tiles only).
+template <class T, bool WVH, int MODE, int ACC = 0> struct DwProblem {
   static constexpr bool kSwapAB = !WVH;  // (H, V) output: dz, the Q operand, feeds the A side (v along registers)
   static constexpr bool kVarK = true;    // whole tiles and segment items have different K extents
   static constexpr bool kKMask = false;  // both operands have K as their slow index: nothing to mask
@@ -299,6 +339,11 @@ template <class T, bool WVH, int MODE> struct DwProblem {
   LCE_DEV void epilogue(int local, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int item, tp, tq, seg;
     decode(local, item, tp, tq, seg);
+    if constexpr (ACC != 0) {
+      float* blk = a.dw_plane + ((int64_t)tq * tiles_p + tp) * (kTile * kTile);
+      dw_plane_io<ACC == 2>(blk, acc);
+      return;
+    }
     if (MODE == kDwStaged || MODE == kDwStaged32) {
       dw_store_rows_hv<T, MODE == kDwStaged32>(a, acc, tp, tq, scratch);
     } else {
@@ -308,12 +353,12 @@ template <class T, bool WVH, int MODE> struct DwProblem {
   }
 };
 
-template <class T, bool WVH, int MODE>
+template <class T, bool WVH, int MODE, int ACC>
 __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DwProblem<T, WVH, MODE> prob(a);
-  Pipe3<T, E, false, E, false, DwProblem<T, WVH, MODE>> pipe(prob);
+  DwProblem<T, WVH, MODE, ACC> prob(a);
+  Pipe3<T, E, false, E, false, DwProblem<T, WVH, MODE, ACC>> pipe(prob);
   pipe.run(prob.ldx, a.vs / kBK, prob.plan.kt, lds);
 }
 
@@ -351,8 +396,8 @@ __global__ __launch_bounds__(256) void dw_tail_kernel(const BwdArgs a) {
   }
 }
 
-template <class T, bool WVH, int MODE> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
-  auto kern = bwd_dw_persistent_kernel<T, WVH, MODE>;
+template <class T, bool WVH, int MODE, int ACC = 0> hipError_t launch_tiles(const BwdArgs& a, hipStream_t s) {
+  auto kern = bwd_dw_persistent_kernel<T, WVH, MODE, ACC>;
   static LdsOptIn optin;
   hipError_t e = optin.ensure(reinterpret_cast<const void*>(kern), kMainloopLds);
   if (e != hipSuccess) return e;
@@ -360,7 +405,51 @@ template <class T, bool WVH, int MODE> hipError_t launch_tiles(const BwdArgs& a,
   return hipGetLastError();
 }
 
+// The plane of sums over chunks of token rows becomes dW: one workgroup per tile, thread t takes the quads that
+// thread t of the tile kernel stored (dw_plane_io) and puts them where dw_epilogue would have.
+template <class T, bool WVH>
+__global__ __launch_bounds__(256) void dw_plane_out_kernel(const BwdArgs a) {
+  typedef typename elem_of<T>::type E;
+  const int tiles_p = (int)(a.Hp / kTile);
+  const int tq = (int)blockIdx.x / tiles_p, tp = (int)blockIdx.x % tiles_p;
+  const DwTileGeom<WVH> g(a, tp, tq);
+  const float coef = final_factor_of(a);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wp = wave & 1, wq = wave >> 1, half = lane >> 5;
+  const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
+  const float* mine = a.dw_plane + (int64_t)blockIdx.x * (kTile * kTile) + threadIdx.x * 4;
+#pragma unroll 4
+  for (int q = 0; q < 64; ++q) {
+    const int i = q >> 4, k = (q >> 2) & 3, rq = q & 3;  // quad rq of acc[i][k]
+    const int rb = WVH ? k : i, cbk = WVH ? i : k;
+    const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + (lane & 31);
+    const int64_t col = g.col0 + w_col * kWaveTile + cbk * kBlk + 8 * rq + 4 * half;
+    const f32x4_t v = *reinterpret_cast<const f32x4_t*>(mine + q * 1024) * coef;
+    if (row >= g.row_limit || col >= g.col_limit) continue;  // a quad that the last column cuts through is written whole, into the stride padding of its row
+    if (a.dw_dtype == DT_F32) {
+      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + row * a.lddw + col) = v;
+    } else {
+      u32x2_t o;
+      o[0] = pack2<T>(v[0], v[1]);
+      o[1] = pack2<T>(v[2], v[3]);
+      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dw) + row * a.lddw + col) = o;
+    }
+  }
+}
+
+// Whole tiles that meet the plane of sums over chunks of token rows (nothing is split along K then).
+template <class T, bool WVH, int MODE> hipError_t launch_plane(const BwdArgs& a, hipStream_t s) {
+  hipError_t e = a.dw_acc == 1 ? launch_tiles<T, WVH, MODE, 1>(a, s) : launch_tiles<T, WVH, MODE, 2>(a, s);
+  if (e != hipSuccess || !a.last_chunk) return e;
+  hipLaunchKernelGGL((dw_plane_out_kernel<T, WVH>), dim3((unsigned)((a.vs / kTile) * (a.Hp / kTile))), dim3(256), 0, s, a);
+  return hipGetLastError();
+}
+
 template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  if (a.dw_acc != 0) {
+    if (a.dw_plane == nullptr || a.dw_part != nullptr || a.dw_acc > 2) return hipErrorInvalidValue;
+    return launch_plane<T, WVH, kDwAll>(a, s);
+  }
   // a last round of tiles may be split along K (the tile count does not depend on the rows; whether its K
   // extent is long enough to split is decided on the device, and a launch without items returns at once)
   const bool tails = a.dw_part != nullptr && dw_tail_blocks(a.Np, a.Hp, a.vs) != 0 &&

@@ -216,7 +216,7 @@ template <class T, bool KMASK, bool WVH, int MODE> struct DxProblem {
     if (MODE == kDxTails) {
       dx_store_segment(a.dx_part + (int64_t)(item - plan.full) * kTile * kTile, acc);
     } else {
-      const bool packed = rows != a.N, copy = packed && a.dxc != nullptr;
+      const bool packed = rows != a.N || a.perm_always != 0, copy = packed && a.dxc != nullptr;
       dx_epilogue<T, MODE == kDxMiddle || MODE == kDxLast, MODE == kDxLast || MODE == kDxOnly>(
           a, rows, copy ? a.dxc : a.dx, copy ? a.lddxc : a.lddx, packed && !copy ? a.perm : nullptr, acc, tp, tq);
     }
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(256) void dx_tail_kernel(const BwdArgs a) {
   if (b >= plan.tail_tiles) return;
   int tp, tq;
   tile_coords(plan.full + b, plan.tiles, tiles_p, tiles_q, 8, 8, tp, tq);
-  const bool packed = rows != a.N, copy = packed && a.dxc != nullptr;
+  const bool packed = rows != a.N || a.perm_always != 0, copy = packed && a.dxc != nullptr;
   void* out = copy ? a.dxc : a.dx;
   const int64_t ldo = copy ? a.lddxc : a.lddx;
   const int* perm = packed && !copy ? a.perm : nullptr;

@@ -62,7 +62,12 @@ constexpr int kDzStoreAux = LCE_DZ_STORE_AUX;  // cache policy of the dz stores:
 // in three parts of Np rows, [hi ; lo ; hi], each lane storing its 16-byte runs itself (this
 // path serves accuracy, not speed).
 // `pf_y`, `pf_lse`: label and lse of this lane's four tokens (DzProblem::prefetch), ignore_index / 0 for rows that do not exist.
-template <class T, bool ZREG, bool VTAIL, bool SPLIT>
+//
+// FUSE (launch_fwd_stage: the logits are computed once, for the loss and for the gradients): the tile leaves
+// e = 2^dz_shift * exp(z - m) instead, m = the largest logit of the token within this wave's 128 columns, for
+// every row, whatever its label; the wave also writes the forward's partials of its slice (m and
+// m + log sum exp(z - m)) and the target logit.  `pf_lse` is not used.
+template <class T, bool ZREG, bool VTAIL, bool SPLIT, bool FUSE>
 LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], const float (&pf_lse)[kNB],
                               f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* pieces) {
   typedef typename elem_of<T>::type E;
@@ -106,9 +111,9 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
     const int64_t yy = pf_y[qb];  // (rows past the last one are staged as zeros, like ignored tokens)
     const int64_t rel = yy - slice_v0;
     const bool valid = yy != a.ignore_index;
-    const float l = pf_lse[qb];
+    const float l = FUSE ? 0.f : pf_lse[qb];
     // (the power-of-two factor of the staged dz rides along in the exponent)
-    nlse[qb] = valid ? fmaf(-l, kLog2e, (float)a.dz_shift) : -INFINITY;
+    nlse[qb] = valid ? fmaf(-l, kLog2e, (float)a.dz_shift) : -INFINITY;  // (FUSE: set per block below)
     gain[qb] = 1.f + 2.f * a.z_reg * l;
     // (with the staging factor 2^10 of fp16 in place: |dz| * 2^10 <= 63 * 2^10 stays finite in fp16 whatever lse is)
     if (a.dz_shift != 0) gain[qb] = fminf(fmaxf(gain[qb], -63.f), 63.f);
@@ -118,6 +123,24 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
 
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
+    float m = -INFINITY, ssum = 0.f;
+    if constexpr (FUSE) {
+      // the largest of this token's logits in the slice: this lane's 64, then the other half's
+#pragma unroll
+      for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq)
+          if (!VTAIL || pb * 4 + rq < nq) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) m = fmaxf(m, acc[pb][qb][rq * 4 + j]);
+          } else if (pb * 4 + rq == nq && cut != 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) m = j < cut_mine ? fmaxf(m, acc[pb][qb][rq * 4 + j]) : m;
+          }
+      m = fmaxf(m, __shfl_xor(m, 32));
+      // (a slice with no column inside the vocabulary: every e below is an exact zero, whatever this is)
+      nlse[qb] = fmaf(-m, c1, (float)a.dz_shift);
+    }
 #pragma unroll
     for (int pb = 0; pb < kNB; ++pb) {
       const unsigned blk_off = (unsigned)((pb >> 1) * grp * 2) + qb * (kBlk * kGroup * 2);  // bytes, uniform
@@ -144,6 +167,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
             for (int i = 4 * h2; i < 4 * h2 + 4; ++i) d[i] = 0.f;
           }
         }
+        if constexpr (FUSE) ssum += ((d[0] + d[1]) + (d[2] + d[3])) + ((d[4] + d[5]) + (d[6] + d[7]));
 #pragma unroll
         for (int part = 0; part < (SPLIT ? 2 : 1); ++part) {
           if (part == 1) {
@@ -193,7 +217,31 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
     // 16-byte piece that holds the column may have been another lane's store).  (These rare branches also keep
     // the compiler from gathering the accumulator reads of all four blocks at the top, which spills.)
     const int yl = ykey[qb];
-    if (yl >= 0) {
+    if constexpr (FUSE) {
+      // the forward's partials of this slice for the token, and its target logit if it lies here
+      ssum += __shfl_xor(ssum, 32);
+      const int64_t tokl = t0 + wq * kWaveTile + qb * kBlk + (lane & 31);
+      const int64_t o = (slice_v0 / kChunkV) * a.nc + tokl;
+      if (lane < 32) {
+        // (no column of the slice inside the vocabulary: m = -inf, ssum = 0 -> -inf, nothing to add to the lse)
+        a.part_max[o] = m * a.scale;
+        a.part_lse[o] = ssum > 0.f ? fmaf(m, a.scale, (__builtin_amdgcn_logf(ssum) - (float)a.dz_shift) * 0.6931471805599453f)
+                                   : -INFINITY;
+      }
+      if (yl >= 0) {
+        const int want = (yl >> 5) * 16 + ((yl >> 3) & 3) * 4 + (yl & 3);  // (block, register) index
+        float zt = 0.f;
+#pragma unroll
+        for (int pb = 0; pb < kNB; ++pb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float v;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[pb][qb][r]));
+            if (want == pb * 16 + r) zt = v;
+          }
+        a.tgt[tokl] = zt * a.scale;
+      }
+    } else if (yl >= 0) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       const int want = (yl >> 5) * 16 + ((yl >> 3) & 3) * 4 + (yl & 3);  // (block, register) index
       float zt = 0.f;
@@ -226,7 +274,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
 // `tp0`: all the full ones, or (VTAIL) those from the one straddling the end
 // of the vocabulary to the end of the padded slab.
 // WVH: the weight is stored (V, H) row-major, so that the P operand runs along K in memory like x does.
-template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> struct DzProblem {
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH, bool FUSE = false> struct DzProblem {
   typedef typename elem_of<T>::type E;
   static constexpr bool kKMask = KMASK;
   static constexpr bool kSwapAB = false;
@@ -278,28 +326,28 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH> stru
       const int64_t tok = (int64_t)tq * kTile + wq * kWaveTile + qb * kBlk + (lane & 31);
       const bool exists = tok < rows;
       pf_y[qb] = exists ? a.y[tok] : a.ignore_index;
-      pf_lse[qb] = exists ? a.lse[tok] : 0.f;
+      pf_lse[qb] = exists && !FUSE ? a.lse[tok] : 0.f;
     }
   }
   LCE_DEV void epilogue(int tile, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int tp, tq;
     coords(tile, tp, tq);
-    dz_epilogue_impl<T, ZREG, VTAIL, SPLIT>(a, pf_y, pf_lse, acc, tp, tq, scratch + kStageBytes);  // (behind the main loop's stages)
+    dz_epilogue_impl<T, ZREG, VTAIL, SPLIT, FUSE>(a, pf_y, pf_lse, acc, tp, tq, scratch + kStageBytes);  // (behind the main loop's stages)
   }
 };
 
-template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH>
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH, bool FUSE>
 __global__ __launch_bounds__(kThreads) void bwd_dz_persistent_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
-  DzProblem<T, ZREG, VTAIL, KMASK, SPLIT, WVH> prob(a);
-  Pipe3<T, E, WVH, E, true, DzProblem<T, ZREG, VTAIL, KMASK, SPLIT, WVH>> pipe(prob);
+  DzProblem<T, ZREG, VTAIL, KMASK, SPLIT, WVH, FUSE> prob(a);
+  Pipe3<T, E, WVH, E, true, DzProblem<T, ZREG, VTAIL, KMASK, SPLIT, WVH, FUSE>> pipe(prob);
   pipe.run(a.ldw, prob.ldx, (int)(padded_k(a.H) / kBK), lds);
 }
 
-template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH>
+template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH, bool FUSE = false>
 hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
-  auto kern = bwd_dz_persistent_kernel<T, ZREG, VTAIL, KMASK, SPLIT, WVH>;
+  auto kern = bwd_dz_persistent_kernel<T, ZREG, VTAIL, KMASK, SPLIT, WVH, FUSE>;
   static LdsOptIn optin;
   hipError_t e = optin.ensure(reinterpret_cast<const void*>(kern), kLdsBytes);
   if (e != hipSuccess) return e;
@@ -309,15 +357,16 @@ hipError_t launch_one(const BwdArgs& a, int64_t tiles, hipStream_t s) {
 }
 
 // All full tile columns of the slab, then the column that straddles the end of the vocabulary.
-template <class T, bool ZREG, bool SPLIT, bool WVH> hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
+template <class T, bool ZREG, bool SPLIT, bool WVH, bool FUSE = false>
+hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
   const int64_t tq = a.Np / kTile, full = a.vw / kTile, tail = a.vs / kTile - full;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = exact_k ? launch_one<T, ZREG, false, false, SPLIT, WVH>(a, full * tq, s)
-                           : launch_one<T, ZREG, false, true, SPLIT, WVH>(a, full * tq, s);
+    hipError_t e = exact_k ? launch_one<T, ZREG, false, false, SPLIT, WVH, FUSE>(a, full * tq, s)
+                           : launch_one<T, ZREG, false, true, SPLIT, WVH, FUSE>(a, full * tq, s);
     if (e != hipSuccess) return e;
   }
-  if (tail > 0) return launch_one<T, ZREG, true, true, SPLIT, WVH>(a, tail * tq, s);
+  if (tail > 0) return launch_one<T, ZREG, true, true, SPLIT, WVH, FUSE>(a, tail * tq, s);
   return hipSuccess;
 }
 
@@ -339,6 +388,17 @@ hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
     return a.split ? launch_persistent<BF16, true, false>(a, s) : launch_persistent<BF16, false, false>(a, s);
   if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return launch_persistent<F16, false, false>(a, s);
   // (an fp32 weight arrives here as a 16-bit slab copy, fp32 activations as bf16 pairs with split set)
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_fwd_stage(const BwdArgs& a, hipStream_t s) {
+  if (a.split || a.part_lse == nullptr || a.part_max == nullptr || a.tgt == nullptr) return hipErrorInvalidValue;
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16)
+    return a.w_vh ? launch_persistent_z<BF16, false, false, true, true>(a, s)
+                  : launch_persistent_z<BF16, false, false, false, true>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16)
+    return a.w_vh ? launch_persistent_z<F16, false, false, true, true>(a, s)
+                  : launch_persistent_z<F16, false, false, false, true>(a, s);
   return hipErrorInvalidValue;
 }
 

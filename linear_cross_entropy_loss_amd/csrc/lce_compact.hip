@@ -99,9 +99,9 @@ __global__ __launch_bounds__(256) void pack_kept_kernel(const int64_t* y, int64_
 __global__ __launch_bounds__(256) void gather_rows_kernel(const char* x, int64_t ldx_bytes, const int* perm,
                                                           const int64_t* n_rows, int64_t N, char* xc,
                                                           int64_t ldxc_bytes, int chunks, int64_t row_bytes,
-                                                          const float* lse, float* lse_c) {
+                                                          const float* lse, float* lse_c, int always) {
   const int64_t rows = packed_rows(n_rows, N);
-  const bool copy_x = rows != N;
+  const bool copy_x = rows != N || always != 0;
   for (int64_t j = blockIdx.x; j < rows; j += gridDim.x) {
     const int64_t src = packed_token(perm, j, N);
     if (lse != nullptr && threadIdx.x == 0) lse_c[j] = lse[src];
@@ -220,10 +220,10 @@ hipError_t launch_gather_rows_split(const float* x, int64_t ldx, int64_t H, cons
 
 hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, int64_t row_bytes, const int* perm,
                               const int64_t* n_rows, int64_t N, void* xc, int64_t ldxc_bytes, const float* lse,
-                              float* lse_c, int num_cus, hipStream_t s) {
+                              float* lse_c, int num_cus, hipStream_t s, bool always) {
   hipLaunchKernelGGL(gather_rows_kernel, dim3(row_grid(N, num_cus)), dim3(256), 0, s,
                      reinterpret_cast<const char*>(x), ldx_bytes, perm, n_rows, N, reinterpret_cast<char*>(xc),
-                     ldxc_bytes, (int)(ldxc_bytes / 16), row_bytes, lse, lse_c);
+                     ldxc_bytes, (int)(ldxc_bytes / 16), row_bytes, lse, lse_c, always ? 1 : 0);
   return hipGetLastError();
 }
 

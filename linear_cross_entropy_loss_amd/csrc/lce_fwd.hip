@@ -431,6 +431,7 @@ __global__ __launch_bounds__(256) void fwd_rows_kernel(const FwdArgs a) {
       if (sh_s[i][r] != 0.f) St += sh_s[i][r] * fast_exp2((sh_m[i][r] - Mt) * kLog2e);
     const float lse = Mt + fast_log(St);
     sh_lse[r] = lse;
+    if (a.lse_rows != nullptr) a.lse_rows[tok] = lse;
     // lse[i] of a token with an ignored label is 0, whether its row was computed (all rows are when they are not
     // packed) or not: a caller sees one thing.  (sh_lse keeps the value: logit_entropy is taken over valid rows only,
     // and the backward never looks at the lse of such a token.)

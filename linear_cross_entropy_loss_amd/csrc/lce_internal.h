@@ -83,6 +83,7 @@ struct FwdArgs {
   float* part_sq;    // [Vp/128][nc]  per-slice sum z^2        (monitoring)
   float* tgt;        // [Np]          target logit (written for tokens whose label is a column of W)
   float* blk;        // [Np/64][8]    per-merge-block partial sums
+  float* lse_rows;   // [Np] or null  lse of every row in the order the tile kernels see them (packed rows), whatever its label
 };
 
 struct BwdArgs {
@@ -148,6 +149,24 @@ struct BwdArgs {
   int64_t ldxc;
   void* dxc;
   int64_t lddxc;
+  // One pass over the logits (lce_forward_backward): the problem is a chunk of token rows against the whole
+  // vocabulary, and the logit kernel (launch_fwd_stage) leaves, instead of dz,
+  //     e[token][v] = 2^dz_shift * exp(z[token][v] - m[token][v / 128])
+  // in the stage, m = the largest logit of the token in that slice of 128 columns, together with the forward's
+  // per-slice partials of the chunk: part_lse, part_max = m ([Vp/128][nc], as in FwdArgs) and the target logits
+  // tgt (first row of the chunk).  Once the rows' lse are known, launch_stage_scale turns e into dz in place.
+  float* part_lse;
+  float* part_max;
+  float* tgt;
+  int64_t nc;
+  // rows of dx always go to the tokens perm[] names (the rows of a chunk can be all there and still not be the
+  // tokens of the same numbers)
+  int perm_always;
+  // dW summed over chunks of token rows: dw_plane holds one 256 x 256 fp32 block per tile of dW, in the order of
+  // the accumulator registers (lce_bwd_dw.hip).  dw_acc: 0 = no plane (dW is stored as it comes), 1 = the sums
+  // are stored to the plane (first chunk), 2 = added to it; last_chunk: the plane is then scaled and stored as dW.
+  float* dw_plane;
+  int dw_acc, last_chunk;
 };
 
 // Element offset of block (row tile, column group) of a dz stage that is `vs` columns wide.
@@ -171,6 +190,14 @@ hipError_t launch_fwd_tiles(const FwdArgs& a, hipStream_t s);
 hipError_t launch_fwd_rows(const FwdArgs& a, hipStream_t s);
 hipError_t launch_fwd_final(const FwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s);
+// The logit kernel of lce_forward_backward and the pass that follows the row merge (see BwdArgs).
+hipError_t launch_fwd_stage(const BwdArgs& a, hipStream_t s);
+hipError_t launch_stage_scale(const BwdArgs& a, hipStream_t s);
+// t[r][c] *= g[0] (device scalar), in fp32; nothing is touched when g[0] == 1.  Rows on 16-byte boundaries.
+hipError_t launch_scale_rows(void* t, int dtype, int64_t rows, int64_t cols, int64_t ld, const float* g, int num_cus,
+                             hipStream_t s);
+// out[c] = rows of chunk c (of `nc` rows each) among the *n_rows packed rows: min(max(*n_rows - c * nc, 0), nc).
+hipError_t launch_chunk_rows(const int64_t* n_rows, int64_t N, int64_t nc, int chunks, int64_t* out, hipStream_t s);
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
 // dst[h][c] = 16-bit rounding of src[h * ld + v0 + c] for c < vw, 0 for vw <= c < dst_ld; h < H.
@@ -201,10 +228,10 @@ hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_ind
                                  int* perm, int64_t* yc, hipStream_t s);
 // xc[j] = x[perm[j]] for j < *n_rows, in 16-byte pieces of rows ldxc_bytes long (skipped when *n_rows == N);
 // row_bytes = bytes of a row that hold elements (nothing past them is read of the last row of x);
-// lse_c[j] = lse[perm[j]] when lse is not null (always).
+// lse_c[j] = lse[perm[j]] when lse is not null (always).  `always`: the rows are copied also when *n_rows == N.
 hipError_t launch_gather_rows(const void* x, int64_t ldx_bytes, int64_t row_bytes, const int* perm,
                               const int64_t* n_rows, int64_t N, void* xc, int64_t ldxc_bytes, const float* lse,
-                              float* lse_c, int num_cus, hipStream_t s);
+                              float* lse_c, int num_cus, hipStream_t s, bool always = false);
 // fp32 activations: xc[j] = [hi | hi | lo] of x[perm[j]] as bf16 (3 H elements per row, row stride ldxc), and
 // -- xk not null -- the same three parts stacked along the tokens, xk[b * Np + j] (row stride ldxk, rows from
 // *n_rows to Np of each block zeroed).  Always made, also when no token is dropped; perm / n_rows may be null

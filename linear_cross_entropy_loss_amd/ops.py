@@ -9,10 +9,15 @@ Mirrors the public interface of the reference's ``linear_cross_entropy/ops.py``:
   weight, no bias, ``monitoring`` / ``latest_metrics``)
 
 The device work is done by hand-written gfx950 kernels behind the C ABI of
-``liblce_gfx950.so``; torch only supplies device memory and the stream.  Unlike
-the reference, ``forward`` computes only the loss (and saves ``lse``); the
-gradients are computed in ``backward`` by recomputing logit tiles, so backward
-may run any number of times and forward-only use pays no gradient cost.
+``liblce_gfx950.so``; torch only supplies device memory and the stream.
+
+When a gradient is wanted, ``forward`` computes it along with the loss from one
+evaluation of the logits (``lce_forward_backward``), as the reference's forward
+does (``ops.py:721-791``), and ``backward`` multiplies the upstream gradient in
+(``ops.py:810``).  Problems that route does not cover (fp32 tensors, monitoring,
+shapes whose scratch bound leaves no room for it) and forward-only calls compute
+only the loss in ``forward`` and save ``lse``; their ``backward`` recomputes the
+logit tiles (``lce_backward``).  So does a second ``backward`` over the same graph.
 """
 from __future__ import annotations
 
@@ -38,6 +43,11 @@ bwd_configs: list = []
 # calling thread / task only (reset with the token it returns); the value seen by a forward call is carried
 # to its backward, which autograd may run on another thread.
 pack_rows: contextvars.ContextVar = contextvars.ContextVar("lce_pack_rows", default=_lib.PACK_AUTO)
+
+
+# Whether a forward that needs gradients computes them in the same pass over the logits (see the module
+# docstring); `one_pass.set(False)` makes every call take the loss-only forward and the recomputing backward.
+one_pass: contextvars.ContextVar = contextvars.ContextVar("lce_one_pass", default=True)
 
 
 @torch.compiler.assume_constant_result
@@ -150,6 +160,86 @@ def _check_dtypes(x, At):
             "float32 master weight under 16-bit activations (under torch.autocast the input is cast for you)")
 
 
+def _problem_views(x_in, y, At):
+    """The (x, y, w) views the kernels read, w's layout, and the shapes (N, H, V)."""
+    _check_inputs(x_in, y, At)
+    _check_dtypes(x_in, At)
+    x = _aligned_rows(x_in.reshape(-1, x_in.shape[-1]))
+    y1 = y.reshape(-1).contiguous()
+    N, H = x.shape
+    H_A, V = At.shape
+    if H_A != H:
+        raise ValueError(f"weight has in_features={H_A}, input has {H}")
+    if y1.shape != (N,):
+        raise ValueError("labels must have one entry per input row")
+    layout = _weight_layout(At, x.dtype)
+    w = _weight_rows(At, layout)
+    return x, y1, w, layout, N, H, V
+
+
+def _alloc_grads(x, w, layout, N, H, V, need_dx, need_dw):
+    vh = layout == _lib.W_VH
+    dx = _empty_rows(N, H, x.dtype, x.device) if need_dx else None
+    dw = (_empty_rows(V, H, w.dtype, x.device) if vh else _empty_rows(H, V, w.dtype, x.device)) if need_dw else None
+    return dx, dw
+
+
+def _finish_grads(dx, dw, layout):
+    if dx is not None and not dx.is_contiguous():
+        dx = dx.contiguous()  # H not a multiple of 8
+    if dw is not None and not dw.is_contiguous():
+        dw = dw.contiguous()  # V not a multiple of 8
+    if dw is not None and layout == _lib.W_VH:
+        dw = dw.t()
+    return dx, dw
+
+
+def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, pack, need_dx, need_dw):
+    """Runs lce_forward_backward with an upstream gradient of 1 when its one-pass route covers the problem.
+    Returns None otherwise, else (out5, lse, n_valid, x, y1, w, layout, dx, dw)."""
+    with torch.cuda.device(x_in.device):
+        x, y1, w, layout, N, H, V = _problem_views(x_in, y, At)
+        if x.dtype == torch.float32 or w.dtype != x.dtype:
+            return None
+        vh = layout == _lib.W_VH
+        w_cols = H if vh else V
+        prob = _lib.make_problem(
+            N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, w_cols + (-w_cols) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
+            ignore_index, logit_scale, z_regularization, N_chunk_size, False, 0, pack, 0, layout,
+        )
+        lib = _lib.load()
+        _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")
+        if _lib.forward_backward_plan(prob)[0] == 0:
+            return None
+        dev = x.device
+        dx, dw = _alloc_grads(x, w, layout, N, H, V, need_dx, need_dw)
+        nbytes = _lib.forward_backward_workspace_bytes(prob)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        lse = torch.empty(N, dtype=torch.float32, device=dev)
+        out5 = torch.empty(5, dtype=torch.float32, device=dev)
+        n_valid = torch.empty(1, dtype=torch.int64, device=dev)
+        one = torch.ones(1, dtype=torch.float32, device=dev)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = lib.lce_forward_backward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(one), _ptr(lse), _ptr(out5),
+                                      _ptr(n_valid), _ptr(dx), _ptr(dw), _ptr(ws), nbytes, ctypes.c_void_p(stream))
+        _lib.raise_for_status(rc, "lce_forward_backward")
+        del ws
+    return out5, lse, n_valid, x, y1, w, layout, dx, dw
+
+
+def _scale_grad(t, grad_output):
+    """t *= grad_output in place, the product formed in fp32 (nothing is touched when grad_output is 1)."""
+    if t is None:
+        return
+    lib = _lib.load()
+    with torch.cuda.device(t.device):
+        g = grad_output.detach().to(device=t.device, dtype=torch.float32).reshape(1).contiguous()
+        stream = torch.cuda.current_stream(t.device).cuda_stream
+        rc = lib.lce_scale(_ptr(t), _lib.dtype_code(t.dtype), t.shape[0], t.shape[1], t.stride(0), _ptr(g),
+                           ctypes.c_void_p(stream))
+        _lib.raise_for_status(rc, "lce_scale")
+
+
 def _forward_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack):
     """Runs lce_forward.  Returns (out5, lse, n_valid), the (x, y, w) views the kernels read and w's layout."""
     _check_inputs(x_in, y, At)
@@ -243,8 +333,18 @@ class LinearXentImplementation(torch.autograd.Function):
         # workspace.
         x_in = _autocast_x(x_in, At)
         pack = _pack_mode()
-        out5, lse, n_valid, x, y1, w, layout = _forward_impl(
-            x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack)
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[2]
+        done = None
+        if (need_dx or need_dw) and not monitoring and one_pass.get():
+            done = _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, pack,
+                                  need_dx, need_dw)
+        if done is not None:
+            out5, lse, n_valid, x, y1, w, layout, dx, dw = done
+            ctx.lce_grads = [dx, dw]  # for the first backward; dropped there
+        else:
+            out5, lse, n_valid, x, y1, w, layout = _forward_impl(
+                x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack)
+            ctx.lce_grads = None
         ctx.save_for_backward(x, y1, w, lse, n_valid)
         ctx.lce_cfg = (ignore_index, z_regularization, logit_scale, N_chunk_size, pack, layout)
         ctx.x_shape = x_in.shape
@@ -257,8 +357,17 @@ class LinearXentImplementation(torch.autograd.Function):
     def backward(ctx, grad_output, void0=None, void1=None, void2=None, void3=None):
         x, y1, w, lse, n_valid = ctx.saved_tensors
         ignore_index, z_regularization, logit_scale, N_chunk_size, pack, layout = ctx.lce_cfg
-        dx, dw = _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,
-                                N_chunk_size, ctx.needs_input_grad[0], ctx.needs_input_grad[2], pack, layout)
+        grads, ctx.lce_grads = ctx.lce_grads, None
+        if grads is not None:
+            # computed in the forward for an upstream gradient of 1 (ops.py:810 does the same multiplication); a
+            # later backward over the same graph finds nothing here and recomputes
+            dx, dw = grads
+            _scale_grad(dx, grad_output)
+            _scale_grad(dw, grad_output)
+            dx, dw = _finish_grads(dx, dw, layout)
+        else:
+            dx, dw = _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,
+                                    N_chunk_size, ctx.needs_input_grad[0], ctx.needs_input_grad[2], pack, layout)
         if dx is not None:
             dx = dx.view(ctx.x_shape)
         return dx, None, dw, None, None, None, None, None
@@ -352,8 +461,10 @@ def linear_cross_entropy(
     """Functional form (``ops.py:814-826``); returns ``(loss, z_reg, logit_max, logit_entropy, logit_norm)``.
 
     While ``torch.compile`` / ``torch.export`` trace, the call goes through the registered operator
-    ``torch.ops.lce_amd.forward``, so it can sit inside a compiled region; in eager mode it goes through
-    ``LinearXentImplementation`` (same device calls, bit-identical results, about 80 us less dispatch
+    ``torch.ops.lce_amd.forward`` (loss in the forward, gradients by a backward that recomputes the logit
+    tiles), so it can sit inside a compiled region; in eager mode it goes through ``LinearXentImplementation``,
+    which computes the gradients along with the loss where it can (module docstring; with ``one_pass`` off:
+    the same device calls as the registered operator, bit-identical results, about 80 us less dispatch
     overhead per forward+backward).  Under autocast ``x`` takes the weight's 16-bit dtype, or the autocast
     dtype when the weight is fp32; an fp32 weight is read as is (no 16-bit copy) and gets an fp32 gradient.
     fp32 ``x`` with an fp32 weight (no autocast) is computed as bf16 pairs, accurate to about 1e-5 of the

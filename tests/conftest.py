@@ -35,6 +35,9 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+ROUTE_MODULES = ("test_parity_gpu", "test_configs_gpu", "test_weight_layout_gpu")
+
+
 def pytest_generate_tests(metafunc):
     # GPU tests run twice: with the tokens of ignored labels packed away before the tile kernels, and
     # without (by default the library chooses by problem size, which would leave small test shapes unpacked)
@@ -42,6 +45,12 @@ def pytest_generate_tests(metafunc):
         return
     if metafunc.definition.get_closest_marker("gpu") is not None and "pack_mode" in metafunc.fixturenames:
         metafunc.parametrize("pack_mode", ["pack", "nopack"], indirect=True)
+    # The parity tests that go through autograd run on both routes: gradients from the forward's single evaluation
+    # of the logits (the default where the problem allows it), and the loss-only forward with a backward that
+    # recomputes the logit tiles.
+    if (metafunc.definition.get_closest_marker("gpu") is not None and "route" in metafunc.fixturenames
+            and metafunc.module.__name__ in ROUTE_MODULES):
+        metafunc.parametrize("route", ["one_pass", "two_pass"], indirect=True)
 
 
 @pytest.fixture(autouse=True)
@@ -55,3 +64,16 @@ def pack_mode(request):
     token = ops.pack_rows.set(_lib.PACK_ALWAYS if mode == "pack" else _lib.PACK_NEVER)
     yield mode
     ops.pack_rows.reset(token)  # (also undoes whatever the test itself set in between)
+
+
+@pytest.fixture(autouse=True)
+def route(request):
+    mode = getattr(request, "param", None)
+    if mode is None:
+        yield None
+        return
+    from linear_cross_entropy_loss_amd import ops
+
+    token = ops.one_pass.set(mode == "one_pass")
+    yield mode
+    ops.one_pass.reset(token)

@@ -456,3 +456,43 @@ def test_a_weight_that_cannot_be_read_in_place_is_copied_with_one_warning():
     with warnings.catch_warnings():
         warnings.simplefilter("error")
         ops._weight_rows(bad, ops._weight_layout(bad, torch.bfloat16))  # the second copy is silent
+
+
+def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
+    """lce_forward_backward_plan: chunks of whole token tiles that cover N, a workspace within n_chunk * V * 4
+    bytes, and no one-pass route for fp32 tensors, monitoring, or a bound that the fp32 plane of dW alone fills."""
+    import random
+
+    from linear_cross_entropy_loss_amd import _lib
+
+    rng = random.Random(5)
+    took = 0
+    for _ in range(300):
+        N = rng.choice([1, 255, 256, 1000, 4096, 16384, 65536, 100000])
+        H = rng.choice([64, 520, 2048, 4096, 8192])
+        V = rng.choice([777, 4096, 32768, 131072, 262144])
+        n_chunk = rng.choice([256, 1024, 4096, 8192, 32768])
+        dt = rng.choice([torch.bfloat16, torch.float16])
+        prob = _lib.make_problem(N, H, V, H + (-H) % 8, V + (-V) % 8, H + (-H) % 8, V + (-V) % 8, dt, dt, dt, dt, -1, 1.0,
+                                 0.0, n_chunk, False)
+        chunks, rows = _lib.forward_backward_plan(prob)
+        total = _lib.forward_backward_workspace_bytes(prob)
+        if chunks == 0:
+            assert total == max(_lib.workspace_bytes(prob))
+            continue
+        took += 1
+        assert rows % 256 == 0 and rows > 0
+        assert chunks * rows >= N and (chunks - 1) * rows < N + 255
+        assert total <= n_chunk * V * 4, (N, H, V, n_chunk, total)
+        if chunks > 1:  # the plane is part of it
+            assert total >= (H + (-H) % 256) * (V + (-V) % 256) * 4
+    assert took > 50
+    # the benchmark's default shape: five chunks of 13 token tiles
+    prob = _lib.make_problem(16384, 2048, 131072, 2048, 131072, 2048, 131072, torch.bfloat16, torch.bfloat16,
+                             torch.bfloat16, torch.bfloat16, -1, 1.0, 0.0, 4096, False)
+    assert _lib.forward_backward_plan(prob) == (5, 3328)
+    for kw in (dict(x=torch.float32, w=torch.float32), dict(x=torch.bfloat16, w=torch.float32), dict(mon=True)):
+        xd, wd = kw.get("x", torch.bfloat16), kw.get("w", torch.bfloat16)
+        prob = _lib.make_problem(4096, 512, 8192, 512, 8192, 512, 8192, xd, wd, xd, wd, -1, 1.0, 0.0, 4096,
+                                 kw.get("mon", False))
+        assert _lib.forward_backward_plan(prob) == (0, 0), kw

@@ -1,0 +1,225 @@
+"""lce_forward_backward: loss and gradients from one evaluation of the logits, through the C ABI.
+
+Checked against the fp64 oracle to the operator's tolerances (loss 1e-3, gradients 2e-2) and against lce_forward +
+lce_backward on the same inputs: lse and loss to fp32 rounding (both sum the same fp32 logits, in another order),
+the gradients to the second rounding of the staged dz (16-bit: 2^-8 relative per element before the contraction).
+"""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import make_inputs, rel_errors
+
+pytestmark = pytest.mark.gpu
+
+
+def P(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _problem(N, H, V, x, w, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, phases=0):
+    from linear_cross_entropy_loss_amd import _lib
+
+    hp, cols = H + (-H) % 8, (H if layout else V)
+    return _lib.make_problem(N, H, V, x.stride(0), w.stride(0), hp, cols + (-cols) % 8, dt, dt, dt, dw_dt, -1, scale,
+                             z_reg, n_chunk, False, phases, pack, 0, layout)
+
+
+def _both_routes(N, H, V, dt, n_chunk, ignore, z_reg=0.0, scale=1.0, pack=0, layout=0, dw_dt=None, grad_out=1.0,
+                 seed=7, want_chunks=None):
+    """Runs the two routes on the same inputs; returns (inputs on the CPU, two-pass outputs, one-pass outputs)."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    lib = _lib.load()
+    x, y, w = make_inputs(N, H, V, dt, seed, ignore_frac=ignore)
+    xd, yd, wd = x.cuda(), y.cuda(), (w.t().contiguous() if layout else w).cuda()
+    if wd.stride(0) % 8:  # rows of the weight on 16-byte boundaries
+        pad = torch.zeros(wd.shape[0], wd.shape[1] + (-wd.shape[1]) % 8, dtype=wd.dtype, device="cuda")
+        pad[:, :wd.shape[1]] = wd
+        wd = pad[:, :wd.shape[1]]
+    if xd.stride(0) % 8:
+        pad = torch.zeros(N, H + (-H) % 8, dtype=xd.dtype, device="cuda")
+        pad[:, :H] = xd
+        xd = pad[:, :H]
+    dw_dt = dw_dt or dt
+    prob = _problem(N, H, V, xd, wd, dt, dw_dt, z_reg, scale, n_chunk, pack, layout)
+    chunks, rows = _lib.forward_backward_plan(prob)
+    print(f"N={N} H={H} V={V} {dt} n_chunk={n_chunk} pack={pack} layout={layout}: {chunks} chunks of {rows} rows", flush=True)
+    assert chunks > 0, "this case is meant to take the one-pass route"
+    if want_chunks is not None:
+        assert chunks >= want_chunks
+    fb, bb = _lib.workspace_bytes(prob)
+    ub = _lib.forward_backward_workspace_bytes(prob)
+    ws = torch.empty(max(fb, bb, ub), dtype=torch.uint8, device="cuda")
+    g = torch.full((1,), grad_out, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    hp = H + (-H) % 8
+
+    def outs():
+        shape = (V, hp) if layout else (H, V + (-V) % 8)
+        return dict(lse=torch.full((N,), 7.0, device="cuda"), out5=torch.zeros(5, device="cuda"),
+                    nv=torch.zeros(1, dtype=torch.int64, device="cuda"),
+                    dx=torch.full((N, hp), 3.0, dtype=dt, device="cuda"), dw=torch.full(shape, 3.0, dtype=dw_dt, device="cuda"))
+
+    a, b = outs(), outs()
+    rc = lib.lce_forward(ctypes.byref(prob), P(xd), P(wd), P(yd), P(a["lse"]), P(a["out5"]), P(a["nv"]), P(ws), ws.numel(), st)
+    assert rc == 0
+    rc = lib.lce_backward(ctypes.byref(prob), P(xd), P(wd), P(yd), P(a["lse"]), P(a["nv"]), P(g), P(a["dx"]), P(a["dw"]),
+                          P(ws), ws.numel(), st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ws.fill_(0x5a)  # nothing in the workspace has to start at any value
+    rc = lib.lce_forward_backward(ctypes.byref(prob), P(xd), P(wd), P(yd), P(g), P(b["lse"]), P(b["out5"]), P(b["nv"]),
+                                  P(b["dx"]), P(b["dw"]), P(ws), ub, st)
+    assert rc == 0, (rc, lib.lce_last_hip_error())
+    torch.cuda.synchronize()
+    for o in (a, b):
+        o["dx"] = o["dx"][:, :H]
+        o["dw"] = o["dw"][:, :H].t() if layout else o["dw"][:, :V]
+    return (x, y, w), a, b
+
+
+def _check(inputs, a, b, z_reg, scale, grad_out=1.0, fp64=True):
+    x, y, w = inputs
+    assert a["nv"].item() == b["nv"].item() == int((y != -1).sum())
+    # the same fp32 logits summed in another order
+    assert abs(a["out5"][0].item() - b["out5"][0].item()) <= 2e-6 * abs(a["out5"][0].item())
+    assert abs(a["out5"][1].item() - b["out5"][1].item()) <= 4e-6 * abs(a["out5"][1].item()) + 1e-12
+    assert rel_errors(b["lse"], a["lse"])[0] <= 1e-6
+    assert (b["lse"].cpu()[y == -1] == 0).all()
+    # ignored tokens: exact zeros
+    assert (b["dx"].cpu()[y == -1] == 0).all()
+    for name in ("dx", "dw"):
+        emax, el2 = rel_errors(b[name], a[name])
+        print(f"  {name} one-pass vs two-pass: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
+        assert emax <= 1.5e-2 and el2 <= 3e-3, (name, emax, el2)
+    if fp64:
+        from oracle import lce_forward_backward_fp64
+
+        ref = lce_forward_backward_fp64(x.double(), y, w.double(), -1, z_reg, scale, grad_out)
+        assert abs(b["out5"][0].item() - ref.loss.item()) <= 1e-3 * abs(ref.loss.item())
+        for name, want in (("dx", ref.dx), ("dw", ref.dw)):
+            emax, el2 = rel_errors(b[name], want)
+            print(f"  {name} one-pass vs fp64: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
+            assert emax <= 2e-2 and el2 <= 2e-2, (name, emax, el2)
+
+
+CASES = [
+    # N, H, V, dtype, n_chunk, ignored, z_reg, scale, pack, layout, dW dtype, grad_out
+    (4096, 512, 4096, torch.bfloat16, 1024, 0.1, 0.0, 1.0, 2, 0, None, 1.0),        # 16 chunks, all rows computed
+    (4096, 512, 4096, torch.bfloat16, 2048, 0.1, 0.0, 1.0, 1, 0, None, 1.0),        # packed rows, several chunks
+    (4000, 520, 5000, torch.float16, 2048, 0.1, 1e-3, 0.7, 1, 0, None, 0.37),       # ragged shapes, fp16, z-reg
+    (4000, 520, 5000, torch.bfloat16, 1200, 0.1, 0.0, 1.0, 2, 1, None, 1.0),        # weight stored (V, H)
+    (4000, 520, 5000, torch.bfloat16, 2048, 0.1, 1e-4, 1.0, 1, 1, None, 2.5),       # (V, H), packed
+    (4000, 520, 5000, torch.bfloat16, 2048, 0.7, 0.0, 1.0, 1, 0, torch.float32, 1.0),   # chunks without a row; fp32 dW
+    (2048, 1024, 8192, torch.bfloat16, 4096, 0.0, 0.0, 1.0, 0, 0, torch.float32, 1.0),  # a single chunk: no plane
+    (1000, 300, 777, torch.float16, 4096, 0.2, 0.0, 2.0, 1, 0, None, 1.0),          # single chunk, nothing a multiple of 8
+    (8192, 1024, 32768, torch.bfloat16, 4096, 0.05, 0.0, 1.0, 0, 0, None, 1.0),     # mid size: 3 chunks
+]
+
+
+@pytest.mark.pack_auto
+@pytest.mark.parametrize("N,H,V,dt,n_chunk,ign,z_reg,scale,pack,layout,dw_dt,grad_out", CASES)
+def test_one_pass_matches_two_pass_and_the_fp64_oracle(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout, dw_dt, grad_out):
+    inputs, a, b = _both_routes(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout, dw_dt, grad_out)
+    _check(inputs, a, b, z_reg, scale, grad_out, fp64=N * V <= 4096 * 8192)
+
+
+@pytest.mark.pack_auto
+def test_fp16_z_regularisation_with_lse_near_a_thousand_on_the_one_pass_route():
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    N, H, V = 1024, 256, 4096
+    x, y, w = make_inputs(N, H, V, torch.float16, seed=11, ignore_frac=0.1)
+    xd, wd = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    out = linear_cross_entropy(xd, y.cuda(), wd, -1, 0.03, 205.0, 4096, False)
+    out[0].backward()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out[0]) and torch.isfinite(xd.grad).all() and torch.isfinite(wd.grad).all()
+    from oracle import lce_forward_backward_fp64
+
+    ref = lce_forward_backward_fp64(x.double(), y, w.double(), -1, 0.03, 205.0, 1.0)
+    assert abs(out[0].item() - ref.loss.item()) <= 1e-3 * abs(ref.loss.item())
+    assert max(rel_errors(xd.grad, ref.dx)) <= 2e-2 and max(rel_errors(wd.grad, ref.dw)) <= 2e-2
+
+
+@pytest.mark.pack_auto
+def test_a_second_backward_recomputes_and_the_upstream_gradient_is_multiplied_in_fp32():
+    from linear_cross_entropy_loss_amd import linear_cross_entropy
+
+    N, H, V = 2048, 512, 8192
+    x, y, w = make_inputs(N, H, V, torch.bfloat16, seed=5, ignore_frac=0.1)
+    xd, wd = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    loss = linear_cross_entropy(xd, y.cuda(), wd, -1, 0.0, 1.0, 4096, False)[0]
+    g = 1.0 / 3.0
+    (loss * g).backward(retain_graph=True)
+    first = (xd.grad.clone(), wd.grad.clone())
+    xd.grad = wd.grad = None
+    (loss * g).backward()  # nothing is left from the forward: the logit tiles are recomputed
+    torch.cuda.synchronize()
+    from oracle import lce_forward_backward_fp64
+
+    ref = lce_forward_backward_fp64(x.double(), y, w.double(), -1, 0.0, 1.0, g)
+    for got in (first, (xd.grad, wd.grad)):
+        assert max(rel_errors(got[0], ref.dx)) <= 2e-2 and max(rel_errors(got[1], ref.dw)) <= 2e-2
+    assert max(rel_errors(first[0], xd.grad)) <= 1.5e-2 and max(rel_errors(first[1], wd.grad)) <= 1.5e-2
+    # the factor is not rounded to 16 bits before it is applied: the sum of dW follows it to 1e-3
+    ones = lce_forward_backward_fp64(x.double(), y, w.double(), -1, 0.0, 1.0, 1.0)
+    ratio = (first[1].double().cpu() * ones.dw).sum() / (ones.dw * ones.dw).sum()
+    assert abs(ratio.item() - g) <= 1e-3 * g
+
+
+@pytest.mark.pack_auto
+def test_scale_with_a_factor_of_one_touches_nothing_and_other_factors_round_once():
+    from linear_cross_entropy_loss_amd import _lib
+
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for dt in (torch.bfloat16, torch.float16, torch.float32):
+        m = 4 if dt == torch.float32 else 8
+        t = torch.randn(37, 104 + m, device="cuda").to(dt)
+        view = t[:, :101]  # the last piece of a row is cut
+        before = t.clone()
+        one = torch.ones(1, device="cuda")
+        assert lib.lce_scale(P(view), _lib.dtype_code(dt), 37, 101, t.stride(0), P(one), st) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(t, before)
+        f = torch.full((1,), 1.0 / 3.0, device="cuda")
+        assert lib.lce_scale(P(view), _lib.dtype_code(dt), 37, 101, t.stride(0), P(f), st) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(t[:, :101], (before[:, :101].float() * f).to(dt))
+        assert torch.equal(t[:, 101:], before[:, 101:])  # nothing past the columns
+    assert lib.lce_scale(P(view), 7, 37, 101, t.stride(0), P(one), st) == _lib.LCE_EINVAL_DTYPE
+    assert lib.lce_scale(P(view), _lib.LCE_F32, 37, 101, 50, P(one), st) == _lib.LCE_EINVAL_ARG
+
+
+@pytest.mark.pack_auto
+def test_problems_outside_the_one_pass_route_take_the_two_calls_inside_the_entry_point():
+    """fp32 activations: lce_forward_backward runs lce_forward and lce_backward itself, bit for bit."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    lib = _lib.load()
+    N, H, V = 512, 256, 4096
+    x, y, w = make_inputs(N, H, V, torch.float32, seed=3, ignore_frac=0.1, device="cuda")
+    prob = _lib.make_problem(N, H, V, H, V, H, V, torch.float32, torch.float32, torch.float32, torch.float32, -1, 1.0, 0.0,
+                             512, False)
+    assert _lib.forward_backward_plan(prob) == (0, 0)
+    fb, bb = _lib.workspace_bytes(prob)
+    ub = _lib.forward_backward_workspace_bytes(prob)
+    assert ub == max(fb, bb)
+    ws = torch.empty(ub, dtype=torch.uint8, device="cuda")
+    g = torch.ones(1, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    outs = lambda: dict(lse=torch.zeros(N, device="cuda"), out5=torch.zeros(5, device="cuda"),
+                        nv=torch.zeros(1, dtype=torch.int64, device="cuda"), dx=torch.zeros(N, H, device="cuda"),
+                        dw=torch.zeros(H, V, device="cuda"))
+    a, b = outs(), outs()
+    assert lib.lce_forward(ctypes.byref(prob), P(x), P(w), P(y), P(a["lse"]), P(a["out5"]), P(a["nv"]), P(ws), ub, st) == 0
+    assert lib.lce_backward(ctypes.byref(prob), P(x), P(w), P(y), P(a["lse"]), P(a["nv"]), P(g), P(a["dx"]), P(a["dw"]),
+                            P(ws), ub, st) == 0
+    assert lib.lce_forward_backward(ctypes.byref(prob), P(x), P(w), P(y), P(g), P(b["lse"]), P(b["out5"]), P(b["nv"]),
+                                    P(b["dx"]), P(b["dw"]), P(ws), ub, st) == 0
+    torch.cuda.synchronize()
+    for k in a:
+        assert torch.equal(a[k], b[k]), k
