@@ -182,6 +182,25 @@ size_t dw_part_bytes(size_t Np, size_t Hp, int64_t vs, int64_t last_vs) {
   return (size_t)(b0 > b1 ? b0 : b1) * 256 * 256 * 4;
 }
 
+// Modelled time of a tile kernel with T output tiles of L K tiles each, in units of one 64-deep K tile of a 256 x 256
+// output tile on a full chip.  A kernel runs its tiles in rounds of kPlanCUs; a last round that fills a
+// fraction f of the compute units runs 1 + 0.9 (1 - f) times faster per compute unit (the part is limited by
+// power: measured 1.14 / 1.30 / 1.46 / 1.54 at f = 0.81 / 0.69 / 0.47 / 0.34), and is cut along K when the
+// partial-sum blocks exist (`parts`; a small kernel then adds the segments: 12 units).  `e`: the epilogue of a
+// tile; a launch costs about 10.
+constexpr double kPlanCUs = 256.0;
+double kernel_cost(double T, double L, double e, bool parts) {
+  const double full = (double)(int64_t)(T / kPlanCUs), r = T - full * kPlanCUs;
+  double cost = full * (L + e) + 10.0;
+  if (r > 0) {
+    double seg = 1;
+    if (parts) while (r * seg * 2 <= kPlanCUs && L / (seg * 2) >= 16) seg *= 2;
+    const double f = r * seg / kPlanCUs;
+    cost += (L / seg + e) / (1.0 + 0.9 * (1.0 - f)) + (seg > 1 ? 12.0 : 0.0);
+  }
+  return cost;
+}
+
 // Vocabulary slabs (of a width that is a multiple of 256 columns; the last one may be narrower) whose staging
 // fits the scratch bound: the fewest that fit, or somewhat more of them when a model of the three kernels'
 // rounds of workgroups says that those run faster (slab_cost below).  The dz stage itself is additionally
@@ -211,29 +230,13 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   b->lse_c = b->pack.end;
   b->dxc = b->lse_c + align_up((size_t)p->N * 4);
 
-  // Modelled time of the three kernels over one slab of `w` columns, in units of one 64-deep K tile of a 256 x 256
-  // output tile on a full chip.  A kernel runs its T tiles in rounds of kPlanCUs; a last round that fills a
-  // fraction f of the compute units runs 1 + 0.9 (1 - f) times faster per compute unit (the part is limited by
-  // power: measured 1.14 / 1.30 / 1.46 / 1.54 at f = 0.81 / 0.69 / 0.47 / 0.34), and is cut along K when the
-  // partial-sum blocks exist (`parts`; a small kernel then adds the segments: 12 units).  Per tile, the epilogues
+  // Modelled time of the three kernels over one slab of `w` columns (kernel_cost above).  Per tile, the epilogues
   // cost about 6 (dz), 21 (dx adding into the fp32 running sum: 512 KiB of traffic at a compute unit's share of the
-  // memory bandwidth; 5 when it is written once) and 5 (dW) units; a launch about 10.  The model ranks the slab
+  // memory bandwidth; 5 when it is written once) and 5 (dW) units.  The model ranks the slab
   // widths measured at N = 16384, H = 2048, V = 32768 and 65536 (2 ... 18 slabs) in their measured order.
-  constexpr double kPlanCUs = 256.0;
   // bands of W tiles that bwd_dz keeps in flight (tile_coords in lce_gemm.h), and the slab width that is a whole group of them
   const int live = lce::live_bands(lce::padded_k(split ? 3 * p->H : p->H) * 2);
   const int64_t gran = live < 8 ? (int64_t)256 * 8 * live : 256;
-  auto kernel_cost = [&](double T, double L, double e, bool parts) -> double {
-    const double full = (double)(int64_t)(T / kPlanCUs), r = T - full * kPlanCUs;
-    double cost = full * (L + e) + 10.0;
-    if (r > 0) {
-      double seg = 1;
-      if (parts) while (r * seg * 2 <= kPlanCUs && L / (seg * 2) >= 16) seg *= 2;
-      const double f = r * seg / kPlanCUs;
-      cost += (L / seg + e) / (1.0 + 0.9 * (1.0 - f)) + (seg > 1 ? 12.0 : 0.0);
-    }
-    return cost;
-  };
   auto slab_cost = [&](int64_t w, bool parts, bool sums) -> double {
     const double tq = (double)(Np / 256), th = (double)(Hp / 256), tv = (double)(w / 256), k3 = split ? 3.0 : 1.0;
     // (bwd_dz runs about 4 % slower on a slab that is not whole groups of the bands it keeps in flight when K is long)
@@ -368,19 +371,40 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     out->total = t;
     return t;
   };
-  // one chunk if it fits; else the fewest chunks of equal length that do
+  // Chunks of equal length (whole token tiles): of the lengths that fit, the one for which a model of the three tile
+  // kernels' rounds of workgroups gives the shortest time -- not always the longest: at the headline shape 13
+  // token tiles fit, whose 104 tiles of dx fill 208 of 256 compute units when each is cut in two along K, while
+  // chunks of 8 token tiles (64 tiles of dx, cut in four) fill them all -- but the part is limited by power, the
+  // partly filled rounds run at a higher clock, and the longer chunk wins: measured 22.07 ms a step with 13 token
+  // tiles, 22.60 with 8, 22.85 with 11, 23.87 with 7, 26.1 with 4, the order the model gives.
   const int64_t tiles = (int64_t)(Np / 256);
-  for (int chunks = 1; chunks <= tiles && chunks <= 1024; ++chunks) {
-    const int64_t nc = (tiles + chunks - 1) / chunks * 256;
-    if ((nc * (chunks - 1)) >= (int64_t)Np) continue;  // the same chunk length as with one chunk fewer
-    if (total_for(nc, chunks, f) + reserve <= bound) {
-      f->nc = nc;
-      f->chunks = (int)(((int64_t)Np + nc - 1) / nc);
+  const double th = (double)(Hp / 256), tv = (double)(Vp / 256);
+  double best = 0;
+  int64_t first = 0;  // chunks of the longest chunk that fits
+  for (int64_t t = tiles; t >= 1; --t) {
+    const int64_t chunks = (tiles + t - 1) / t;
+    if (chunks > 1024 || (first != 0 && chunks > 4 * first + 8)) break;
+    if (t < tiles && (tiles + t) / (t + 1) == chunks) continue;  // a longer chunk gives the same number of chunks
+    const int64_t t_even = (tiles + chunks - 1) / chunks;  // equal lengths
+    FusedPlan cand = *f;
+    if (total_for(t_even * 256, (int)chunks, &cand) + reserve > bound) continue;
+    const int64_t t_last = tiles - (chunks - 1) * t_even;
+    auto chunk_cost = [&](double tt) -> double {
+      return kernel_cost(tt * tv, (double)(lce::padded_k(p->H) / 64), 8.0, false) +
+             (want_dx ? kernel_cost(tt * th, (double)(Vp / 64), 5.0, true) : 0.0) +
+             (want_dw ? kernel_cost(tv * th, tt * 4.0, chunks > 1 ? 12.0 : 5.0, chunks == 1) : 0.0);
+    };
+    const double cost = (double)(chunks - 1) * chunk_cost((double)t_even) + chunk_cost((double)t_last);
+    if (first == 0) first = chunks;
+    if (!f->ok || cost < best) {
+      best = cost;
+      *f = cand;
+      f->nc = t_even * 256;
+      f->chunks = (int)chunks;
       f->ok = true;
-      return true;
     }
   }
-  return false;
+  return f->ok;
 }
 
 bool misaligned(const void* p) { return ((uintptr_t)p & 15) != 0; }

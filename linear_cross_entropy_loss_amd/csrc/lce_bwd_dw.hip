@@ -192,7 +192,8 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
 // as the registers do -- quad (rb, cbk, rq) of thread t at float 4 * (((rb * 4 + cbk) * 4 + rq) * 256 + t) -- so
 // that every load and store of a wave covers 1 KiB of consecutive addresses.  LOAD: the block is added to the
 // accumulator before the sums go (back) to the block.  After the last chunk dw_plane_out_kernel scales the sums
-// and stores dW.
+// and stores dW.  (Hardware fp32 atomic adds instead of the load - add - store were measured at the headline shape:
+// the 268 M atomics of a chunk take longer than the chunk's matrix work, 30.6 ms a step against 22.3.)
 // The four quads of an accumulator block are fetched together before any is used.
 template <bool LOAD>
 LCE_DEV void dw_plane_io(float* blk, f32x16_t (&acc)[kNB][kNB]) {
@@ -405,11 +406,19 @@ template <class T, bool WVH, int MODE, int ACC = 0> hipError_t launch_tiles(cons
   return hipGetLastError();
 }
 
-// The plane of sums over chunks of token rows becomes dW: one workgroup per tile, thread t takes the quads that
-// thread t of the tile kernel stored (dw_plane_io) and puts them where dw_epilogue would have.
-template <class T, bool WVH>
+// The plane of sums over chunks of token rows becomes dW: one workgroup per tile, each wave on the 128 x 128
+// sub-tile whose quads its threads stored (dw_plane_io).  A wave takes 32 rows of the stored matrix at a time, 256
+// bytes of each (128 columns of 16-bit data, 64 of fp32): the quads come in as they lie in the plane (1 KiB per
+// load), are scaled, rounded and written to the wave's slice of LDS where dw_epilogue would have put them in
+// memory, and leave as whole 256-byte rows, four rows per store instruction.  (Rows of the slice are 272 bytes
+// apart: 16-byte pieces stay aligned, and lanes on consecutive rows use different banks.)
+template <class T, bool WVH, bool F32OUT>
 __global__ __launch_bounds__(256) void dw_plane_out_kernel(const BwdArgs a) {
   typedef typename elem_of<T>::type E;
+  typedef typename std::conditional<F32OUT, float, E>::type O;
+  constexpr int kPassCols = F32OUT ? 64 : 128, kPassBlocks = kPassCols / kBlk, kPieceCols = 16 / (int)sizeof(O);
+  constexpr int kRowBytes = 256 + 16;
+  __shared__ __attribute__((aligned(16))) char sh[4][kBlk * kRowBytes];
   const int tiles_p = (int)(a.Hp / kTile);
   const int tq = (int)blockIdx.x / tiles_p, tp = (int)blockIdx.x % tiles_p;
   const DwTileGeom<WVH> g(a, tp, tq);
@@ -418,30 +427,53 @@ __global__ __launch_bounds__(256) void dw_plane_out_kernel(const BwdArgs a) {
   const int wp = wave & 1, wq = wave >> 1, half = lane >> 5;
   const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
   const float* mine = a.dw_plane + (int64_t)blockIdx.x * (kTile * kTile) + threadIdx.x * 4;
-#pragma unroll 4
-  for (int q = 0; q < 64; ++q) {
-    const int i = q >> 4, k = (q >> 2) & 3, rq = q & 3;  // quad rq of acc[i][k]
-    const int rb = WVH ? k : i, cbk = WVH ? i : k;
-    const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + (lane & 31);
-    const int64_t col = g.col0 + w_col * kWaveTile + cbk * kBlk + 8 * rq + 4 * half;
-    const f32x4_t v = *reinterpret_cast<const f32x4_t*>(mine + q * 1024) * coef;
-    if (row >= g.row_limit || col >= g.col_limit) continue;  // a quad that the last column cuts through is written whole, into the stride padding of its row
-    if (a.dw_dtype == DT_F32) {
-      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.dw) + row * a.lddw + col) = v;
-    } else {
-      u32x2_t o;
-      o[0] = pack2<T>(v[0], v[1]);
-      o[1] = pack2<T>(v[2], v[3]);
-      *reinterpret_cast<u32x2_t*>(reinterpret_cast<E*>(a.dw) + row * a.lddw + col) = o;
+  char* my = sh[wave];
+  O* out = reinterpret_cast<O*>(a.dw);
+#pragma unroll 1
+  for (int rb = 0; rb < kNB; ++rb)
+#pragma unroll 1
+    for (int cp = 0; cp < kNB / kPassBlocks; ++cp) {
+#pragma unroll
+      for (int cb = 0; cb < kPassBlocks; ++cb) {
+        const int cbk = cp * kPassBlocks + cb;
+        const int i = WVH ? cbk : rb, k = WVH ? rb : cbk;  // the block is acc[i][k] of the tile kernel
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const f32x4_t v = *reinterpret_cast<const f32x4_t*>(mine + ((i * 4 + k) * 4 + rq) * 1024) * coef;
+          char* at = my + (lane & 31) * kRowBytes + (cb * kBlk + 8 * rq + 4 * half) * (int)sizeof(O);
+          if (F32OUT) {
+            *reinterpret_cast<f32x4_t*>(at) = v;
+          } else {
+            u32x2_t o;
+            o[0] = pack2<T>(v[0], v[1]);
+            o[1] = pack2<T>(v[2], v[3]);
+            *reinterpret_cast<u32x2_t*>(at) = o;
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int r = it * 4 + (lane >> 4), piece = lane & 15;
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(my + r * kRowBytes + piece * 16);
+        const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + r;
+        const int64_t col = g.col0 + w_col * kWaveTile + cp * kPassCols + piece * kPieceCols;
+        // pieces that start at or past the last column are not stored; one that it cuts through is written whole,
+        // into the stride padding of its row
+        if (row < g.row_limit && col < g.col_limit)
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + row * a.lddw + col));
+      }
+      __builtin_amdgcn_wave_barrier();
     }
-  }
 }
 
 // Whole tiles that meet the plane of sums over chunks of token rows (nothing is split along K then).
 template <class T, bool WVH, int MODE> hipError_t launch_plane(const BwdArgs& a, hipStream_t s) {
   hipError_t e = a.dw_acc == 1 ? launch_tiles<T, WVH, MODE, 1>(a, s) : launch_tiles<T, WVH, MODE, 2>(a, s);
   if (e != hipSuccess || !a.last_chunk) return e;
-  hipLaunchKernelGGL((dw_plane_out_kernel<T, WVH>), dim3((unsigned)((a.vs / kTile) * (a.Hp / kTile))), dim3(256), 0, s, a);
+  const dim3 grid((unsigned)((a.vs / kTile) * (a.Hp / kTile)));
+  if (a.dw_dtype == DT_F32) hipLaunchKernelGGL((dw_plane_out_kernel<T, WVH, true>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((dw_plane_out_kernel<T, WVH, false>), grid, dim3(256), 0, s, a);
   return hipGetLastError();
 }
 
