@@ -91,7 +91,7 @@ typedef struct lce_problem {
   int32_t pack_rows;    /* LCE_PACK_AUTO | LCE_PACK_ALWAYS | LCE_PACK_NEVER: see below        */
   int32_t max_workgroups; /* profiling aid: cap on the persistent workgroups of the tile kernels (0 = one per compute unit) */
   int32_t w_layout;     /* LCE_W_HV (0) | LCE_W_VH: how w and dw are stored, see below */
-  int32_t reserved;     /* 0 */
+  int32_t route;        /* lce_forward_backward only: LCE_ROUTE_AUTO (0) | LCE_ROUTE_ONE_PASS | LCE_ROUTE_TWO_PASS, see there */
 } lce_problem;
 
 /*
@@ -261,6 +261,12 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
                  const float* lse, const int64_t* n_valid, const float* grad_out,
                  void* dx, void* dw, void* ws, size_t ws_bytes, void* stream);
 
+enum {
+  LCE_ROUTE_AUTO = 0,
+  LCE_ROUTE_ONE_PASS = 1,
+  LCE_ROUTE_TWO_PASS = 2
+};
+
 /*
  * Forward and backward in one call, from ONE evaluation of the logits.
  * Replaces LinearXentImplementation.forward as the reference runs it when a
@@ -280,6 +286,12 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
  * (the reference's fp32 At_grad, ops.py:692; no plane with a single chunk).
  * The chunk is the longest for which all of it stays within n_chunk * V * 4
  * bytes.  8*N*H*V FLOPs become 6*N*H*V.
+ *
+ * lce_problem.route: LCE_ROUTE_AUTO takes this route when a model of the tile
+ * kernels' rounds of workgroups says it is the faster one (short chunks are
+ * not: every chunk costs a round trip of the whole plane, so small problems
+ * and tight bounds take two passes); LCE_ROUTE_ONE_PASS takes it whenever it
+ * fits the bound; LCE_ROUTE_TWO_PASS never.
  *
  * Problems this route does not cover take the two calls above, one after the
  * other on the same workspace, inside this entry point: fp32 activations, a

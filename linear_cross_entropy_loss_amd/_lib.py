@@ -13,6 +13,7 @@ LCE_BF16, LCE_F16, LCE_F32 = 0, 1, 2
 LCE_OK = 0
 PHASE_FWD_TILES, PHASE_FWD_REDUCE, PHASE_BWD_DZ, PHASE_BWD_DX, PHASE_BWD_DW, PHASE_PACK = 1, 2, 4, 8, 16, 32
 PACK_AUTO, PACK_ALWAYS, PACK_NEVER = 0, 1, 2
+ROUTE_AUTO, ROUTE_ONE_PASS, ROUTE_TWO_PASS = 0, 1, 2  # lce_problem.route (lce_forward_backward)
 W_HV, W_VH = 0, 1  # lce_problem.w_layout: weight stored (H, V) / (V, H) row-major
 LCE_EINVAL_SHAPE, LCE_EINVAL_DTYPE, LCE_EINVAL_ARG, LCE_EWORKSPACE, LCE_EHIP, LCE_ESTATIC = -1, -2, -3, -4, -5, -6
 STATIC_SCRATCH_BYTES = 64 << 20
@@ -60,7 +61,7 @@ class LceProblem(ctypes.Structure):
         ("pack_rows", ctypes.c_int32),
         ("max_workgroups", ctypes.c_int32),
         ("w_layout", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("route", ctypes.c_int32),
     ]
 
 
@@ -136,14 +137,14 @@ def raise_for_status(rc: int, what: str) -> None:
 
 def make_problem(N, H, V, ldx, ldw, lddx, lddw, x_dtype, w_dtype, dx_dtype, dw_dtype, ignore_index,
                  logit_scale, z_reg, n_chunk, monitoring, phases=0, pack_rows=0, max_workgroups=0,
-                 w_layout=0) -> LceProblem:
+                 w_layout=0, route=0) -> LceProblem:
     return LceProblem(
         N=N, H=H, V=V, ldx=ldx, ldw=ldw, lddx=lddx, lddw=lddw,
         x_dtype=dtype_code(x_dtype), w_dtype=dtype_code(w_dtype),
         dx_dtype=dtype_code(dx_dtype), dw_dtype=dtype_code(dw_dtype),
         ignore_index=int(ignore_index), logit_scale=float(logit_scale), z_reg=float(z_reg),
         n_chunk=int(n_chunk), monitoring=1 if monitoring else 0, phases=int(phases), pack_rows=int(pack_rows),
-        max_workgroups=int(max_workgroups), w_layout=int(w_layout), reserved=0,
+        max_workgroups=int(max_workgroups), w_layout=int(w_layout), route=int(route),
     )
 
 

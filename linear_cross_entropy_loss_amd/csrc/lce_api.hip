@@ -39,6 +39,7 @@ int check(const lce_problem* p, bool backward) {
   if (p->pack_rows != LCE_PACK_AUTO && p->pack_rows != LCE_PACK_ALWAYS && p->pack_rows != LCE_PACK_NEVER) return LCE_EINVAL_ARG;
   if (p->max_workgroups < 0) return LCE_EINVAL_ARG;
   if (p->w_layout != LCE_W_HV && p->w_layout != LCE_W_VH) return LCE_EINVAL_ARG;
+  if (p->route != LCE_ROUTE_AUTO && p->route != LCE_ROUTE_ONE_PASS && p->route != LCE_ROUTE_TWO_PASS) return LCE_EINVAL_ARG;
   const bool vh = p->w_layout == LCE_W_VH;
   // (V, H) weight: both operands of the logit contraction run along H in memory, so no 16-byte piece may
   // straddle the end of a row (H a multiple of 8), and there is no bf16-pair form of it
@@ -161,6 +162,7 @@ FwdPlan plan_fwd(const lce_problem* p) {
 
 struct BwdPlan {
   int64_t slabs, vs;
+  double cost;  // modelled time of the plan's tile kernels (kernel_cost units)
   PackPlan pack;
   size_t lse_c, dxc;  // lse of the packed rows; packed dx before it is moved to its place (only for a dx of >= 2 GiB)
   bool stage_dx;
@@ -311,10 +313,10 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
   BwdPlan full = *b, lean = *b;
   double cost_full = 0, cost_lean = 0;
   const bool ok_full = choose(0, &full, &cost_full), ok_lean = choose(1, &lean, &cost_lean);
-  if (ok_full && (!ok_lean || cost_full <= cost_lean)) { *b = full; return LCE_OK; }
-  if (ok_lean) { *b = lean; return LCE_OK; }
-  double unused = 0;
-  if (choose(2, b, &unused)) return LCE_OK;
+  if (ok_full && (!ok_lean || cost_full <= cost_lean)) { *b = full; b->cost = cost_full; return LCE_OK; }
+  if (ok_lean) { *b = lean; b->cost = cost_lean; return LCE_OK; }
+  double wide = 0;
+  if (choose(2, b, &wide)) { b->cost = wide; return LCE_OK; }
   return LCE_EWORKSPACE;
 }
 
@@ -338,7 +340,7 @@ struct FusedPlan {
 bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) {
   memset(f, 0, sizeof(*f));
   const bool x16 = p->x_dtype == LCE_BF16 || p->x_dtype == LCE_F16;
-  if (!x16 || p->w_dtype != p->x_dtype || p->monitoring) return false;
+  if (!x16 || p->w_dtype != p->x_dtype || p->monitoring || p->route == LCE_ROUTE_TWO_PASS) return false;
   const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V), Hp = (size_t)lce::padded_hidden(p->H);
   const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
   // (packed rows of dx go to their tokens through 32-bit offsets into dx)
@@ -396,6 +398,8 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     };
     const double cost = (double)(chunks - 1) * chunk_cost((double)t_even) + chunk_cost((double)t_last);
     if (first == 0) first = chunks;
+    // (what the chunks do not change: the pass over the stage at 4 bytes per logit, the plane's way out at
+    // 6 bytes per element of dW -- about 8 MB of memory traffic per unit)
     if (!f->ok || cost < best) {
       best = cost;
       *f = cand;
@@ -404,7 +408,19 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
       f->ok = true;
     }
   }
-  return f->ok;
+  if (!f->ok) return false;
+  // The two-pass route by the same model: the forward over all tokens, then the backward's plan.  It wins where the
+  // scratch bound leaves only short chunks (every chunk adds a round trip of the whole fp32 plane of dW).
+  BwdPlan b;
+  if (p->route == LCE_ROUTE_AUTO && plan_bwd(p, &b) == LCE_OK) {
+    const double fixed = (double)Np * (double)Vp * 4.0 / 8.0e6 + (f->chunks > 1 && want_dw ? (double)Hp * (double)Vp * 6.0 / 8.0e6 : 0.0);
+    const double two = kernel_cost((double)tiles * tv, (double)(lce::padded_k(p->H) / 64), 4.0, false) + b.cost;
+    if (best + fixed > two) {
+      f->ok = false;
+      return false;
+    }
+  }
+  return true;
 }
 
 bool misaligned(const void* p) { return ((uintptr_t)p & 15) != 0; }

@@ -46,7 +46,9 @@ pack_rows: contextvars.ContextVar = contextvars.ContextVar("lce_pack_rows", defa
 
 
 # Whether a forward that needs gradients computes them in the same pass over the logits (see the module
-# docstring); `one_pass.set(False)` makes every call take the loss-only forward and the recomputing backward.
+# docstring): True -- where the library's model of its kernels says that this is the faster route (lce_problem.route
+# = LCE_ROUTE_AUTO); "always" -- wherever the route fits the scratch bound; False -- never: every call takes the
+# loss-only forward and the recomputing backward.
 one_pass: contextvars.ContextVar = contextvars.ContextVar("lce_one_pass", default=True)
 
 
@@ -206,6 +208,7 @@ def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_c
         prob = _lib.make_problem(
             N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, w_cols + (-w_cols) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
             ignore_index, logit_scale, z_regularization, N_chunk_size, False, 0, pack, 0, layout,
+            _lib.ROUTE_ONE_PASS if one_pass.get() == "always" else _lib.ROUTE_AUTO,
         )
         lib = _lib.load()
         _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")

@@ -474,8 +474,14 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
         n_chunk = rng.choice([256, 1024, 4096, 8192, 32768])
         dt = rng.choice([torch.bfloat16, torch.float16])
         prob = _lib.make_problem(N, H, V, H + (-H) % 8, V + (-V) % 8, H + (-H) % 8, V + (-V) % 8, dt, dt, dt, dt, -1, 1.0,
+                                 0.0, n_chunk, False, route=_lib.ROUTE_ONE_PASS)
+        auto = _lib.make_problem(N, H, V, H + (-H) % 8, V + (-V) % 8, H + (-H) % 8, V + (-V) % 8, dt, dt, dt, dt, -1, 1.0,
                                  0.0, n_chunk, False)
+        never = _lib.make_problem(N, H, V, H + (-H) % 8, V + (-V) % 8, H + (-H) % 8, V + (-V) % 8, dt, dt, dt, dt, -1, 1.0,
+                                  0.0, n_chunk, False, route=_lib.ROUTE_TWO_PASS)
         chunks, rows = _lib.forward_backward_plan(prob)
+        assert _lib.forward_backward_plan(never) == (0, 0)
+        assert _lib.forward_backward_plan(auto) in ((0, 0), (chunks, rows))  # the library's choice: the same plan, or two passes
         total = _lib.forward_backward_workspace_bytes(prob)
         if chunks == 0:
             assert total == max(_lib.workspace_bytes(prob))

@@ -23,7 +23,7 @@ def _problem(N, H, V, x, w, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, phas
 
     hp, cols = H + (-H) % 8, (H if layout else V)
     return _lib.make_problem(N, H, V, x.stride(0), w.stride(0), hp, cols + (-cols) % 8, dt, dt, dt, dw_dt, -1, scale,
-                             z_reg, n_chunk, False, phases, pack, 0, layout)
+                             z_reg, n_chunk, False, phases, pack, 0, layout, _lib.ROUTE_ONE_PASS)
 
 
 def _both_routes(N, H, V, dt, n_chunk, ignore, z_reg=0.0, scale=1.0, pack=0, layout=0, dw_dt=None, grad_out=1.0,
@@ -128,7 +128,9 @@ def test_one_pass_matches_two_pass_and_the_fp64_oracle(N, H, V, dt, n_chunk, ign
 
 @pytest.mark.pack_auto
 def test_fp16_z_regularisation_with_lse_near_a_thousand_on_the_one_pass_route():
-    from linear_cross_entropy_loss_amd import linear_cross_entropy
+    from linear_cross_entropy_loss_amd import linear_cross_entropy, ops
+
+    ops.one_pass.set("always")  # (the autouse fixtures of conftest.py put the default back)
 
     N, H, V = 1024, 256, 4096
     x, y, w = make_inputs(N, H, V, torch.float16, seed=11, ignore_frac=0.1)
@@ -146,7 +148,9 @@ def test_fp16_z_regularisation_with_lse_near_a_thousand_on_the_one_pass_route():
 
 @pytest.mark.pack_auto
 def test_a_second_backward_recomputes_and_the_upstream_gradient_is_multiplied_in_fp32():
-    from linear_cross_entropy_loss_amd import linear_cross_entropy
+    from linear_cross_entropy_loss_amd import linear_cross_entropy, ops
+
+    ops.one_pass.set("always")
 
     N, H, V = 2048, 512, 8192
     x, y, w = make_inputs(N, H, V, torch.bfloat16, seed=5, ignore_frac=0.1)
