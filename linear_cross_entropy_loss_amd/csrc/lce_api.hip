@@ -396,7 +396,8 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
              (want_dx ? kernel_cost(tt * th, (double)(Vp / 64), 5.0, true) : 0.0) +
              (want_dw ? kernel_cost(tv * th, tt * 4.0, chunks > 1 ? 12.0 : 5.0, chunks == 1) : 0.0);
     };
-    const double cost = (double)(chunks - 1) * chunk_cost((double)t_even) + chunk_cost((double)t_last);
+    // (per chunk, besides the tile kernels: the row merge, the kernel that adds dx's K segments, launch gaps -- about 25 units)
+    const double cost = (double)(chunks - 1) * chunk_cost((double)t_even) + chunk_cost((double)t_last) + 25.0 * (double)chunks;
     if (first == 0) first = chunks;
     // (what the chunks do not change: the pass over the stage at 4 bytes per logit, the plane's way out at
     // 6 bytes per element of dW -- about 8 MB of memory traffic per unit)

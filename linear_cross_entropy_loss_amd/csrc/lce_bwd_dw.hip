@@ -194,38 +194,41 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
 // accumulator before the sums go (back) to the block.  After the last chunk dw_plane_out_kernel scales the sums
 // and stores dW.  (Hardware fp32 atomic adds instead of the load - add - store were measured at the headline shape:
 // the 268 M atomics of a chunk take longer than the chunk's matrix work, 30.6 ms a step against 22.3.)
-// The four quads of an accumulator block are fetched together before any is used.
+#ifndef LCE_DW_PLANE_BATCH
+#define LCE_DW_PLANE_BATCH 16
+#endif
 template <bool LOAD>
 LCE_DEV void dw_plane_io(float* blk, f32x16_t (&acc)[kNB][kNB]) {
   // one descriptor over the block, the thread's 16 bytes as the vector offset, the quad as a scalar offset: no
   // 64-bit address per quad
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(blk, 0, kTile * kTile * 4, 0x00020000);
   const int voff = opaque_tid() * 16;
+  // kPlaneBatch quads are fetched together before any is used: the loads of a batch are in flight together, and a
+  // tile waits for 64 / kPlaneBatch round trips to memory
+  constexpr int kPlaneBatch = LCE_DW_PLANE_BATCH;
 #pragma unroll
-  for (int rb = 0; rb < kNB; ++rb)
+  for (int q0 = 0; q0 < 64; q0 += kPlaneBatch) {
+    u32x4_t old[kPlaneBatch];
+    if (LOAD) {
 #pragma unroll
-    for (int cb = 0; cb < kNB; ++cb) {
-      u32x4_t old[4];
-      if (LOAD) {
-#pragma unroll
-        for (int rq = 0; rq < 4; ++rq)
-          old[rq] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, ((rb * 4 + cb) * 4 + rq) * 4096, 0);
-      }
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        f32x4_t v;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          // (a volatile read: the compiler would otherwise read all 256 accumulator registers before the first load)
-          float t;
-          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[rb][cb][rq * 4 + j]));
-          v[j] = t;
-        }
-        if (LOAD) v += __builtin_bit_cast(f32x4_t, old[rq]);
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), rsrc, voff, ((rb * 4 + cb) * 4 + rq) * 4096, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);  // (the quads of one accumulator block in registers at a time: an operand tile is in flight)
+      for (int u = 0; u < kPlaneBatch; ++u) old[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, (q0 + u) * 4096, 0);
     }
+#pragma unroll
+    for (int u = 0; u < kPlaneBatch; ++u) {
+      const int q = q0 + u, rb = q >> 4, cb = (q >> 2) & 3, rq = q & 3;
+      f32x4_t v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // (a volatile read: the compiler would otherwise read all 256 accumulator registers before the first load)
+        float t;
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[rb][cb][rq * 4 + j]));
+        v[j] = t;
+      }
+      if (LOAD) v += __builtin_bit_cast(f32x4_t, old[u]);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), rsrc, voff, q * 4096, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // (one batch in registers at a time: an operand tile is in flight)
+  }
 }
 
 // How one launch divides its work: as for dx (lce_bwd_dx.hip).  The T = (vs/256) x (Hp/256) output tiles
