@@ -107,15 +107,16 @@ def test_static_forward_refuses_what_does_not_fit():
     with pytest.raises(RuntimeError, match="static"):
         _lib.raise_for_status(rc, "lce_forward_static")
     # The sizes include/lce.h quotes at V = 131072, H = 2048: 4096 rows fit without the monitoring values (32.1 MiB)
-    # and do not with them (four partial buffers instead of one: 64.02 MiB); 2048 rows with monitoring fit.
+    # and do not with them (four partial buffers instead of one, no packed copy of x: 64.02 MiB); 2048 rows with
+    # monitoring fit.
     for rows, mon, fits in ((4096, False, True), (4096, True, False), (2048, True, True)):
         p = _lib.make_problem(rows, 2048, 131072, 2048, 131072, 2048, 131072, x.dtype, w.dtype, x.dtype, w.dtype, -1,
-                              1.0, 0.0, 4096, mon, 0, _lib.PACK_NEVER)
+                              1.0, 0.0, 4096, mon, 0, _lib.PACK_AUTO)
         need, _ = _lib.workspace_bytes(p)
         assert (need <= _lib.STATIC_SCRATCH_BYTES) == fits, (rows, mon, need)
         if not fits:  # refused before any pointer is looked at (these buffers are far too small for the problem)
             assert lib.lce_forward_static(ctypes.byref(p), _P(x), _P(w), _P(y), _P(lse), _P(out5), _P(nv), stream) == _lib.LCE_ESTATIC
     sizes = {mon: _lib.workspace_bytes(_lib.make_problem(4096, 2048, 131072, 2048, 131072, 2048, 131072, x.dtype, w.dtype,
-                                                         x.dtype, w.dtype, -1, 1.0, 0.0, 4096, mon, 0, _lib.PACK_NEVER))[0]
+                                                         x.dtype, w.dtype, -1, 1.0, 0.0, 4096, mon, 0, _lib.PACK_AUTO))[0]
              for mon in (False, True)}
     assert abs(sizes[False] / 2**20 - 32.1) < 0.1 and abs(sizes[True] / 2**20 - 64.02) < 0.1, sizes
