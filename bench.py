@@ -340,7 +340,14 @@ def c4_sweep(args, torch):
         peak = torch.cuda.max_memory_allocated() - base
         grads = x.numel() * x.element_size() + w.numel() * w.element_size()
         ms = median_step_ms(step, torch, reps=max(5, args.steps // 10), flush=False)
-        points.append(dict(V=V, N_chunk_size=nc, ms=ms, tflops_8NHV=8.0 * N * H * V / ms / 1e9,
+        from linear_cross_entropy_loss_amd import _lib, ops
+
+        plan = (0, 0)
+        if ops.one_pass.get():
+            plan = _lib.forward_backward_plan(_lib.make_problem(N, H, V, H, V, H, V, x.dtype, w.dtype, x.dtype, w.dtype, -1,
+                                                                1.0, 0.0, nc, False))
+        points.append(dict(V=V, N_chunk_size=nc, ms=ms, route="one_pass" if plan[0] else "two_pass",
+                           chunks=plan[0], chunk_rows=plan[1], tflops_8NHV=8.0 * N * H * V / ms / 1e9,
                            pct_mfma_peak=100.0 * 8.0 * N * H * V / ms / 1e9 / PEAK_TFLOPS["bf16"],
                            peak_hbm_bytes_incl_grads=int(peak), peak_hbm_bytes_extra=int(peak - grads),
                            scratch_budget_bytes=int(nc * V * 4), within_budget=bool(peak - grads <= nc * V * 4),
@@ -482,7 +489,7 @@ def main():
             tr = json.load(f)
         # counters collected on other kernel sources say nothing about this build
         if tr.get("sources_sha16") == sources_sha16():
-            roofline["traffic"] = tr.get(args.workload, {}).get(dom)
+            roofline["traffic"] = tr.get(args.workload, {}).get(route, {}).get(dom)
             roofline["traffic_note"] = tr.get("note")
         else:
             roofline["traffic_note"] = "profiles/hbm_traffic.json was collected on other kernel sources: dropped"
