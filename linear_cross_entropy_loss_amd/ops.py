@@ -500,12 +500,13 @@ class LinearCrossEntropyLoss(torch.nn.Linear):
         ignore_index: label value that is skipped. Default -100.
         logit_scale: positive factor applied to the logits before the loss. Default 1.0.
         z_regularization: weight of the ``mean(logsumexp(z)^2)`` penalty. Default 0.0.
-        N_chunk_size: target for the scratch memory of the backward, ``N_chunk_size * out_features * 4`` bytes
-            (what the reference spends on one chunk of logits); the backward works through the vocabulary in
-            as many slabs as that takes, and the forward through the tokens in chunks of
-            ``max(N_chunk_size, 16384)`` rows.  The number of rows of ``x`` is free; what grows with it is the
-            backward's fp32 running sum of ``dx`` and the packed copy of ``x`` (``6 * in_features`` bytes per
-            token).  Default 4096.
+        N_chunk_size: bound on the scratch memory, ``N_chunk_size * out_features * 4`` bytes (what the reference spends
+            on one chunk of logits).  Where it leaves room, a forward that needs gradients computes them from its one
+            evaluation of the logits, in chunks of token rows (16-bit staging of a chunk against the whole vocabulary plus
+            an fp32 sum of the weight gradient, ``in_features * out_features * 4`` bytes); otherwise the backward
+            recomputes the logits and works through the vocabulary in as many slabs as the bound takes, and the forward
+            through the tokens in chunks of ``max(N_chunk_size, 16384)`` rows.  A larger value buys longer chunks (faster)
+            at more scratch.  The number of rows of ``x`` is free.  Default 4096.
         init_method: optional callable applied to the weight instead of the default truncated normal.
 
     Set ``module.monitoring = True`` to also collect ``logit_norm``, ``logit_max``, ``logit_entropy`` and
