@@ -463,7 +463,7 @@ def main():
     peak = PEAK_TFLOPS[cfg["dtype"]]
     # which route the steps above took (ops.LinearXentImplementation.forward decides the same way)
     route = "two_pass"
-    if not args.two_pass and not cfg["monitoring"] and cfg["dtype"] != "f32" and cfg.get("w_dtype", cfg["dtype"]) == cfg["dtype"]:
+    if not args.two_pass and not cfg["monitoring"] and cfg["dtype"] != "f32":
         wr = w.detach().t() if cfg.get("w_vh") else w.detach()
         pr = _lib.make_problem(N, H, V, x.stride(0), wr.stride(0), H, wr.stride(0), x.dtype, wr.dtype, x.dtype, wr.dtype, -1,
                                cfg["scale"], cfg["z_reg"], cfg["n_chunk"], False, 0, 0, 0,

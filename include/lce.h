@@ -302,7 +302,12 @@ enum {
  * that turns e into dz.
  *
  *   grad_out   device pointer to 1 float: upstream gradient of the loss
- *              (the reference multiplies it in afterwards, ops.py:810)
+ *              (the reference multiplies it in afterwards, ops.py:810).  A
+ *              caller that learns it later passes a stand-in and rescales
+ *              with lce_scale: 1 for bf16 / fp32 gradients; for fp16
+ *              gradients a power of two near the number of valid labels,
+ *              since entries of order 1/n_valid would leave fp16's normal
+ *              range before a loss scale could be applied
  *   dx, dw     as for lce_backward; with both NULL this is lce_forward
  *   ws         lce_forward_backward_workspace_bytes(p) bytes
  */

@@ -333,29 +333,39 @@ struct FusedPlan {
   int64_t nc;
   int chunks;
   PackPlan k;
-  size_t chunk_rows, lse_rows, tgt, blk, part_lse, part_max, stage, plane, part, total;
+  size_t chunk_rows, lse_rows, tgt, blk, w16, xc, part_lse, part_max, stage, plane, part, total;
+  int64_t ld16;    // row stride of the 16-bit copy of an fp32 weight
   bool parts_on;
+  bool dw_direct;  // fp32 dW: the chunks' terms are added in the caller's buffer, there is no plane
 };
 
 bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) {
   memset(f, 0, sizeof(*f));
   const bool x16 = p->x_dtype == LCE_BF16 || p->x_dtype == LCE_F16;
-  if (!x16 || p->w_dtype != p->x_dtype || p->monitoring || p->route == LCE_ROUTE_TWO_PASS) return false;
+  if (!x16 || (p->w_dtype != p->x_dtype && p->w_dtype != LCE_F32) || p->monitoring || p->route == LCE_ROUTE_TWO_PASS) return false;
   const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V), Hp = (size_t)lce::padded_hidden(p->H);
   const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
   // (packed rows of dx go to their tokens through 32-bit offsets into dx)
   f->pack = packs_rows(p) && (size_t)p->N * (size_t)p->lddx * dxes < ((size_t)1 << 31);
+  f->dw_direct = p->dw_dtype == LCE_F32;
   f->k = plan_pack(p, 0, false);
-  size_t o = f->pack ? f->k.end : f->k.xc;  // the labels are always counted; the copy of x only exists for packed rows
+  size_t o = f->k.xc;  // the labels are always counted; the packed copy of x is made chunk by chunk (below)
   f->chunk_rows = o; o += align_up(1024 * 8);
   f->lse_rows = o; o += align_up(Np * 4);
   f->tgt = o; o += align_up(Np * 4);
   f->blk = o; o += align_up(Np / lce::kMergeRows * 8 * sizeof(double));
+  // an fp32 master weight is rounded to the compute type once per call, all of it
+  const bool vh = p->w_layout == LCE_W_VH;
+  f->ld16 = vh ? p->H : (int64_t)Vp;
+  f->w16 = o;
+  if (p->w_dtype == LCE_F32) o += align_up((vh ? (size_t)p->V : (size_t)p->H) * (size_t)f->ld16 * 2);
   const size_t fixed = o;
   const size_t bound = (size_t)p->n_chunk * (size_t)p->V * 4;
   const size_t reserve = align_up((size_t)p->N * 4) + 4096;  // what the caller holds besides the workspace: lse and a few scalars
   auto total_for = [&](int64_t nc, int chunks, FusedPlan* out) -> size_t {
     size_t t = fixed;
+    out->xc = t;
+    if (f->pack) t += align_up((size_t)nc * (size_t)f->k.ldxc * 2);
     const size_t part = align_up(Vp / lce::kChunkV * (size_t)nc * 4);
     out->part_lse = t; t += part;
     out->part_max = t; t += part;
@@ -369,7 +379,7 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     out->part = t; t += pb;
     out->parts_on = pb != 0;
     out->plane = t;
-    if (chunks > 1 && want_dw) t += align_up(Hp * Vp * 4);
+    if (chunks > 1 && want_dw && !f->dw_direct) t += align_up(Hp * Vp * 4);
     out->total = t;
     return t;
   };
@@ -394,7 +404,7 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     auto chunk_cost = [&](double tt) -> double {
       return kernel_cost(tt * tv, (double)(lce::padded_k(p->H) / 64), 8.0, false) +
              (want_dx ? kernel_cost(tt * th, (double)(Vp / 64), 5.0, true) : 0.0) +
-             (want_dw ? kernel_cost(tv * th, tt * 4.0, chunks > 1 ? 12.0 : 5.0, chunks == 1) : 0.0);
+             (want_dw ? kernel_cost(tv * th, tt * 4.0, chunks > 1 ? (f->dw_direct ? 16.0 : 12.0) : 5.0, chunks == 1) : 0.0);
     };
     // (per chunk, besides the tile kernels: the row merge, the kernel that adds dx's K segments, launch gaps -- about 25 units)
     const double cost = (double)(chunks - 1) * chunk_cost((double)t_even) + chunk_cost((double)t_last) + 25.0 * (double)chunks;
@@ -414,7 +424,8 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
   // scratch bound leaves only short chunks (every chunk adds a round trip of the whole fp32 plane of dW).
   BwdPlan b;
   if (p->route == LCE_ROUTE_AUTO && plan_bwd(p, &b) == LCE_OK) {
-    const double fixed = (double)Np * (double)Vp * 4.0 / 8.0e6 + (f->chunks > 1 && want_dw ? (double)Hp * (double)Vp * 6.0 / 8.0e6 : 0.0);
+    const double fixed = (double)Np * (double)Vp * 4.0 / 8.0e6 +
+                         (f->chunks > 1 && want_dw && !f->dw_direct ? (double)Hp * (double)Vp * 6.0 / 8.0e6 : 0.0);
     const double two = kernel_cost((double)tiles * tv, (double)(lce::padded_k(p->H) / 64), 4.0, false) + b.cost;
     if (best + fixed > two) {
       f->ok = false;
@@ -610,19 +621,31 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
     if (e != hipSuccess) return hip_fail(e, "compact_labels");
   }
   if (f.pack && (ph & LCE_PHASE_PACK)) {
-    e = lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, perm, n_rows, p->N, base + k.xc, k.ldxc * 2, nullptr, nullptr,
-                                num_cus, s, true);
-    if (e != hipSuccess) return hip_fail(e, "gather_rows");
     e = lce::launch_chunk_rows(n_rows, p->N, f.nc, f.chunks, chunk_rows, s);
     if (e != hipSuccess) return hip_fail(e, "chunk_rows");
+  }
+  // an fp32 master weight: one 16-bit copy of all of it, which the three tile kernels of every chunk read
+  const void* wk = w;
+  int64_t ldwk = p->ldw;
+  int wk_dtype = p->w_dtype;
+  if (p->w_dtype == LCE_F32) {
+    wk = base + f.w16;
+    ldwk = f.ld16;
+    wk_dtype = compute_dtype(p);
+    if (ph & LCE_PHASE_PACK) {
+      e = p->w_layout == LCE_W_VH
+              ? lce::launch_convert_w_rows((const float*)w, p->ldw, p->H, 0, p->V, base + f.w16, f.ld16, compute_dtype(p), s)
+              : lce::launch_convert_w_slab((const float*)w, p->ldw, p->H, 0, p->V, base + f.w16, f.ld16, compute_dtype(p), false, s);
+      if (e != hipSuccess) return hip_fail(e, "convert_w");
+    }
   }
 
   lce::BwdArgs b;
   memset(&b, 0, sizeof(b));
-  b.w = w; b.n_valid = n_rows; b.grad_out = grad_out;
+  b.w = wk; b.n_valid = n_rows; b.grad_out = grad_out;
   b.H = p->H; b.V = p->V; b.Hp = lce::padded_hidden(p->H);
-  b.ldw = p->ldw; b.lddx = p->lddx; b.lddw = p->lddw;
-  b.x_dtype = p->x_dtype; b.w_dtype = p->w_dtype; b.dx_dtype = p->dx_dtype; b.dw_dtype = p->dw_dtype;
+  b.ldw = ldwk; b.lddx = p->lddx; b.lddw = p->lddw;
+  b.x_dtype = p->x_dtype; b.w_dtype = wk_dtype; b.dx_dtype = p->dx_dtype; b.dw_dtype = p->dw_dtype;
   b.w_vh = p->w_layout == LCE_W_VH;
   b.ignore_index = p->ignore_index;
   b.scale = p->logit_scale; b.z_reg = p->z_reg;
@@ -638,7 +661,7 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
   b.nc = f.nc;
   b.dx_part = f.parts_on && dx ? (float*)(base + f.part) : nullptr;
   b.dw_part = f.parts_on && dw && f.chunks == 1 ? (float*)(base + f.part) : nullptr;
-  b.dw_plane = f.chunks > 1 ? (float*)(base + f.plane) : nullptr;
+  b.dw_plane = f.chunks > 1 && !f.dw_direct ? (float*)(base + f.plane) : nullptr;
 
   for (int c = 0; c < f.chunks; ++c) {
     const int64_t row0 = (int64_t)c * f.nc;
@@ -652,7 +675,7 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
       a.n_rows = chunk_rows + c;
       a.perm = perm + row0;
       a.perm_always = 1;
-      a.x = a.xc = base + k.xc + (size_t)row0 * (size_t)k.ldxc * 2;
+      a.x = a.xc = base + f.xc;  // the chunk's kept rows, gathered just below
       a.ldx = a.ldxc = k.ldxc;
       a.y = yc + row0;
       a.dx = dx;
@@ -663,8 +686,14 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
       a.y = y + row0;
       a.dx = dx ? (char*)dx + (size_t)row0 * (size_t)p->lddx * dxes : nullptr;
     }
-    a.dw_acc = f.chunks == 1 ? 0 : (c == 0 ? 1 : 2);
+    // dW over the chunks: the plane (1: store, 2: add), or -- fp32 dW -- the caller's buffer itself (3: store, 4: add)
+    a.dw_acc = f.chunks == 1 ? 0 : (f.dw_direct ? (c == 0 ? 3 : 4) : (c == 0 ? 1 : 2));
     a.last_chunk = c == f.chunks - 1;
+    if (f.pack && (ph & (LCE_PHASE_PACK | LCE_PHASE_FWD_TILES | LCE_PHASE_BWD_DW))) {
+      e = lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, perm + row0, chunk_rows + c, p->N, base + f.xc, k.ldxc * 2,
+                                  nullptr, nullptr, num_cus, s, true);
+      if (e != hipSuccess) return hip_fail(e, "gather_rows");
+    }
     if (ph & LCE_PHASE_FWD_TILES) {
       e = lce::launch_fwd_stage(a, s);
       if (e != hipSuccess) return hip_fail(e, "fwd_stage");

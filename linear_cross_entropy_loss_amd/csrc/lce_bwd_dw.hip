@@ -231,6 +231,58 @@ LCE_DEV void dw_plane_io(float* blk, f32x16_t (&acc)[kNB][kNB]) {
   }
 }
 
+// fp32 dW summed over chunks of token rows in the caller's buffer itself (BwdArgs::dw_acc 3 / 4): the tile's sum times
+// the final factor is stored (first chunk) or added to what is there (ADD), in the 16-byte quads a lane holds -- rows
+// of the stored matrix along the lanes, as in dw_epilogue; the four quads of an accumulator block are fetched
+// together before any is used.
+template <bool WVH, bool ADD>
+LCE_DEV void dw_epilogue_f32_sum(const BwdArgs& a, f32x16_t (&acc)[kNB][kNB], int tp, int tq) {
+  const DwTileGeom<WVH> g(a, tp, tq);
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wp = wave & 1, wq = wave >> 1;
+  const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
+  const int half = lane >> 5;
+  const float coef = final_factor_of(a);
+#pragma unroll
+  for (int rb = 0; rb < kNB; ++rb) {
+    const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + (lane & 31);
+    const bool row_exists = row < g.row_limit;
+    const int64_t c0 = g.col0 + w_col * kWaveTile + 4 * half;  // this lane's first column
+    float* prow = reinterpret_cast<float*>(a.dw) + row * a.lddw + c0;
+#pragma unroll
+    for (int cbk = 0; cbk < kNB; ++cbk) {
+      f32x4_t old[4];
+      bool ok[4];
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        // quads that start at or past the last column are left alone; one that it cuts through is written whole,
+        // into the stride padding of its row
+        ok[rq] = row_exists && c0 + cbk * kBlk + 8 * rq < g.col_limit;
+        if (ADD) {
+          const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+          old[rq] = ok[rq] ? *reinterpret_cast<const f32x4_t*>(prow + cbk * kBlk + 8 * rq) : zero;
+        }
+      }
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        f32x4_t v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          // (a volatile read: the compiler would otherwise read all 256 accumulator registers before the first load)
+          float t;
+          if (WVH) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[cbk][rb][rq * 4 + j]));
+          else asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[rb][cbk][rq * 4 + j]));
+          v[j] = t * coef;
+        }
+        if (ADD) v += old[rq];
+        if (ok[rq]) *reinterpret_cast<f32x4_t*>(prow + cbk * kBlk + 8 * rq) = v;
+      }
+      __builtin_amdgcn_sched_barrier(0);  // (one block in registers at a time: an operand tile is in flight)
+    }
+  }
+}
+
 // How one launch divides its work: as for dx (lce_bwd_dx.hip).  The T = (vs/256) x (Hp/256) output tiles
 // go to G persistent workgroups in rounds; a last round with r <= G/2 tiles is cut along K = tokens into
 // `nseg` segments of `kseg` K tiles (r * nseg <= G, at least 16 K tiles each), whose fp32 sums meet in
@@ -343,7 +395,10 @@ template <class T, bool WVH, int MODE, int ACC = 0> struct DwProblem {
   LCE_DEV void epilogue(int local, f32x16_t (&acc)[kNB][kNB], char* scratch) const {
     int item, tp, tq, seg;
     decode(local, item, tp, tq, seg);
-    if constexpr (ACC != 0) {
+    if constexpr (ACC == 3 || ACC == 4) {
+      dw_epilogue_f32_sum<WVH, ACC == 4>(a, acc, tp, tq);
+      return;
+    } else if constexpr (ACC != 0) {
       float* blk = a.dw_plane + ((int64_t)tq * tiles_p + tp) * (kTile * kTile);
       dw_plane_io<ACC == 2>(blk, acc);
       return;
@@ -481,6 +536,10 @@ template <class T, bool WVH, int MODE> hipError_t launch_plane(const BwdArgs& a,
 }
 
 template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
+  if (a.dw_acc == 3 || a.dw_acc == 4) {  // fp32 dW summed in the caller's buffer: whole tiles only
+    if (a.dw_dtype != DT_F32 || a.dw_part != nullptr) return hipErrorInvalidValue;
+    return a.dw_acc == 3 ? launch_tiles<T, WVH, kDwAll, 3>(a, s) : launch_tiles<T, WVH, kDwAll, 4>(a, s);
+  }
   if (a.dw_acc != 0) {
     if (a.dw_plane == nullptr || a.dw_part != nullptr || a.dw_acc > 2) return hipErrorInvalidValue;
     return launch_plane<T, WVH, kDwAll>(a, s);

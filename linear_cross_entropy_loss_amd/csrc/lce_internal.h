@@ -165,6 +165,7 @@ struct BwdArgs {
   // dW summed over chunks of token rows: dw_plane holds one 256 x 256 fp32 block per tile of dW, in the order of
   // the accumulator registers (lce_bwd_dw.hip).  dw_acc: 0 = no plane (dW is stored as it comes), 1 = the sums
   // are stored to the plane (first chunk), 2 = added to it; last_chunk: the plane is then scaled and stored as dW.
+  // fp32 dW needs no plane: 3 = the sums times the final factor are stored to dw itself (first chunk), 4 = added to it.
   float* dw_plane;
   int dw_acc, last_chunk;
 };

@@ -197,11 +197,12 @@ def _finish_grads(dx, dw, layout):
 
 
 def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, pack, need_dx, need_dw):
-    """Runs lce_forward_backward with an upstream gradient of 1 when its one-pass route covers the problem.
-    Returns None otherwise, else (out5, lse, n_valid, x, y1, w, layout, dx, dw)."""
+    """Runs lce_forward_backward when its one-pass route covers the problem.  Returns None otherwise, else
+    (out5, lse, n_valid, x, y1, w, layout, dx, dw, pre): the gradients for an upstream gradient of `pre` (a device
+    scalar; None stands for 1)."""
     with torch.cuda.device(x_in.device):
         x, y1, w, layout, N, H, V = _problem_views(x_in, y, At)
-        if x.dtype == torch.float32 or w.dtype != x.dtype:
+        if x.dtype == torch.float32 or w.dtype not in (x.dtype, torch.float32):
             return None
         vh = layout == _lib.W_VH
         w_cols = H if vh else V
@@ -221,13 +222,20 @@ def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_c
         lse = torch.empty(N, dtype=torch.float32, device=dev)
         out5 = torch.empty(5, dtype=torch.float32, device=dev)
         n_valid = torch.empty(1, dtype=torch.int64, device=dev)
-        one = torch.ones(1, dtype=torch.float32, device=dev)
+        # The upstream gradient is not known yet.  bf16 / fp32 gradients are formed for an upstream gradient of 1.  fp16
+        # ones would fall below fp16's normal range on the way (entries of order 1/n_valid; a loss scale arrives too
+        # late to save them): they are formed for the largest power of two that is not above the number of valid
+        # labels -- entries of the order of the per-token gradient -- and backward divides it out again.
+        if x.dtype == torch.float16:
+            pre = torch.exp2(torch.floor(torch.log2((y1 != ignore_index).sum().clamp(min=1).to(torch.float32)))).reshape(1)
+        else:
+            pre = torch.ones(1, dtype=torch.float32, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream
-        rc = lib.lce_forward_backward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(one), _ptr(lse), _ptr(out5),
+        rc = lib.lce_forward_backward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(pre), _ptr(lse), _ptr(out5),
                                       _ptr(n_valid), _ptr(dx), _ptr(dw), _ptr(ws), nbytes, ctypes.c_void_p(stream))
         _lib.raise_for_status(rc, "lce_forward_backward")
         del ws
-    return out5, lse, n_valid, x, y1, w, layout, dx, dw
+    return out5, lse, n_valid, x, y1, w, layout, dx, dw, (pre if x.dtype == torch.float16 else None)
 
 
 def _scale_grad(t, grad_output):
@@ -342,8 +350,8 @@ class LinearXentImplementation(torch.autograd.Function):
             done = _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, pack,
                                   need_dx, need_dw)
         if done is not None:
-            out5, lse, n_valid, x, y1, w, layout, dx, dw = done
-            ctx.lce_grads = [dx, dw]  # for the first backward; dropped there
+            out5, lse, n_valid, x, y1, w, layout, dx, dw, pre = done
+            ctx.lce_grads = [dx, dw, pre]  # for the first backward; dropped there
         else:
             out5, lse, n_valid, x, y1, w, layout = _forward_impl(
                 x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack)
@@ -364,9 +372,10 @@ class LinearXentImplementation(torch.autograd.Function):
         if grads is not None:
             # computed in the forward for an upstream gradient of 1 (ops.py:810 does the same multiplication); a
             # later backward over the same graph finds nothing here and recomputes
-            dx, dw = grads
-            _scale_grad(dx, grad_output)
-            _scale_grad(dw, grad_output)
+            dx, dw, pre = grads
+            factor = grad_output.detach().to(torch.float32) if pre is None else grad_output.detach().to(torch.float32) / pre
+            _scale_grad(dx, factor)
+            _scale_grad(dw, factor)
             dx, dw = _finish_grads(dx, dw, layout)
         else:
             dx, dw = _backward_impl(x, y1, w, lse, n_valid, grad_output, ignore_index, z_regularization, logit_scale,

@@ -497,8 +497,25 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
     prob = _lib.make_problem(16384, 2048, 131072, 2048, 131072, 2048, 131072, torch.bfloat16, torch.bfloat16,
                              torch.bfloat16, torch.bfloat16, -1, 1.0, 0.0, 4096, False)
     assert _lib.forward_backward_plan(prob) == (5, 3328)
-    for kw in (dict(x=torch.float32, w=torch.float32), dict(x=torch.bfloat16, w=torch.float32), dict(mon=True)):
+    for kw in (dict(x=torch.float32, w=torch.float32), dict(mon=True)):
         xd, wd = kw.get("x", torch.bfloat16), kw.get("w", torch.bfloat16)
         prob = _lib.make_problem(4096, 512, 8192, 512, 8192, 512, 8192, xd, wd, xd, wd, -1, 1.0, 0.0, 4096,
                                  kw.get("mon", False))
         assert _lib.forward_backward_plan(prob) == (0, 0), kw
+    # an fp32 master weight under 16-bit activations: one 16-bit copy of all of it in the workspace, and its fp32 gradient
+    # is summed over the chunks in the caller's buffer (no plane)
+    kw = dict(N=8192, H=1024, V=32768, ldx=1024, ldw=32768, lddx=1024, lddw=32768, x_dtype=torch.bfloat16,
+              dx_dtype=torch.bfloat16, ignore_index=-1, logit_scale=1.0, z_reg=0.0, n_chunk=2048, monitoring=False,
+              route=_lib.ROUTE_ONE_PASS)
+    p32 = _lib.make_problem(w_dtype=torch.float32, dw_dtype=torch.float32, **kw)
+    p16 = _lib.make_problem(w_dtype=torch.bfloat16, dw_dtype=torch.bfloat16, **kw)
+    p16_32 = _lib.make_problem(w_dtype=torch.bfloat16, dw_dtype=torch.float32, **kw)
+    c32, r32 = _lib.forward_backward_plan(p32)
+    c16, r16 = _lib.forward_backward_plan(p16)
+    c1632, r1632 = _lib.forward_backward_plan(p16_32)
+    assert c32 > 1 and c16 > 1 and c1632 > 1
+    plane, copy = 1024 * 32768 * 4, 1024 * 32768 * 2
+    assert r1632 >= r16  # without the plane there is room for longer chunks
+    assert _lib.forward_backward_workspace_bytes(p32) >= copy + r32 * 32768 * 2
+    assert _lib.forward_backward_workspace_bytes(p16) >= plane + r16 * 32768 * 2
+    assert _lib.forward_backward_workspace_bytes(p16_32) < plane + r1632 * 32768 * 2

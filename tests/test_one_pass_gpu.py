@@ -22,18 +22,20 @@ def _problem(N, H, V, x, w, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, phas
     from linear_cross_entropy_loss_amd import _lib
 
     hp, cols = H + (-H) % 8, (H if layout else V)
-    return _lib.make_problem(N, H, V, x.stride(0), w.stride(0), hp, cols + (-cols) % 8, dt, dt, dt, dw_dt, -1, scale,
+    return _lib.make_problem(N, H, V, x.stride(0), w.stride(0), hp, cols + (-cols) % 8, dt, w.dtype, dt, dw_dt, -1, scale,
                              z_reg, n_chunk, False, phases, pack, 0, layout, _lib.ROUTE_ONE_PASS)
 
 
 def _both_routes(N, H, V, dt, n_chunk, ignore, z_reg=0.0, scale=1.0, pack=0, layout=0, dw_dt=None, grad_out=1.0,
-                 seed=7, want_chunks=None):
+                 seed=7, want_chunks=None, w_dt=None):
     """Runs the two routes on the same inputs; returns (inputs on the CPU, two-pass outputs, one-pass outputs)."""
     from linear_cross_entropy_loss_amd import _lib
 
     lib = _lib.load()
-    x, y, w = make_inputs(N, H, V, dt, seed, ignore_frac=ignore)
+    x, y, w = make_inputs(N, H, V, dt, seed, ignore_frac=ignore, w_dtype=w_dt)
     xd, yd, wd = x.cuda(), y.cuda(), (w.t().contiguous() if layout else w).cuda()
+    if w_dt is not None:
+        dw_dt = w_dt  # (the gradient of an fp32 master weight is fp32)
     if wd.stride(0) % 8:  # rows of the weight on 16-byte boundaries
         pad = torch.zeros(wd.shape[0], wd.shape[1] + (-wd.shape[1]) % 8, dtype=wd.dtype, device="cuda")
         pad[:, :wd.shape[1]] = wd
@@ -117,6 +119,22 @@ CASES = [
     (1000, 300, 777, torch.float16, 4096, 0.2, 0.0, 2.0, 1, 0, None, 1.0),          # single chunk, nothing a multiple of 8
     (8192, 1024, 32768, torch.bfloat16, 4096, 0.05, 0.0, 1.0, 0, 0, None, 1.0),     # mid size: 3 chunks
 ]
+
+# fp32 master weight under 16-bit activations: N, H, V, dtype of x, n_chunk, ignored, z_reg, scale, pack, layout
+MASTER_CASES = [
+    (4096, 512, 4096, torch.bfloat16, 2048, 0.1, 0.0, 1.0, 1, 0),
+    (4000, 520, 5000, torch.float16, 2048, 0.1, 1e-3, 0.7, 1, 0),
+    (4000, 520, 5000, torch.bfloat16, 2048, 0.3, 0.0, 1.0, 2, 1),
+    (1000, 304, 777, torch.float16, 4096, 0.2, 0.0, 2.0, 1, 0),      # a single chunk
+]
+
+
+@pytest.mark.pack_auto
+@pytest.mark.parametrize("N,H,V,dt,n_chunk,ign,z_reg,scale,pack,layout", MASTER_CASES)
+def test_one_pass_with_an_fp32_master_weight(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout):
+    inputs, a, b = _both_routes(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout, w_dt=torch.float32)
+    assert b["dw"].dtype == torch.float32
+    _check(inputs, a, b, z_reg, scale, 1.0, fp64=True)
 
 
 @pytest.mark.pack_auto
