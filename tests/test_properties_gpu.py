@@ -666,19 +666,27 @@ def test_function_and_registered_operator_agree_bitwise():
             assert torch.equal(a, b)
 
 
-def test_forward_backward_can_be_captured_in_a_hip_graph():
+@pytest.mark.parametrize("one_pass", [False, True])
+def test_forward_backward_can_be_captured_in_a_hip_graph(one_pass):
     """The library only enqueues kernels on the caller's stream (no synchronisation, no memset nodes, no
     allocation of its own), so a whole loss + backward step can be captured once and replayed; every replay,
-    with eager work and synchronisations in between, must equal the eager result bit for bit."""
-    from linear_cross_entropy_loss_amd import linear_cross_entropy
+    with eager work and synchronisations in between, must equal the eager result bit for bit.  On both routes:
+    two passes (here with the monitoring values), and loss and gradients from one evaluation of the logits in
+    several chunks of token rows, whose row counts the kernels also take from device memory."""
+    from linear_cross_entropy_loss_amd import _lib, linear_cross_entropy, ops
 
-    print("hip graph capture", flush=True)
-    N, H, V = 1024, 512, 10000
+    print(f"hip graph capture, one pass: {one_pass}", flush=True)
+    N, H, V = (4096 if one_pass else 1024), 512, 10000
     x, y, w = make_inputs(N, H, V, torch.bfloat16, seed=3, ignore_frac=0.1, device="cuda")
     xs, ws, ys = x.clone().requires_grad_(True), w.clone().requires_grad_(True), y.clone()
+    if one_pass:
+        ops.one_pass.set("always")  # (the autouse fixtures of conftest.py put the default back)
+        prob = _lib.make_problem(N, H, V, H, V, H, V, torch.bfloat16, torch.bfloat16, torch.bfloat16, torch.bfloat16, -1,
+                                 1.0, 1e-4, 1500, False, 0, int(ops.pack_rows.get()), 0, 0, _lib.ROUTE_ONE_PASS)
+        assert _lib.forward_backward_plan(prob)[0] > 1
 
     def step(xi, yi, wi):
-        out = linear_cross_entropy(xi, yi, wi, -1, 1e-4, 1.0, 512, True)
+        out = linear_cross_entropy(xi, yi, wi, -1, 1e-4, 1.0, 1500 if one_pass else 512, not one_pass)
         out[0].backward()
         return out
 
