@@ -96,7 +96,7 @@ def time_phases_one_pass(cfg, x, y, w, prob, chunks, torch, reps):
     rows = int(nv.item()) if 8.0 * N * H * V >= 2.0 ** 41 else N
     out = {}
     for name, ph, flops, nbytes in (
-        ("fwd_stage", _lib.PHASE_FWD_TILES, 2.0 * rows * H * V / chunks, 0.0),
+        ("fwd_stage", _lib.PHASE_FWD_TILES, 2.0 * (N if cfg["monitoring"] else rows) * H * V / chunks, 0.0),
         # 2 bytes read and 2 written per logit: bound by memory traffic, not by matrix instructions
         ("stage_scale", _lib.PHASE_BWD_DZ, 0.0, 4.0 * rows * V / chunks),
         ("bwd_dx", _lib.PHASE_BWD_DX, 2.0 * rows * H * V / chunks, 0.0),
@@ -138,7 +138,7 @@ def time_phases(cfg, x, y, w, torch, reps=5, one_pass=True):
                                  _lib.W_VH if vh else _lib.W_HV)
 
     chunks, _ = _lib.forward_backward_plan(prob(0))
-    if chunks > 0 and not cfg["monitoring"] and one_pass:
+    if chunks > 0 and one_pass:
         return time_phases_one_pass(cfg, x, y, w, prob, chunks, torch, reps)
     fwd_b, bwd_b = _lib.workspace_bytes(prob(0))
     # one workspace per call: a call restricted to one kernel relies on what the full call left in it
@@ -463,14 +463,14 @@ def main():
     peak = PEAK_TFLOPS[cfg["dtype"]]
     # which route the steps above took (ops.LinearXentImplementation.forward decides the same way)
     route = "two_pass"
-    if not args.two_pass and not cfg["monitoring"] and cfg["dtype"] != "f32":
+    if not args.two_pass and cfg["dtype"] != "f32":
         wr = w.detach().t() if cfg.get("w_vh") else w.detach()
         pr = _lib.make_problem(N, H, V, x.stride(0), wr.stride(0), H, wr.stride(0), x.dtype, wr.dtype, x.dtype, wr.dtype, -1,
-                               cfg["scale"], cfg["z_reg"], cfg["n_chunk"], False, 0, 0, 0,
+                               cfg["scale"], cfg["z_reg"], cfg["n_chunk"], cfg["monitoring"], 0, 0, 0,
                                _lib.W_VH if cfg.get("w_vh") else _lib.W_HV)
         if _lib.forward_backward_plan(pr)[0] > 0:
             route = "one_pass"
-    flops_executed = flops if route == "two_pass" else 6.0 * rows * H * V
+    flops_executed = flops if route == "two_pass" else (2.0 * (N if cfg["monitoring"] else rows) + 4.0 * rows) * H * V
 
     ms_median = median_step_ms(step, torch, reps=20, flush=False)
     ms_median_flushed = median_step_ms(step, torch, reps=20, flush=True)

@@ -333,7 +333,7 @@ struct FusedPlan {
   int64_t nc;
   int chunks;
   PackPlan k;
-  size_t chunk_rows, lse_rows, tgt, blk, w16, xc, part_lse, part_max, stage, plane, part, total;
+  size_t chunk_rows, lse_rows, tgt, blk, w16, xc, part_lse, part_max, part_pz, part_sq, stage, plane, part, total;
   int64_t ld16;    // row stride of the 16-bit copy of an fp32 weight
   bool parts_on;
   bool dw_direct;  // fp32 dW: the chunks' terms are added in the caller's buffer, there is no plane
@@ -342,11 +342,15 @@ struct FusedPlan {
 bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) {
   memset(f, 0, sizeof(*f));
   const bool x16 = p->x_dtype == LCE_BF16 || p->x_dtype == LCE_F16;
-  if (!x16 || (p->w_dtype != p->x_dtype && p->w_dtype != LCE_F32) || p->monitoring || p->route == LCE_ROUTE_TWO_PASS) return false;
+  if (!x16 || (p->w_dtype != p->x_dtype && p->w_dtype != LCE_F32) || p->route == LCE_ROUTE_TWO_PASS) return false;
+  // (the logit kernel of this route has no variant with both the monitoring sums and a K mask: lce_bwd_dz.hip)
+  if (p->monitoring && lce::padded_k(p->H) != p->H) return false;
   const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V), Hp = (size_t)lce::padded_hidden(p->H);
   const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
   // (packed rows of dx go to their tokens through 32-bit offsets into dx)
-  f->pack = packs_rows(p) && (size_t)p->N * (size_t)p->lddx * dxes < ((size_t)1 << 31);
+  // (the monitoring values are taken over all rows: nothing is packed away then, and the pass over the stage
+  // zeroes the rows of tokens with an ignored label)
+  f->pack = !p->monitoring && packs_rows(p) && (size_t)p->N * (size_t)p->lddx * dxes < ((size_t)1 << 31);
   f->dw_direct = p->dw_dtype == LCE_F32;
   f->k = plan_pack(p, 0, false);
   size_t o = f->k.xc;  // the labels are always counted; the packed copy of x is made chunk by chunk (below)
@@ -369,6 +373,8 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     const size_t part = align_up(Vp / lce::kChunkV * (size_t)nc * 4);
     out->part_lse = t; t += part;
     out->part_max = t; t += part;
+    out->part_pz = t; if (p->monitoring) t += part;
+    out->part_sq = t; if (p->monitoring) t += part;
     out->stage = t; t += align_up((size_t)nc * Vp * 2);
     // split-K partial sums of dx (and, with a single chunk, of dW): one buffer
     size_t pb = want_dx ? dx_part_bytes((size_t)nc, Hp, (int64_t)Vp, (int64_t)Vp) : 0;
@@ -600,9 +606,12 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
   fa.Np = Np; fa.Vp = Vp;
   fa.x_dtype = p->x_dtype; fa.w_dtype = p->w_dtype;
   fa.ignore_index = p->ignore_index;
-  fa.scale = p->logit_scale; fa.z_reg = p->z_reg; fa.monitoring = 0;
+  fa.scale = p->logit_scale; fa.z_reg = p->z_reg; fa.monitoring = p->monitoring ? 1 : 0;
   fa.lse = lse; fa.out5 = out5; fa.n_valid = n_valid;
   fa.part_lse = (float*)(base + f.part_lse);
+  fa.part_max = (float*)(base + f.part_max);
+  fa.part_pz = (float*)(base + f.part_pz);
+  fa.part_sq = (float*)(base + f.part_sq);
   fa.tgt = (float*)(base + f.tgt);
   fa.blk = (float*)(base + f.blk);
   fa.lse_rows = (float*)(base + f.lse_rows);
@@ -658,6 +667,8 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
   b.live = lce::live_bands(lce::padded_k(p->H) * 2);
   b.part_lse = (float*)(base + f.part_lse);
   b.part_max = (float*)(base + f.part_max);
+  b.part_pz = p->monitoring ? (float*)(base + f.part_pz) : nullptr;
+  b.part_sq = p->monitoring ? (float*)(base + f.part_sq) : nullptr;
   b.nc = f.nc;
   b.dx_part = f.parts_on && dx ? (float*)(base + f.part) : nullptr;
   b.dw_part = f.parts_on && dw && f.chunks == 1 ? (float*)(base + f.part) : nullptr;

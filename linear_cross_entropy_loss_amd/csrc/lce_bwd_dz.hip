@@ -66,9 +66,12 @@ constexpr int kDzStoreAux = LCE_DZ_STORE_AUX;  // cache policy of the dz stores:
 // FUSE (launch_fwd_stage: the logits are computed once, for the loss and for the gradients): the tile leaves
 // e = 2^dz_shift * exp(z - m) instead, m = the largest logit of the token within this wave's 128 columns, for
 // every row, whatever its label; the wave also writes the forward's partials of its slice (m and
-// m + log sum exp(z - m)) and the target logit.  `pf_lse` is not used.
+// m + log sum exp(z - m)) and the target logit.  `pf_lse` is not used, and there is no gain to apply: under FUSE the
+// switch ZREG stands for the monitoring values instead (the slice's sum softmax * z and sum z^2, as lce_fwd.hip forms them).
+constexpr int kNoLabel = -0x7fffffff - 1;  // ignore_index, or no such row
+constexpr int kOffLabel = -1;              // a label that is no column of W (V <= 2^30): matches nothing
 template <class T, bool ZREG, bool VTAIL, bool SPLIT, bool FUSE>
-LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], const float (&pf_lse)[kNB],
+LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int (&pf_y)[kNB], const float (&pf_lse)[kNB],
                               f32x16_t (&acc)[kNB][kNB], int tp, int tq, char* pieces) {
   typedef typename elem_of<T>::type E;
   const int64_t v0 = a.v0 + (int64_t)tp * kTile, t0 = (int64_t)tq * kTile;
@@ -90,6 +93,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
   E* wave_base = reinterpret_cast<E*>(a.dz) + dz_block_offset(tq, tp * (kTile / kGroup) + wpu * (kWaveTile / kGroup), a.vs) +
                  wqu * kWaveTile * kGroup;
   E* row = wave_base + (lane & 31) * kGroup;
+  constexpr bool MON = FUSE && ZREG;
   const int64_t blk = a.Np * a.vs;  // SPLIT: elements between the three parts of the stage
   // Stores go through a buffer descriptor over this wave's part of the stage (scalar base, one 32-bit offset per
   // lane, the block's offset as a scalar): no 64-bit vector address arithmetic.  All offsets stay below 2^31
@@ -108,9 +112,10 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
   int ykey[kNB];
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
-    const int64_t yy = pf_y[qb];  // (rows past the last one are staged as zeros, like ignored tokens)
-    const int64_t rel = yy - slice_v0;
-    const bool valid = yy != a.ignore_index;
+    // (rows past the last one are staged as zeros, like ignored tokens)
+    const int yy = pf_y[qb];  // the label as DzProblem::prefetch keeps it: kNoLabel, or the column (kOffLabel: none of W's)
+    const int64_t rel = (int64_t)yy - slice_v0;
+    const bool valid = yy != kNoLabel;
     const float l = FUSE ? 0.f : pf_lse[qb];
     // (the power-of-two factor of the staged dz rides along in the exponent)
     nlse[qb] = valid ? fmaf(-l, kLog2e, (float)a.dz_shift) : -INFINITY;  // (FUSE: set per block below)
@@ -123,7 +128,7 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
 
 #pragma unroll
   for (int qb = 0; qb < kNB; ++qb) {
-    float m = -INFINITY, ssum = 0.f;
+    float m = -INFINITY, ssum = 0.f, mpz = 0.f, msq = 0.f;
     if constexpr (FUSE) {
       // the largest of this token's logits in the slice: this lane's 64, then the other half's
 #pragma unroll
@@ -152,15 +157,27 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
           if (!VTAIL || pb * 4 + g + h2 < nq) {
 #pragma unroll
             for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
-              d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
-              if (ZREG) d[i] *= gain[qb];
+              const float zr = acc[pb][qb][g * 4 + i];
+              d[i] = __builtin_amdgcn_exp2f(fmaf(zr, c1, nlse[qb]));
+              if (ZREG && !FUSE) d[i] *= gain[qb];
+              if constexpr (MON) {
+                const float z = zr * a.scale;
+                mpz = fmaf(d[i], z, mpz);
+                msq = fmaf(z, z, msq);
+              }
             }
           } else if (pb * 4 + g + h2 == nq && cut != 0) {
 #pragma unroll
             for (int i = 4 * h2; i < 4 * h2 + 4; ++i) {
-              d[i] = __builtin_amdgcn_exp2f(fmaf(acc[pb][qb][g * 4 + i], c1, nlse[qb]));
-              if (ZREG) d[i] *= gain[qb];
+              const float zr = acc[pb][qb][g * 4 + i];
+              d[i] = __builtin_amdgcn_exp2f(fmaf(zr, c1, nlse[qb]));
+              if (ZREG && !FUSE) d[i] *= gain[qb];
               d[i] = (i - 4 * h2) < cut_mine ? d[i] : 0.f;
+              if constexpr (MON) {
+                const float z = zr * a.scale;
+                mpz = fmaf(d[i], z, mpz);
+                msq = (i - 4 * h2) < cut_mine ? fmaf(z, z, msq) : msq;
+              }
             }
           } else {
 #pragma unroll
@@ -227,6 +244,14 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int64_t (&pf_y)[kNB], cons
         a.part_max[o] = m * a.scale;
         a.part_lse[o] = ssum > 0.f ? fmaf(m, a.scale, (__builtin_amdgcn_logf(ssum) - (float)a.dz_shift) * 0.6931471805599453f)
                                    : -INFINITY;
+      }
+      if constexpr (MON) {
+        mpz += __shfl_xor(mpz, 32);
+        msq += __shfl_xor(msq, 32);
+        if (lane < 32) {
+          a.part_pz[o] = ssum > 0.f ? mpz / ssum : 0.f;  // (both sums carry the factor 2^dz_shift)
+          a.part_sq[o] = msq;
+        }
       }
       if (yl >= 0) {
         const int want = (yl >> 5) * 16 + ((yl >> 3) & 3) * 4 + (yl & 3);  // (block, register) index
@@ -315,7 +340,7 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH, bool
   LCE_DEV int k_valid(int) const { return (int)a.H; }
   // The epilogue starts with the label and lse of each of this lane's four tokens: fetched while the last K tiles
   // of the tile are still being multiplied, instead of one exposed round trip to memory per tile.
-  int64_t pf_y[kNB];
+  int pf_y[kNB];  // kNoLabel / kOffLabel / the column: four registers held over the last K tiles instead of eight
   float pf_lse[kNB];
   LCE_DEV void prefetch(int tile) {
     int tp, tq;
@@ -325,7 +350,8 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH, bool
     for (int qb = 0; qb < kNB; ++qb) {
       const int64_t tok = (int64_t)tq * kTile + wq * kWaveTile + qb * kBlk + (lane & 31);
       const bool exists = tok < rows;
-      pf_y[qb] = exists ? a.y[tok] : a.ignore_index;
+      const int64_t yy = exists ? a.y[tok] : a.ignore_index;
+      pf_y[qb] = yy == a.ignore_index ? kNoLabel : (yy >= 0 && yy < a.V ? (int)yy : kOffLabel);
       pf_lse[qb] = exists && !FUSE ? a.lse[tok] : 0.f;
     }
   }
@@ -362,8 +388,16 @@ hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
   const int64_t tq = a.Np / kTile, full = a.vw / kTile, tail = a.vs / kTile - full;
   const bool exact_k = padded_k(a.H) == a.H;  // the K tiles cover H exactly: no K mask needed
   if (full > 0) {
-    hipError_t e = exact_k ? launch_one<T, ZREG, false, false, SPLIT, WVH, FUSE>(a, full * tq, s)
-                           : launch_one<T, ZREG, false, true, SPLIT, WVH, FUSE>(a, full * tq, s);
+    hipError_t e;
+    if constexpr (FUSE && ZREG) {
+      // (the monitoring sums on top of the K mask do not fit the registers; such problems -- a hidden size that is not
+      // a multiple of 128 -- take two passes, lce_api.hip)
+      if (!exact_k) return hipErrorInvalidValue;
+      e = launch_one<T, ZREG, false, false, SPLIT, WVH, FUSE>(a, full * tq, s);
+    } else {
+      e = exact_k ? launch_one<T, ZREG, false, false, SPLIT, WVH, FUSE>(a, full * tq, s)
+                  : launch_one<T, ZREG, false, true, SPLIT, WVH, FUSE>(a, full * tq, s);
+    }
     if (e != hipSuccess) return e;
   }
   if (tail > 0) return launch_one<T, ZREG, true, true, SPLIT, WVH, FUSE>(a, tail * tq, s);
@@ -391,14 +425,17 @@ hipError_t launch_bwd_dz(const BwdArgs& a, hipStream_t s) {
   return hipErrorInvalidValue;
 }
 
+template <class T, bool WVH> hipError_t launch_stage(const BwdArgs& a, hipStream_t s) {
+  // (the second template argument: the monitoring values, see dz_epilogue_impl)
+  return a.part_pz != nullptr ? launch_persistent_z<T, true, false, WVH, true>(a, s)
+                              : launch_persistent_z<T, false, false, WVH, true>(a, s);
+}
+
 hipError_t launch_fwd_stage(const BwdArgs& a, hipStream_t s) {
   if (a.split || a.part_lse == nullptr || a.part_max == nullptr || a.tgt == nullptr) return hipErrorInvalidValue;
-  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16)
-    return a.w_vh ? launch_persistent_z<BF16, false, false, true, true>(a, s)
-                  : launch_persistent_z<BF16, false, false, false, true>(a, s);
-  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16)
-    return a.w_vh ? launch_persistent_z<F16, false, false, true, true>(a, s)
-                  : launch_persistent_z<F16, false, false, false, true>(a, s);
+  if ((a.part_pz == nullptr) != (a.part_sq == nullptr)) return hipErrorInvalidValue;
+  if (a.x_dtype == DT_BF16 && a.w_dtype == DT_BF16) return a.w_vh ? launch_stage<BF16, true>(a, s) : launch_stage<BF16, false>(a, s);
+  if (a.x_dtype == DT_F16 && a.w_dtype == DT_F16) return a.w_vh ? launch_stage<F16, true>(a, s) : launch_stage<F16, false>(a, s);
   return hipErrorInvalidValue;
 }
 

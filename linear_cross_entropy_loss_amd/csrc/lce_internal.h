@@ -157,6 +157,8 @@ struct BwdArgs {
   // tgt (first row of the chunk).  Once the rows' lse are known, launch_stage_scale turns e into dz in place.
   float* part_lse;
   float* part_max;
+  float* part_pz;  // both null, or the monitoring partials of FwdArgs as well
+  float* part_sq;
   float* tgt;
   int64_t nc;
   // rows of dx always go to the tokens perm[] names (the rows of a chunk can be all there and still not be the

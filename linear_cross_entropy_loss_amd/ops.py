@@ -14,7 +14,7 @@ The device work is done by hand-written gfx950 kernels behind the C ABI of
 When a gradient is wanted, ``forward`` computes it along with the loss from one
 evaluation of the logits (``lce_forward_backward``), as the reference's forward
 does (``ops.py:721-791``), and ``backward`` multiplies the upstream gradient in
-(``ops.py:810``).  Problems that route does not cover (fp32 tensors, monitoring,
+(``ops.py:810``).  Problems that route does not cover (fp32 activations,
 shapes whose scratch bound leaves no room for it) and forward-only calls compute
 only the loss in ``forward`` and save ``lse``; their ``backward`` recomputes the
 logit tiles (``lce_backward``).  So does a second ``backward`` over the same graph.
@@ -196,7 +196,8 @@ def _finish_grads(dx, dw, layout):
     return dx, dw
 
 
-def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, pack, need_dx, need_dw):
+def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack, need_dx,
+                   need_dw):
     """Runs lce_forward_backward when its one-pass route covers the problem.  Returns None otherwise, else
     (out5, lse, n_valid, x, y1, w, layout, dx, dw, pre): the gradients for an upstream gradient of `pre` (a device
     scalar; None stands for 1)."""
@@ -208,7 +209,7 @@ def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_c
         w_cols = H if vh else V
         prob = _lib.make_problem(
             N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, w_cols + (-w_cols) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
-            ignore_index, logit_scale, z_regularization, N_chunk_size, False, 0, pack, 0, layout,
+            ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring, 0, pack, 0, layout,
             _lib.ROUTE_ONE_PASS if one_pass.get() == "always" else _lib.ROUTE_AUTO,
         )
         lib = _lib.load()
@@ -346,8 +347,8 @@ class LinearXentImplementation(torch.autograd.Function):
         pack = _pack_mode()
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[2]
         done = None
-        if (need_dx or need_dw) and not monitoring and one_pass.get():
-            done = _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, pack,
+        if (need_dx or need_dw) and one_pass.get():
+            done = _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack,
                                   need_dx, need_dw)
         if done is not None:
             out5, lse, n_valid, x, y1, w, layout, dx, dw, pre = done

@@ -497,11 +497,15 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
     prob = _lib.make_problem(16384, 2048, 131072, 2048, 131072, 2048, 131072, torch.bfloat16, torch.bfloat16,
                              torch.bfloat16, torch.bfloat16, -1, 1.0, 0.0, 4096, False)
     assert _lib.forward_backward_plan(prob) == (5, 3328)
-    for kw in (dict(x=torch.float32, w=torch.float32), dict(mon=True)):
-        xd, wd = kw.get("x", torch.bfloat16), kw.get("w", torch.bfloat16)
-        prob = _lib.make_problem(4096, 512, 8192, 512, 8192, 512, 8192, xd, wd, xd, wd, -1, 1.0, 0.0, 4096,
-                                 kw.get("mon", False))
+    # no one-pass route for fp32 activations, nor for the monitoring values with a hidden size that needs the K mask
+    for kw in (dict(x=torch.float32, w=torch.float32), dict(mon=True, H=520)):
+        xd, wd, Hh = kw.get("x", torch.bfloat16), kw.get("w", torch.bfloat16), kw.get("H", 512)
+        prob = _lib.make_problem(4096, Hh, 8192, Hh, 8192, Hh, 8192, xd, wd, xd, wd, -1, 1.0, 0.0, 4096,
+                                 kw.get("mon", False), route=_lib.ROUTE_ONE_PASS)
         assert _lib.forward_backward_plan(prob) == (0, 0), kw
+    prob = _lib.make_problem(4096, 512, 8192, 512, 8192, 512, 8192, torch.bfloat16, torch.bfloat16, torch.bfloat16,
+                             torch.bfloat16, -1, 1.0, 0.0, 4096, True, route=_lib.ROUTE_ONE_PASS)
+    assert _lib.forward_backward_plan(prob)[0] > 0  # monitoring with H a multiple of 128: covered
     # an fp32 master weight under 16-bit activations: one 16-bit copy of all of it in the workspace, and its fp32 gradient
     # is summed over the chunks in the caller's buffer (no plane)
     kw = dict(N=8192, H=1024, V=32768, ldx=1024, ldw=32768, lddx=1024, lddw=32768, x_dtype=torch.bfloat16,

@@ -18,16 +18,16 @@ def P(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
 
-def _problem(N, H, V, x, w, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, phases=0):
+def _problem(N, H, V, x, w, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, phases=0, mon=False):
     from linear_cross_entropy_loss_amd import _lib
 
     hp, cols = H + (-H) % 8, (H if layout else V)
     return _lib.make_problem(N, H, V, x.stride(0), w.stride(0), hp, cols + (-cols) % 8, dt, w.dtype, dt, dw_dt, -1, scale,
-                             z_reg, n_chunk, False, phases, pack, 0, layout, _lib.ROUTE_ONE_PASS)
+                             z_reg, n_chunk, mon, phases, pack, 0, layout, _lib.ROUTE_ONE_PASS)
 
 
 def _both_routes(N, H, V, dt, n_chunk, ignore, z_reg=0.0, scale=1.0, pack=0, layout=0, dw_dt=None, grad_out=1.0,
-                 seed=7, want_chunks=None, w_dt=None):
+                 seed=7, want_chunks=None, w_dt=None, mon=False):
     """Runs the two routes on the same inputs; returns (inputs on the CPU, two-pass outputs, one-pass outputs)."""
     from linear_cross_entropy_loss_amd import _lib
 
@@ -45,7 +45,7 @@ def _both_routes(N, H, V, dt, n_chunk, ignore, z_reg=0.0, scale=1.0, pack=0, lay
         pad[:, :H] = xd
         xd = pad[:, :H]
     dw_dt = dw_dt or dt
-    prob = _problem(N, H, V, xd, wd, dt, dw_dt, z_reg, scale, n_chunk, pack, layout)
+    prob = _problem(N, H, V, xd, wd, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, mon=mon)
     chunks, rows = _lib.forward_backward_plan(prob)
     print(f"N={N} H={H} V={V} {dt} n_chunk={n_chunk} pack={pack} layout={layout}: {chunks} chunks of {rows} rows", flush=True)
     assert chunks > 0, "this case is meant to take the one-pass route"
@@ -142,6 +142,34 @@ def test_one_pass_with_an_fp32_master_weight(N, H, V, dt, n_chunk, ign, z_reg, s
 def test_one_pass_matches_two_pass_and_the_fp64_oracle(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout, dw_dt, grad_out):
     inputs, a, b = _both_routes(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout, dw_dt, grad_out)
     _check(inputs, a, b, z_reg, scale, grad_out, fp64=N * V <= 4096 * 8192)
+
+
+# the monitoring values on the one-pass route (the forward then runs on all rows): N, H, V, dtype, n_chunk, ignored, z_reg,
+# scale, pack, layout
+MON_CASES = [
+    (4096, 512, 4096, torch.bfloat16, 2048, 0.1, 1e-4, 1.0, 1, 0),
+    (4000, 512, 5000, torch.float16, 2048, 0.3, 1e-3, 0.5, 2, 0),    # the tile column that straddles V
+    (4000, 640, 5000, torch.bfloat16, 2048, 0.1, 0.0, 2.0, 1, 1),    # weight stored (V, H)
+    (1000, 384, 777, torch.float16, 4096, 0.2, 0.0, 1.0, 0, 0),      # a single chunk
+]
+
+
+@pytest.mark.pack_auto
+@pytest.mark.parametrize("N,H,V,dt,n_chunk,ign,z_reg,scale,pack,layout", MON_CASES)
+def test_one_pass_with_the_monitoring_values(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout):
+    inputs, a, b = _both_routes(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout, mon=True)
+    _check(inputs, a, b, z_reg, scale, 1.0, fp64=True)
+    # logit_max exactly, entropy and norm to fp32 summation order
+    assert a["out5"][2].item() == b["out5"][2].item()
+    for i in (3, 4):
+        assert abs(a["out5"][i].item() - b["out5"][i].item()) <= 2e-5 * abs(a["out5"][i].item()), (i, a["out5"], b["out5"])
+    from oracle import lce_forward_backward_fp64
+
+    x, y, w = inputs
+    ref = lce_forward_backward_fp64(x.double(), y, w.double(), -1, z_reg, scale, 1.0)
+    assert abs(b["out5"][2].item() - ref.logit_max.item()) <= 1e-3 * abs(ref.logit_max.item())
+    assert abs(b["out5"][3].item() - ref.logit_entropy.item()) <= 2e-3 * abs(ref.logit_entropy.item())
+    assert abs(b["out5"][4].item() - ref.logit_norm.item()) <= 2e-3 * abs(ref.logit_norm.item())
 
 
 @pytest.mark.pack_auto
