@@ -323,7 +323,8 @@ int plan_bwd(const lce_problem* p, BwdPlan* b) {
 // lce_forward_backward: the logits are computed once.  The tokens go through in chunks of `nc` rows against the
 // whole vocabulary: logit kernel (partials of the loss, and e = exp(z - slice max) into the stage), row merge
 // (lse), the pass that turns e into dz, then dx of the chunk (complete: K = the vocabulary) and the chunk's
-// term of dW, which is summed over the chunks in an fp32 plane (the reference's fp32 At_grad, ops.py:692).
+// term of dW, which is summed over the chunks in fp32 (the reference's fp32 At_grad, ops.py:692): in the caller's
+// buffer if dW is fp32, else as 16-bit halves -- the upper ones in the caller's dW, the lower ones in a plane here.
 // Everything counts towards the bound n_chunk * V * 4 (the reference's logits chunk, ops.py:700): the chunk is
 // the longest that fits.  Problems outside the set below -- and those whose plane alone does not fit -- take the
 // two-pass route (forward, then a backward that recomputes the logits).
@@ -333,7 +334,7 @@ struct FusedPlan {
   int64_t nc;
   int chunks;
   PackPlan k;
-  size_t chunk_rows, lse_rows, tgt, blk, w16, xc, part_lse, part_max, part_pz, part_sq, stage, plane, part, total;
+  size_t chunk_rows, lse_rows, tgt, blk, w16, xc, part_lse, part_max, part_pz, part_sq, stage, plane, plane_hi, part, total;
   int64_t ld16;    // row stride of the 16-bit copy of an fp32 weight
   bool parts_on;
   bool dw_direct;  // fp32 dW: the chunks' terms are added in the caller's buffer, there is no plane
@@ -385,7 +386,11 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     out->part = t; t += pb;
     out->parts_on = pb != 0;
     out->plane = t;
-    if (chunks > 1 && want_dw && !f->dw_direct) t += align_up(Hp * Vp * 4);
+    if (chunks > 1 && want_dw && !f->dw_direct) t += align_up(Hp * Vp * 2);
+    // (upper halves of the tiles that the edge of dW cuts: the last tile row over h, the last over v)
+    out->plane_hi = t;
+    if (chunks > 1 && want_dw && !f->dw_direct)
+      t += align_up(((Hp != (size_t)p->H ? Vp / 256 : 0) + (Vp != (size_t)p->V ? Hp / 256 : 0)) * (size_t)(256 * 256 * 2));
     out->total = t;
     return t;
   };
@@ -672,7 +677,8 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
   b.nc = f.nc;
   b.dx_part = f.parts_on && dx ? (float*)(base + f.part) : nullptr;
   b.dw_part = f.parts_on && dw && f.chunks == 1 ? (float*)(base + f.part) : nullptr;
-  b.dw_plane = f.chunks > 1 && !f.dw_direct ? (float*)(base + f.plane) : nullptr;
+  b.dw_plane = f.chunks > 1 && !f.dw_direct ? (void*)(base + f.plane) : nullptr;
+  b.dw_plane_hi = f.chunks > 1 && !f.dw_direct && f.total != f.plane_hi ? (void*)(base + f.plane_hi) : nullptr;
 
   for (int c = 0; c < f.chunks; ++c) {
     const int64_t row0 = (int64_t)c * f.nc;

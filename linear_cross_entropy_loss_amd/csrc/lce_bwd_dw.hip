@@ -188,44 +188,87 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
   }
 }
 
-// dW summed over chunks of token rows (BwdArgs::dw_plane): the tile's block of the plane holds the accumulator
-// as the registers do -- quad (rb, cbk, rq) of thread t at float 4 * (((rb * 4 + cbk) * 4 + rq) * 256 + t) -- so
-// that every load and store of a wave covers 1 KiB of consecutive addresses.  LOAD: the block is added to the
-// accumulator before the sums go (back) to the block.  After the last chunk dw_plane_out_kernel scales the sums
-// and stores dW.  (Hardware fp32 atomic adds instead of the load - add - store were measured at the headline shape:
-// the 268 M atomics of a chunk take longer than the chunk's matrix work, 30.6 ms a step against 22.3.)
 #ifndef LCE_DW_PLANE_BATCH
 #define LCE_DW_PLANE_BATCH 16
 #endif
-template <bool LOAD>
-LCE_DEV void dw_plane_io(float* blk, f32x16_t (&acc)[kNB][kNB]) {
-  // one descriptor over the block, the thread's 16 bytes as the vector offset, the quad as a scalar offset: no
-  // 64-bit address per quad
-  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(blk, 0, kTile * kTile * 4, 0x00020000);
-  const int voff = opaque_tid() * 16;
-  // kPlaneBatch quads are fetched together before any is used: the loads of a batch are in flight together, and a
-  // tile waits for 64 / kPlaneBatch round trips to memory
-  constexpr int kPlaneBatch = LCE_DW_PLANE_BATCH;
+// dW summed over chunks of token rows when dW is 16-bit (BwdArgs::dw_plane): the fp32 sums of a tile are kept as two
+// 16-bit halves.  The upper halves lie in the caller's dW itself, in the 256 rows x 512 bytes that the tile's
+// results will take -- nothing else needs that memory before the last chunk is done --, the lower halves in a
+// 128 KiB block of the plane; a tile that the matrix' edge cuts has no whole region of dW, and its upper halves
+// go to a block of BwdArgs::dw_plane_hi.  Both halves together are the fp32 sum, bit for bit.
+//   Two register quads of a thread (the pair p: quads 2p and 2p+1, eight sums) give 16 bytes of upper and 16 of
+// lower halves.  Lower halves: pair p of thread t at byte p * 4096 + t * 16 of the block.  Upper halves: each
+// wave keeps to the 128 rows x 256 bytes of its own quarter of the tile's results, and within those the eight
+// pairs of one block row of results (32 rows) to the 32 rows x 256 bytes that these results will take: pair
+// j = 2 * column block + rq / 2 of a block row is 4 rows, a lane's 16 bytes at row 4 j + lane / 16, byte
+// (lane % 16) * 16.  So dw_plane_split_out_kernel can turn the sums into dW in place, 32 rows at a time.
+// (Hardware fp32 atomic adds into an fp32 plane instead of load - add - store were measured at the headline
+// shape: the 268 M atomics of a chunk take longer than the chunk's matrix work, 30.6 ms a step against 22.3.)
+constexpr unsigned kSelLow = 0x05040100u, kSelHigh = 0x07060302u;  // v_perm selectors: the lower / upper halves of (S0, S1)
+
+// Where the upper halves of tile (tp, tq) lie, and the distance of their rows in bytes.
+template <bool WVH>
+LCE_DEV char* dw_hi_block(const BwdArgs& a, int tp, int tq, int& stride) {
+  const DwTileGeom<WVH> g(a, tp, tq);
+  if (g.row0 + kTile <= g.row_limit && g.col0 + kTile <= g.col_limit) {
+    stride = (int)a.lddw * 2;
+    return reinterpret_cast<char*>(a.dw) + (g.row0 * a.lddw + g.col0) * 2;
+  }
+  // tiles cut by the edge, numbered: those of the last tile row over h first (if H cuts it), then the last over v
+  const int tiles_p = (int)(a.Hp / kTile), tiles_q = (int)(a.vs / kTile);
+  const bool cut_p = a.Hp != a.H;
+  const int e = cut_p && tp == tiles_p - 1 ? tq : (cut_p ? tiles_q : 0) + tp;
+  stride = 512;
+  return reinterpret_cast<char*>(a.dw_plane_hi) + (int64_t)e * (kTile * kTile * 2);
+}
+
+template <bool LOAD, bool WVH>
+LCE_DEV void dw_plane_split_io(char* hi, int hi_stride, char* lo, f32x16_t (&acc)[kNB][kNB]) {
+  // one descriptor per block, the thread's place as the vector offset, the pair as a scalar offset: no 64-bit
+  // address per pair
+  const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(hi, 0, 255 * hi_stride + 512, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rl = __builtin_amdgcn_make_buffer_rsrc(lo, 0, kTile * kTile * 2, 0x00020000);
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wp = wave & 1, wq = wave >> 1;
+  const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
+  const int vh = (w_row * kWaveTile + (lane >> 4)) * hi_stride + w_col * 256 + (lane & 15) * 16;
+  const int vl = tid * 16;
+  // kBatch pairs are fetched together before any is used: their loads are in flight together
+  constexpr int kBatch = LCE_DW_PLANE_BATCH / 2;
 #pragma unroll
-  for (int q0 = 0; q0 < 64; q0 += kPlaneBatch) {
-    u32x4_t old[kPlaneBatch];
+  for (int p0 = 0; p0 < 32; p0 += kBatch) {
+    u32x4_t oh[kBatch], ol[kBatch];
     if (LOAD) {
 #pragma unroll
-      for (int u = 0; u < kPlaneBatch; ++u) old[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, (q0 + u) * 4096, 0);
+      for (int u = 0; u < kBatch; ++u) {
+        const int p = p0 + u, i = p >> 3, k = (p >> 1) & 3, rb = WVH ? k : i, cb = WVH ? i : k;
+        oh[u] = __builtin_amdgcn_raw_buffer_load_b128(rh, vh, (rb * kBlk + (cb * 2 + (p & 1)) * 4) * hi_stride, 0);
+        ol[u] = __builtin_amdgcn_raw_buffer_load_b128(rl, vl, p * 4096, 0);
+      }
     }
 #pragma unroll
-    for (int u = 0; u < kPlaneBatch; ++u) {
-      const int q = q0 + u, rb = q >> 4, cb = (q >> 2) & 3, rq = q & 3;
-      f32x4_t v;
+    for (int u = 0; u < kBatch; ++u) {
+      const int p = p0 + u, i = p >> 3, k = (p >> 1) & 3, rb = WVH ? k : i, cb = WVH ? i : k;
+      float f[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < 8; ++j) {
         // (a volatile read: the compiler would otherwise read all 256 accumulator registers before the first load)
-        float t;
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[rb][cb][rq * 4 + j]));
-        v[j] = t;
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(f[j]) : "a"(acc[i][k][(p & 1) * 8 + j]));
       }
-      if (LOAD) v += __builtin_bit_cast(f32x4_t, old[u]);
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), rsrc, voff, q * 4096, 0);
+      u32x4_t nh, nl;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        if (LOAD) {
+          f[2 * d] += __builtin_bit_cast(float, __builtin_amdgcn_perm(oh[u][d], ol[u][d], kSelLow));
+          f[2 * d + 1] += __builtin_bit_cast(float, __builtin_amdgcn_perm(oh[u][d], ol[u][d], kSelHigh));
+        }
+        const unsigned f0 = __builtin_bit_cast(unsigned, f[2 * d]), f1 = __builtin_bit_cast(unsigned, f[2 * d + 1]);
+        nh[d] = __builtin_amdgcn_perm(f1, f0, kSelHigh);
+        nl[d] = __builtin_amdgcn_perm(f1, f0, kSelLow);
+      }
+      __builtin_amdgcn_raw_buffer_store_b128(nh, rh, vh, (rb * kBlk + (cb * 2 + (p & 1)) * 4) * hi_stride, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(nl, rl, vl, p * 4096, 0);
     }
     __builtin_amdgcn_sched_barrier(0);  // (one batch in registers at a time: an operand tile is in flight)
   }
@@ -399,8 +442,10 @@ template <class T, bool WVH, int MODE, int ACC = 0> struct DwProblem {
       dw_epilogue_f32_sum<WVH, ACC == 4>(a, acc, tp, tq);
       return;
     } else if constexpr (ACC != 0) {
-      float* blk = a.dw_plane + ((int64_t)tq * tiles_p + tp) * (kTile * kTile);
-      dw_plane_io<ACC == 2>(blk, acc);
+      int stride;
+      char* hi = dw_hi_block<WVH>(a, tp, tq, stride);
+      char* lo = reinterpret_cast<char*>(a.dw_plane) + ((int64_t)tq * tiles_p + tp) * (kTile * kTile * 2);
+      dw_plane_split_io<ACC == 2, WVH>(hi, stride, lo, acc);
       return;
     }
     if (MODE == kDwStaged || MODE == kDwStaged32) {
@@ -464,17 +509,16 @@ template <class T, bool WVH, int MODE, int ACC = 0> hipError_t launch_tiles(cons
   return hipGetLastError();
 }
 
-// The plane of sums over chunks of token rows becomes dW: one workgroup per tile, each wave on the 128 x 128
-// sub-tile whose quads its threads stored (dw_plane_io).  A wave takes 32 rows of the stored matrix at a time, 256
-// bytes of each (128 columns of 16-bit data, 64 of fp32): the quads come in as they lie in the plane (1 KiB per
-// load), are scaled, rounded and written to the wave's slice of LDS where dw_epilogue would have put them in
-// memory, and leave as whole 256-byte rows, four rows per store instruction.  (Rows of the slice are 272 bytes
-// apart: 16-byte pieces stay aligned, and lanes on consecutive rows use different banks.)
-template <class T, bool WVH, bool F32OUT>
-__global__ __launch_bounds__(256) void dw_plane_out_kernel(const BwdArgs a) {
+// The sums over chunks of token rows become dW: one workgroup per tile, each wave on the 128 x 128 quarter whose
+// sums its threads stored (dw_plane_split_io).  A wave takes 32 rows of the stored matrix at a time: the 8 KiB of
+// upper halves come from exactly the 32 rows x 256 bytes that the results will take, the lower halves from the
+// plane; the sums are put together, scaled, rounded and written to the wave's slice of LDS where dw_epilogue would
+// have put them in memory, and leave as whole 256-byte rows, four rows per store instruction -- all loads of the
+// 32 rows are done before their first store.  (Rows of the slice are 272 bytes apart: 16-byte pieces stay aligned,
+// and lanes on consecutive rows use different banks.)
+template <class T, bool WVH>
+__global__ __launch_bounds__(256) void dw_plane_split_out_kernel(const BwdArgs a) {
   typedef typename elem_of<T>::type E;
-  typedef typename std::conditional<F32OUT, float, E>::type O;
-  constexpr int kPassCols = F32OUT ? 64 : 128, kPassBlocks = kPassCols / kBlk, kPieceCols = 16 / (int)sizeof(O);
   constexpr int kRowBytes = 256 + 16;
   __shared__ __attribute__((aligned(16))) char sh[4][kBlk * kRowBytes];
   const int tiles_p = (int)(a.Hp / kTile);
@@ -484,45 +528,52 @@ __global__ __launch_bounds__(256) void dw_plane_out_kernel(const BwdArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wp = wave & 1, wq = wave >> 1, half = lane >> 5;
   const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
-  const float* mine = a.dw_plane + (int64_t)blockIdx.x * (kTile * kTile) + threadIdx.x * 4;
+  int stride;
+  const char* hi = dw_hi_block<WVH>(a, tp, tq, stride) + (int64_t)(w_row * kWaveTile + (lane >> 4)) * stride + w_col * 256 +
+                   (lane & 15) * 16;
+  const char* lo = reinterpret_cast<const char*>(a.dw_plane) + (int64_t)blockIdx.x * (kTile * kTile * 2) + threadIdx.x * 16;
   char* my = sh[wave];
-  O* out = reinterpret_cast<O*>(a.dw);
+  E* out = reinterpret_cast<E*>(a.dw);
 #pragma unroll 1
-  for (int rb = 0; rb < kNB; ++rb)
-#pragma unroll 1
-    for (int cp = 0; cp < kNB / kPassBlocks; ++cp) {
+  for (int rb = 0; rb < kNB; ++rb) {
+    u32x4_t h[8], l[8];
 #pragma unroll
-      for (int cb = 0; cb < kPassBlocks; ++cb) {
-        const int cbk = cp * kPassBlocks + cb;
-        const int i = WVH ? cbk : rb, k = WVH ? rb : cbk;  // the block is acc[i][k] of the tile kernel
-#pragma unroll
-        for (int rq = 0; rq < 4; ++rq) {
-          const f32x4_t v = *reinterpret_cast<const f32x4_t*>(mine + ((i * 4 + k) * 4 + rq) * 1024) * coef;
-          char* at = my + (lane & 31) * kRowBytes + (cb * kBlk + 8 * rq + 4 * half) * (int)sizeof(O);
-          if (F32OUT) {
-            *reinterpret_cast<f32x4_t*>(at) = v;
-          } else {
-            u32x2_t o;
-            o[0] = pack2<T>(v[0], v[1]);
-            o[1] = pack2<T>(v[2], v[3]);
-            *reinterpret_cast<u32x2_t*>(at) = o;
-          }
-        }
-      }
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int r = it * 4 + (lane >> 4), piece = lane & 15;
-        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(my + r * kRowBytes + piece * 16);
-        const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + r;
-        const int64_t col = g.col0 + w_col * kWaveTile + cp * kPassCols + piece * kPieceCols;
-        // pieces that start at or past the last column are not stored; one that it cuts through is written whole,
-        // into the stride padding of its row
-        if (row < g.row_limit && col < g.col_limit)
-          __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + row * a.lddw + col));
-      }
-      __builtin_amdgcn_wave_barrier();
+    for (int j = 0; j < 8; ++j) {
+      const int cb = j >> 1, i = WVH ? cb : rb, k = WVH ? rb : cb;  // the pair is of block acc[i][k] of the tile kernel
+      h[j] = *reinterpret_cast<const u32x4_t*>(hi + (int64_t)(rb * kBlk + j * 4) * stride);
+      l[j] = *reinterpret_cast<const u32x4_t*>(lo + ((i * 4 + k) * 2 + (j & 1)) * 4096);
     }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+#pragma unroll
+      for (int qq = 0; qq < 2; ++qq) {
+        float v[4];
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+          v[2 * d] = __builtin_bit_cast(float, __builtin_amdgcn_perm(h[j][2 * qq + d], l[j][2 * qq + d], kSelLow)) * coef;
+          v[2 * d + 1] = __builtin_bit_cast(float, __builtin_amdgcn_perm(h[j][2 * qq + d], l[j][2 * qq + d], kSelHigh)) * coef;
+        }
+        const int rq = (j & 1) * 2 + qq;
+        u32x2_t o;
+        o[0] = pack2<T>(v[0], v[1]);
+        o[1] = pack2<T>(v[2], v[3]);
+        *reinterpret_cast<u32x2_t*>(my + (lane & 31) * kRowBytes + ((j >> 1) * kBlk + 8 * rq + 4 * half) * 2) = o;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int r = it * 4 + (lane >> 4), piece = lane & 15;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(my + r * kRowBytes + piece * 16);
+      const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + r;
+      const int64_t col = g.col0 + w_col * kWaveTile + piece * 8;
+      // pieces that start at or past the last column are not stored; one that it cuts through is written whole,
+      // into the stride padding of its row
+      if (row < g.row_limit && col < g.col_limit)
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + row * a.lddw + col));
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
 }
 
 // Whole tiles that meet the plane of sums over chunks of token rows (nothing is split along K then).
@@ -530,8 +581,7 @@ template <class T, bool WVH, int MODE> hipError_t launch_plane(const BwdArgs& a,
   hipError_t e = a.dw_acc == 1 ? launch_tiles<T, WVH, MODE, 1>(a, s) : launch_tiles<T, WVH, MODE, 2>(a, s);
   if (e != hipSuccess || !a.last_chunk) return e;
   const dim3 grid((unsigned)((a.vs / kTile) * (a.Hp / kTile)));
-  if (a.dw_dtype == DT_F32) hipLaunchKernelGGL((dw_plane_out_kernel<T, WVH, true>), grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL((dw_plane_out_kernel<T, WVH, false>), grid, dim3(256), 0, s, a);
+  hipLaunchKernelGGL((dw_plane_split_out_kernel<T, WVH>), grid, dim3(256), 0, s, a);
   return hipGetLastError();
 }
 
@@ -541,7 +591,10 @@ template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipS
     return a.dw_acc == 3 ? launch_tiles<T, WVH, kDwAll, 3>(a, s) : launch_tiles<T, WVH, kDwAll, 4>(a, s);
   }
   if (a.dw_acc != 0) {
-    if (a.dw_plane == nullptr || a.dw_part != nullptr || a.dw_acc > 2) return hipErrorInvalidValue;
+    // (16-bit dW only, and a place for the upper halves of the tiles that the edge of the matrix cuts)
+    const bool cut = a.Hp != a.H || a.v0 + a.vs != a.V;
+    if (a.dw_plane == nullptr || a.dw_part != nullptr || a.dw_acc > 2 || a.dw_dtype == DT_F32 || (cut && a.dw_plane_hi == nullptr))
+      return hipErrorInvalidValue;
     return launch_plane<T, WVH, kDwAll>(a, s);
   }
   // a last round of tiles may be split along K (the tile count does not depend on the rows; whether its K

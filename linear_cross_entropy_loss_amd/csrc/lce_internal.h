@@ -164,11 +164,14 @@ struct BwdArgs {
   // rows of dx always go to the tokens perm[] names (the rows of a chunk can be all there and still not be the
   // tokens of the same numbers)
   int perm_always;
-  // dW summed over chunks of token rows: dw_plane holds one 256 x 256 fp32 block per tile of dW, in the order of
-  // the accumulator registers (lce_bwd_dw.hip).  dw_acc: 0 = no plane (dW is stored as it comes), 1 = the sums
-  // are stored to the plane (first chunk), 2 = added to it; last_chunk: the plane is then scaled and stored as dW.
-  // fp32 dW needs no plane: 3 = the sums times the final factor are stored to dw itself (first chunk), 4 = added to it.
-  float* dw_plane;
+  // 16-bit dW summed over chunks of token rows: the fp32 sums are kept as 16-bit halves, the upper ones in dw
+  // itself, the lower ones in dw_plane (one block of 256 x 256 halves per tile of dW); dw_plane_hi takes the upper
+  // halves of the tiles that the edge of the matrix cuts (null if there is none) -- see lce_bwd_dw.hip.
+  // dw_acc: 0 = no sums over chunks (dW is stored as it comes), 1 = the sums are stored (first chunk), 2 = added
+  // to; last_chunk: they are then scaled and stored as dW.
+  // fp32 dW: 3 = the sums times the final factor are stored to dw itself (first chunk), 4 = added to it.
+  void* dw_plane;
+  void* dw_plane_hi;
   int dw_acc, last_chunk;
 };
 

@@ -490,13 +490,13 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
         assert rows % 256 == 0 and rows > 0
         assert chunks * rows >= N and (chunks - 1) * rows < N + 255
         assert total <= n_chunk * V * 4, (N, H, V, n_chunk, total)
-        if chunks > 1:  # the plane is part of it
-            assert total >= (H + (-H) % 256) * (V + (-V) % 256) * 4
+        if chunks > 1:  # the lower halves of the fp32 sums of dW are part of it (the upper halves lie in dW itself)
+            assert total >= (H + (-H) % 256) * (V + (-V) % 256) * 2
     assert took > 50
-    # the benchmark's default shape: five chunks of 13 token tiles
+    # the benchmark's default shape: four chunks of 16 token tiles
     prob = _lib.make_problem(16384, 2048, 131072, 2048, 131072, 2048, 131072, torch.bfloat16, torch.bfloat16,
                              torch.bfloat16, torch.bfloat16, -1, 1.0, 0.0, 4096, False)
-    assert _lib.forward_backward_plan(prob) == (5, 3328)
+    assert _lib.forward_backward_plan(prob) == (4, 4096)
     # no one-pass route for fp32 activations, nor for the monitoring values with a hidden size that needs the K mask
     for kw in (dict(x=torch.float32, w=torch.float32), dict(mon=True, H=520)):
         xd, wd, Hh = kw.get("x", torch.bfloat16), kw.get("w", torch.bfloat16), kw.get("H", 512)
