@@ -282,22 +282,27 @@ enum {
  * per-slice partials and, in the 16-bit compute type, e = exp(z - slice max)
  * for every logit (chunk_rows * V * 2 bytes); the row merge gives lse; one pass
  * over the stage turns e into dz; dx of the chunk is complete after one
- * contraction; dW is summed over the chunks in an fp32 plane of H * V * 4 bytes
- * (the reference's fp32 At_grad, ops.py:692; no plane with a single chunk).
- * The chunk is the longest for which all of it stays within n_chunk * V * 4
- * bytes.  8*N*H*V FLOPs become 6*N*H*V.
+ * contraction; dW is summed over the chunks in fp32 (the reference's fp32
+ * At_grad, ops.py:692): an fp32 dW in the caller's buffer itself; a 16-bit dW
+ * as two 16-bit halves per sum, the upper halves in the caller's dw -- which
+ * holds no meaningful values until the call is done --, the lower halves in
+ * H * V * 2 bytes of the workspace (nothing of this with a single chunk).
+ * The chunks are as long as n_chunk * V * 4 bytes allow, or shorter where the
+ * library's model of its kernels finds that faster.  8*N*H*V FLOPs become
+ * 6*N*H*V.
  *
  * lce_problem.route: LCE_ROUTE_AUTO takes this route when a model of the tile
  * kernels' rounds of workgroups says it is the faster one (short chunks are
- * not: every chunk costs a round trip of the whole plane, so small problems
+ * not: every chunk costs a round trip of dW's fp32 sums, so small problems
  * and tight bounds take two passes); LCE_ROUTE_ONE_PASS takes it whenever it
  * fits the bound; LCE_ROUTE_TWO_PASS never.
  *
  * Problems this route does not cover take the two calls above, one after the
  * other on the same workspace, inside this entry point: fp32 activations, a
- * weight whose dtype differs from x's, monitoring != 0, and shapes whose plane
- * leaves no room for a chunk within the bound (lce_forward_backward_plan then
- * reports 0 chunks).  `phases` selects kernels of either route; on the one-pass
+ * weight that is neither of x's dtype nor fp32, monitoring != 0 with a hidden
+ * size that is not a multiple of 128, and shapes whose sums of dW leave no
+ * room for a chunk within the bound (a 16-bit dW with H near 2 * n_chunk or
+ * above; lce_forward_backward_plan then reports 0 chunks).  `phases` selects kernels of either route; on the one-pass
  * route LCE_PHASE_FWD_TILES is the logit kernel and LCE_PHASE_BWD_DZ the pass
  * that turns e into dz.
  *

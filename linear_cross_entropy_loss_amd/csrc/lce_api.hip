@@ -349,13 +349,13 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
   const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V), Hp = (size_t)lce::padded_hidden(p->H);
   const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
   // (packed rows of dx go to their tokens through 32-bit offsets into dx)
-  // (the monitoring values are taken over all rows: nothing is packed away then, and the pass over the stage
-  // zeroes the rows of tokens with an ignored label)
-  f->pack = !p->monitoring && packs_rows(p) && (size_t)p->N * (size_t)p->lddx * dxes < ((size_t)1 << 31);
+  // (the monitoring values are taken over all rows: the dropped tokens then follow the kept ones, the logit kernel
+  // and the row merge run over all of a chunk's rows, the gradient kernels over its kept ones)
+  f->pack = packs_rows(p) && (size_t)p->N * (size_t)p->lddx * dxes < ((size_t)1 << 31);
   f->dw_direct = p->dw_dtype == LCE_F32;
   f->k = plan_pack(p, 0, false);
   size_t o = f->k.xc;  // the labels are always counted; the packed copy of x is made chunk by chunk (below)
-  f->chunk_rows = o; o += align_up(1024 * 8);
+  f->chunk_rows = o; o += align_up(2048 * 8);
   f->lse_rows = o; o += align_up(Np * 4);
   f->tgt = o; o += align_up(Np * 4);
   f->blk = o; o += align_up(Np / lce::kMergeRows * 8 * sizeof(double));
@@ -622,8 +622,9 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
   fa.lse_rows = (float*)(base + f.lse_rows);
   fa.num_cus = num_cus;
   fa.nc = f.nc;
+  const bool all_rows = f.pack && p->monitoring;  // every row is computed, the kept ones first
   if (f.pack) {
-    fa.n_rows = n_rows; fa.perm = perm; fa.y0 = y; fa.y = yc;
+    fa.n_rows = all_rows ? nullptr : n_rows; fa.perm = perm; fa.y0 = y; fa.y = yc;
   }
 
   // (a call restricted to some kernels works on what a full call left in the workspace)
@@ -707,12 +708,14 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
     a.dw_acc = f.chunks == 1 ? 0 : (f.dw_direct ? (c == 0 ? 3 : 4) : (c == 0 ? 1 : 2));
     a.last_chunk = c == f.chunks - 1;
     if (f.pack && (ph & (LCE_PHASE_PACK | LCE_PHASE_FWD_TILES | LCE_PHASE_BWD_DW))) {
-      e = lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, perm + row0, chunk_rows + c, p->N, base + f.xc, k.ldxc * 2,
-                                  nullptr, nullptr, num_cus, s, true);
+      e = lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, perm + row0, chunk_rows + (all_rows ? 1024 : 0) + c, p->N,
+                                  base + f.xc, k.ldxc * 2, nullptr, nullptr, num_cus, s, true);
       if (e != hipSuccess) return hip_fail(e, "gather_rows");
     }
     if (ph & LCE_PHASE_FWD_TILES) {
-      e = lce::launch_fwd_stage(a, s);
+      lce::BwdArgs af = a;
+      if (all_rows) af.n_rows = chunk_rows + 1024 + c;
+      e = lce::launch_fwd_stage(af, s);
       if (e != hipSuccess) return hip_fail(e, "fwd_stage");
     }
     if (ph & LCE_PHASE_FWD_REDUCE) {

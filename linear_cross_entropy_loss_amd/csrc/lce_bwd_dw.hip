@@ -462,6 +462,8 @@ __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdAr
   extern __shared__ __attribute__((aligned(16))) char lds[];
   typedef typename elem_of<T>::type E;
   DwProblem<T, WVH, MODE, ACC> prob(a);
+  // (a chunk without a kept row adds nothing to the sums of the earlier chunks)
+  if ((ACC == 2 || ACC == 4) && prob.rows == 0) return;
   Pipe3<T, E, false, E, false, DwProblem<T, WVH, MODE, ACC>> pipe(prob);
   pipe.run(prob.ldx, a.vs / kBK, prob.plan.kt, lds);
 }

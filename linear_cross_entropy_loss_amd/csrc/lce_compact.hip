@@ -6,7 +6,9 @@
 // here synchronises with the host.  (The reference computes the ignored rows
 // and multiplies them away.)
 //
-//   compact_labels  perm[j] = original index of the j-th kept token, yc[j] its label, n_rows = how many
+//   compact_labels  perm[j] = original index of the j-th kept token, yc[j] its label, n_rows = how many; the dropped
+//                   tokens follow in perm from n_rows on, in their order (yc = ignore_index), for a caller that
+//                   wants all rows with the kept ones first
 //   gather_rows     xc[j] = x[perm[j]], lse_c[j] = lse[perm[j]]  (fp32 activations: as bf16 pairs, see gather_rows_split_kernel)
 //   scatter_rows    rows of dropped tokens of dx = 0 (and dx[perm[j]] = dxc[j] where dx was staged packed)
 //
@@ -71,7 +73,7 @@ __global__ __launch_bounds__(256) void scan_counts_kernel(int* cnt, int64_t nseg
 }
 
 __global__ __launch_bounds__(256) void pack_kept_kernel(const int64_t* y, int64_t N, int64_t ignore_index,
-                                                        const int* offs, int* perm, int64_t* yc) {
+                                                        const int* offs, const int64_t* n_rows, int* perm, int64_t* yc) {
   __shared__ int sh[4];
   const int64_t base = (int64_t)blockIdx.x * kSegTokens + (int64_t)threadIdx.x * kPerThread;
   int64_t lab[kPerThread];
@@ -84,13 +86,15 @@ __global__ __launch_bounds__(256) void pack_kept_kernel(const int64_t* y, int64_
   int excl;
   block_scan(c, excl, sh);
   int64_t j = (int64_t)offs[blockIdx.x] + excl;
+  const int64_t kept = n_rows[0];
 #pragma unroll
-  for (int k = 0; k < kPerThread; ++k)
-    if (lab[k] != ignore_index) {
-      perm[j] = (int)(base + k);
-      yc[j] = lab[k];
-      ++j;
-    }
+  for (int k = 0; k < kPerThread; ++k) {
+    if (base + k >= N) break;
+    // j kept tokens come before token base + k: a dropped one is number base + k - j among the dropped
+    const int64_t at = lab[k] != ignore_index ? j++ : kept + (base + k - j);
+    perm[at] = (int)(base + k);
+    yc[at] = lab[k];
+  }
 }
 
 // One workgroup per packed row (grid-stride).  Rows are moved in 16-byte pieces; `chunks` pieces per row.
@@ -204,7 +208,7 @@ hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_ind
   const int64_t nseg = compact_segments(N);
   hipLaunchKernelGGL(count_kept_kernel, dim3((unsigned)nseg), dim3(256), 0, s, y, N, ignore_index, cnt);
   hipLaunchKernelGGL(scan_counts_kernel, dim3(1), dim3(256), 0, s, cnt, nseg, n_rows);
-  hipLaunchKernelGGL(pack_kept_kernel, dim3((unsigned)nseg), dim3(256), 0, s, y, N, ignore_index, cnt, perm, yc);
+  hipLaunchKernelGGL(pack_kept_kernel, dim3((unsigned)nseg), dim3(256), 0, s, y, N, ignore_index, cnt, n_rows, perm, yc);
   return hipGetLastError();
 }
 

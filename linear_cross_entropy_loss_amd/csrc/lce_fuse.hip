@@ -91,6 +91,8 @@ __global__ void chunk_rows_kernel(const int64_t* n_rows, int64_t N, int64_t nc, 
   if (c >= chunks) return;
   const int64_t left = packed_rows(n_rows, N) - (int64_t)c * nc;
   out[c] = left < 0 ? 0 : (left > nc ? nc : left);
+  const int64_t all = N - (int64_t)c * nc;  // the chunk's rows when the dropped tokens follow the kept ones
+  out[1024 + c] = all < 0 ? 0 : (all > nc ? nc : all);
 }
 
 // t[r][c] *= g[0] for r < rows, c < cols (row stride ld, rows on 16-byte boundaries), the product formed in fp32;

@@ -202,7 +202,8 @@ hipError_t launch_stage_scale(const BwdArgs& a, hipStream_t s);
 // t[r][c] *= g[0] (device scalar), in fp32; nothing is touched when g[0] == 1.  Rows on 16-byte boundaries.
 hipError_t launch_scale_rows(void* t, int dtype, int64_t rows, int64_t cols, int64_t ld, const float* g, int num_cus,
                              hipStream_t s);
-// out[c] = rows of chunk c (of `nc` rows each) among the *n_rows packed rows: min(max(*n_rows - c * nc, 0), nc).
+// out[c] = rows of chunk c (of `nc` rows each) among the *n_rows packed rows: min(max(*n_rows - c * nc, 0), nc);
+// out[1024 + c] = the same among all N rows (out holds 2048 entries).
 hipError_t launch_chunk_rows(const int64_t* n_rows, int64_t N, int64_t nc, int chunks, int64_t* out, hipStream_t s);
 hipError_t launch_bwd_dx(const BwdArgs& a, hipStream_t s);
 hipError_t launch_bwd_dw(const BwdArgs& a, hipStream_t s);
@@ -228,7 +229,7 @@ __device__ __forceinline__ int64_t packed_token(const int* perm, int64_t j, int6
 }
 
 // Packing of the tokens whose label is not ignore_index (lce_compact.hip).  `cnt` holds one int per
-// compact_segments(N); perm and yc hold N entries each, of which the first *n_rows are written.
+// compact_segments(N); perm and yc hold N entries each: the kept tokens first (*n_rows of them), then the dropped ones.
 int64_t compact_segments(int64_t N);
 hipError_t launch_compact_labels(const int64_t* y, int64_t N, int64_t ignore_index, int* cnt, int64_t* n_rows,
                                  int* perm, int64_t* yc, hipStream_t s);

@@ -151,6 +151,10 @@ MON_CASES = [
     (4000, 512, 5000, torch.float16, 2048, 0.3, 1e-3, 0.5, 2, 0),    # the tile column that straddles V
     (4000, 640, 5000, torch.bfloat16, 2048, 0.1, 0.0, 2.0, 1, 1),    # weight stored (V, H)
     (1000, 384, 777, torch.float16, 4096, 0.2, 0.0, 1.0, 0, 0),      # a single chunk
+    # packed (1 = always): the dropped tokens follow the kept ones; 8 chunks of 512 rows, the last five without a kept row
+    (4096, 512, 4096, torch.bfloat16, 1024, 0.7, 1e-4, 1.0, 1, 0),
+    (6000, 256, 3000, torch.float16, 1024, 0.45, 0.0, 0.5, 1, 1),    # 6 chunks, the edge of dW cuts tiles, (V, H)
+    (4096, 512, 4096, torch.float16, 1024, 0.97, 0.0, 1.0, 1, 0),    # kept rows in the first chunk only
 ]
 
 
