@@ -353,6 +353,9 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
   // and the row merge run over all of a chunk's rows, the gradient kernels over its kept ones)
   f->pack = packs_rows(p) && (size_t)p->N * (size_t)p->lddx * dxes < ((size_t)1 << 31);
   f->dw_direct = p->dw_dtype == LCE_F32;
+  // (a 16-bit dW summed over chunks keeps the upper halves of its sums in dW itself, addressed through 32-bit
+  // offsets that span the 256 rows of a tile: lce_bwd_dw.hip)
+  const bool halves_ok = (size_t)p->lddw * 2 * 256 < ((size_t)1 << 31);
   f->k = plan_pack(p, 0, false);
   size_t o = f->k.xc;  // the labels are always counted; the packed copy of x is made chunk by chunk (below)
   f->chunk_rows = o; o += align_up(2048 * 8);
@@ -408,6 +411,7 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     const int64_t chunks = (tiles + t - 1) / t;
     if (chunks > 1024 || (first != 0 && chunks > 4 * first + 8)) break;
     if (t < tiles && (tiles + t) / (t + 1) == chunks) continue;  // a longer chunk gives the same number of chunks
+    if (chunks > 1 && want_dw && !f->dw_direct && !halves_ok) continue;
     const int64_t t_even = (tiles + chunks - 1) / chunks;  // equal lengths
     FusedPlan cand = *f;
     if (total_for(t_even * 256, (int)chunks, &cand) + reserve > bound) continue;
@@ -754,7 +758,7 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
 
 extern "C" {
 
-int lce_version(void) { return 400; }  // 0.4.0: lce_problem.w_layout (weight and dW stored (V, H))
+int lce_version(void) { return 500; }  // 0.5.0: lce_problem.route, lce_forward_backward, lce_scale
 
 const char* lce_strerror(int status) {
   switch (status) {

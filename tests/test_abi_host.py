@@ -506,6 +506,14 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
     prob = _lib.make_problem(4096, 512, 8192, 512, 8192, 512, 8192, torch.bfloat16, torch.bfloat16, torch.bfloat16,
                              torch.bfloat16, -1, 1.0, 0.0, 4096, True, route=_lib.ROUTE_ONE_PASS)
     assert _lib.forward_backward_plan(prob)[0] > 0  # monitoring with H a multiple of 128: covered
+    # a 16-bit dW whose rows are 8 MiB apart or more: its sums over chunks cannot live in it (32-bit offsets over the
+    # 256 rows of a tile), so more than one chunk is not planned; an fp32 dW is summed in place and may
+    V = 1 << 22
+    for dwt, want in ((torch.bfloat16, (0, 1)), (torch.float32, None)):
+        prob = _lib.make_problem(8192, 256, V, 256, V, 256, V, torch.bfloat16, torch.bfloat16, torch.bfloat16, dwt, -1, 1.0,
+                                 0.0, 1024, False, route=_lib.ROUTE_ONE_PASS)
+        chunks = _lib.forward_backward_plan(prob)[0]
+        assert (chunks in want) if want else chunks > 1, (dwt, chunks)
     # an fp32 master weight under 16-bit activations: one 16-bit copy of all of it in the workspace, and its fp32 gradient
     # is summed over the chunks in the caller's buffer (no plane)
     kw = dict(N=8192, H=1024, V=32768, ldx=1024, ldw=32768, lddx=1024, lddw=32768, x_dtype=torch.bfloat16,

@@ -277,3 +277,47 @@ def test_problems_outside_the_one_pass_route_take_the_two_calls_inside_the_entry
     torch.cuda.synchronize()
     for k in a:
         assert torch.equal(a[k], b[k]), k
+
+
+@pytest.mark.pack_auto
+@pytest.mark.parametrize("layout", [0, 1])
+def test_sums_over_chunks_kept_in_dw_stay_inside_dw(layout):
+    """A 16-bit dW summed over several chunks holds the upper halves of its fp32 sums while the call runs: with dW a
+    view of a wider buffer (rows 72 elements longer than they need to be), nothing beyond the 8 elements of stride
+    padding that the stores of a row may touch is written, the rows behind the last one included, and the result is
+    the one a dense dW gets, bit for bit."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    lib = _lib.load()
+    N, H, V, dt = 3000, 520, 5000, torch.bfloat16   # the edge of dW cuts tiles in both directions
+    x, y, w = make_inputs(N, H, V, dt, seed=11, ignore_frac=0.1, device="cuda")
+    hp, vp = H + (-H) % 8, V + (-V) % 8
+    xd = torch.zeros(N, hp, dtype=dt, device="cuda")
+    xd[:, :H] = x
+    rows, cols = (V, H) if layout else (H, V)
+    cp = cols + (-cols) % 8
+    wd = torch.zeros(rows, cp, dtype=dt, device="cuda")
+    wd[:, :cols] = w.t() if layout else w
+    g = torch.ones(1, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    results = []
+    for extra in (0, 72):
+        ld = cp + extra
+        prob = _lib.make_problem(N, H, V, hp, cp, hp, ld, dt, dt, dt, dt, -1, 1.0, 0.0, 1024, False, 0, 1, 0, layout,
+                                 _lib.ROUTE_ONE_PASS)
+        chunks, _ = _lib.forward_backward_plan(prob)
+        assert chunks >= 3
+        ub = _lib.forward_backward_workspace_bytes(prob)
+        ws = torch.empty(ub, dtype=torch.uint8, device="cuda")
+        buf = torch.full((rows + 4, ld), 7.0, dtype=dt, device="cuda")   # four more rows behind dW
+        lse, out5 = torch.zeros(N, device="cuda"), torch.zeros(5, device="cuda")
+        nv, dx = torch.zeros(1, dtype=torch.int64, device="cuda"), torch.zeros(N, hp, dtype=dt, device="cuda")
+        print(f"layout={layout} ld={ld}: {chunks} chunks", flush=True)
+        rc = lib.lce_forward_backward(ctypes.byref(prob), P(xd), P(wd), P(y), P(g), P(lse), P(out5), P(nv), P(dx), P(buf),
+                                      P(ws), ub, st)
+        assert rc == 0, (rc, lib.lce_last_hip_error())
+        torch.cuda.synchronize()
+        assert (buf[rows:] == 7.0).all()
+        assert (buf[:rows, cp:] == 7.0).all()
+        results.append(buf[:rows, :cols].clone())
+    assert torch.equal(results[0], results[1])
