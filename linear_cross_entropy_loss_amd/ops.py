@@ -58,6 +58,14 @@ def _pack_mode() -> int:
     return int(pack_rows.get())
 
 
+@torch.compiler.assume_constant_result
+def _route_mode() -> int:
+    """Current value of `one_pass` as a number (0: False, 1: True, 2: "always"); baked into a traced graph like the
+    packing mode."""
+    v = one_pass.get()
+    return 2 if v == "always" else (1 if v else 0)
+
+
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
@@ -196,11 +204,23 @@ def _finish_grads(dx, dw, layout):
     return dx, dw
 
 
+def _stand_in_gradient(x, y1, ignore_index):
+    """The upstream gradient that gradients are formed for before the real one is known: 1 for bf16 / fp32 ones.  fp16
+    ones would fall below fp16's normal range on the way (entries of order 1/n_valid; a loss scale arrives too late to
+    save them): they are formed for the largest power of two that is not above the number of valid labels -- entries
+    of the order of the per-token gradient -- and divided by it again when the real one is multiplied in."""
+    if x.dtype == torch.float16:
+        return torch.exp2(torch.floor(torch.log2((y1 != ignore_index).sum().clamp(min=1).to(torch.float32)))).reshape(1)
+    return torch.ones(1, dtype=torch.float32, device=x.device)
+
+
 def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, pack, need_dx,
-                   need_dw):
+                   need_dw, always=None):
     """Runs lce_forward_backward when its one-pass route covers the problem.  Returns None otherwise, else
     (out5, lse, n_valid, x, y1, w, layout, dx, dw, pre): the gradients for an upstream gradient of `pre` (a device
-    scalar; None stands for 1)."""
+    scalar; None stands for 1).  `always`: take the route wherever it fits (default: what `one_pass` says)."""
+    if always is None:
+        always = one_pass.get() == "always"
     with torch.cuda.device(x_in.device):
         x, y1, w, layout, N, H, V = _problem_views(x_in, y, At)
         if x.dtype == torch.float32 or w.dtype not in (x.dtype, torch.float32):
@@ -210,7 +230,7 @@ def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_c
         prob = _lib.make_problem(
             N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, w_cols + (-w_cols) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
             ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring, 0, pack, 0, layout,
-            _lib.ROUTE_ONE_PASS if one_pass.get() == "always" else _lib.ROUTE_AUTO,
+            _lib.ROUTE_ONE_PASS if always else _lib.ROUTE_AUTO,
         )
         lib = _lib.load()
         _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")
@@ -223,14 +243,7 @@ def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_c
         lse = torch.empty(N, dtype=torch.float32, device=dev)
         out5 = torch.empty(5, dtype=torch.float32, device=dev)
         n_valid = torch.empty(1, dtype=torch.int64, device=dev)
-        # The upstream gradient is not known yet.  bf16 / fp32 gradients are formed for an upstream gradient of 1.  fp16
-        # ones would fall below fp16's normal range on the way (entries of order 1/n_valid; a loss scale arrives too
-        # late to save them): they are formed for the largest power of two that is not above the number of valid
-        # labels -- entries of the order of the per-token gradient -- and backward divides it out again.
-        if x.dtype == torch.float16:
-            pre = torch.exp2(torch.floor(torch.log2((y1 != ignore_index).sum().clamp(min=1).to(torch.float32)))).reshape(1)
-        else:
-            pre = torch.ones(1, dtype=torch.float32, device=dev)
+        pre = _stand_in_gradient(x, y1, ignore_index)  # (the upstream gradient is not known yet)
         stream = torch.cuda.current_stream(dev).cuda_stream
         rc = lib.lce_forward_backward(ctypes.byref(prob), _ptr(x), _ptr(w), _ptr(y1), _ptr(pre), _ptr(lse), _ptr(out5),
                                       _ptr(n_valid), _ptr(dx), _ptr(dw), _ptr(ws), nbytes, ctypes.c_void_p(stream))
@@ -427,13 +440,7 @@ def _op_backward(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, lse: torch.
 @_op_backward.register_fake
 def _(x, y, At, lse, n_valid, grad_loss, ignore_index, z_regularization, logit_scale, N_chunk_size, need_dx, need_dw,
       pack_rows_mode=0):
-    if not need_dw:
-        dw = At.new_empty((0,))
-    elif _weight_layout(At, x.dtype) == _lib.W_VH:
-        dw = At.new_empty((At.shape[1], At.shape[0])).t()  # stored like the weight: (V, H) rows
-    else:
-        dw = torch.empty_like(At, memory_format=torch.contiguous_format)
-    return (torch.empty_like(x, memory_format=torch.contiguous_format) if need_dx else x.new_empty((0,))), dw
+    return _fake_grads(x, At, need_dx, need_dw)
 
 
 def _op_setup_context(ctx, inputs, output):
@@ -461,6 +468,93 @@ def _op_autograd(ctx, grad_out5, grad_lse, grad_n_valid):
 _op_forward.register_autograd(_op_autograd, setup_context=_op_setup_context)
 
 
+# Loss and gradients from one call, for traced graphs whose loss needs a gradient: what LinearXentImplementation does
+# in eager mode.  The gradients come out for the stand-in upstream gradient `pre`; the autograd formula multiplies the
+# real one in (lce_amd::scale, which returns a new tensor: the saved gradients stay as they are, so the graph can be
+# differentiated again).
+@torch.library.custom_op("lce_amd::forward_grads", mutates_args=(), device_types="cuda")
+def _op_forward_grads(x: torch.Tensor, y: torch.Tensor, At: torch.Tensor, ignore_index: int, z_regularization: float,
+                      logit_scale: float, N_chunk_size: int, monitoring: bool, need_dx: bool, need_dw: bool,
+                      pack_rows_mode: int = 0, always: bool = False
+                      ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    _check_inputs(x, y, At)
+    _check_dtypes(x, At)
+    done = _one_pass_impl(x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring,
+                          pack_rows_mode, need_dx, need_dw, always)
+    if done is not None:
+        out5, lse, n_valid, x2, y1, _, layout, dx, dw, pre = done
+        dx, dw = _finish_grads(dx, dw, layout)
+        if pre is None:
+            pre = torch.ones(1, dtype=torch.float32, device=x.device)
+    else:  # (a problem the one-pass route does not cover: the two device calls, one after the other)
+        out5, lse, n_valid, x2, y1, w, layout = _forward_impl(x, y, At, ignore_index, z_regularization, logit_scale,
+                                                              N_chunk_size, monitoring, pack_rows_mode)
+        pre = _stand_in_gradient(x2, y1, ignore_index)
+        dx, dw = _backward_impl(x2, y1, w, lse, n_valid, pre, ignore_index, z_regularization, logit_scale, N_chunk_size,
+                                need_dx, need_dw, pack_rows_mode, layout)
+    dx = dx.view(x.shape) if dx is not None else x.new_empty((0,))
+    dw = dw if dw is not None else At.new_empty((0,))
+    return out5, lse, n_valid, dx, dw, pre
+
+
+def _fake_grads(x, At, need_dx, need_dw):
+    if not need_dw:
+        dw = At.new_empty((0,))
+    elif _weight_layout(At, x.dtype) == _lib.W_VH:
+        dw = At.new_empty((At.shape[1], At.shape[0])).t()  # stored like the weight: (V, H) rows
+    else:
+        dw = torch.empty_like(At, memory_format=torch.contiguous_format)
+    return (torch.empty_like(x, memory_format=torch.contiguous_format) if need_dx else x.new_empty((0,))), dw
+
+
+@_op_forward_grads.register_fake
+def _(x, y, At, ignore_index, z_regularization, logit_scale, N_chunk_size, monitoring, need_dx, need_dw,
+      pack_rows_mode=0, always=False):
+    n = x.numel() // x.shape[-1]
+    dx, dw = _fake_grads(x, At, need_dx, need_dw)
+    return (x.new_empty((5,), dtype=torch.float32), x.new_empty((n,), dtype=torch.float32),
+            x.new_empty((1,), dtype=torch.int64), dx, dw, x.new_empty((1,), dtype=torch.float32))
+
+
+@torch.library.custom_op("lce_amd::scale", mutates_args=(), device_types="cuda")
+def _op_scale(t: torch.Tensor, factor: torch.Tensor) -> torch.Tensor:
+    """A copy of t (dense, row-major or the transposed view of such a matrix) times factor[0], the product formed in fp32."""
+    out = t.clone()
+    flat = out.view(-1) if out.is_contiguous() else out.t().view(-1)
+    n = flat.numel()
+    if n:
+        lib = _lib.load()
+        with torch.cuda.device(t.device):
+            g = factor.detach().to(device=t.device, dtype=torch.float32).reshape(1).contiguous()
+            stream = torch.cuda.current_stream(t.device).cuda_stream
+            # (one row of n elements: any dense tensor, whatever its row length)
+            rc = lib.lce_scale(_ptr(flat), _lib.dtype_code(t.dtype), 1, n, n + (-n) % 8, _ptr(g), ctypes.c_void_p(stream))
+            _lib.raise_for_status(rc, "lce_scale")
+    return out
+
+
+@_op_scale.register_fake
+def _(t, factor):
+    return torch.empty_like(t)
+
+
+def _fg_setup_context(ctx, inputs, output):
+    _, _, _, dx, dw, pre = output
+    ctx.save_for_backward(dx, dw, pre)
+
+
+def _fg_autograd(ctx, grad_out5, grad_lse, grad_n_valid, grad_dx, grad_dw, grad_pre):
+    # only the loss (entry 0 of the 5 scalars) is differentiable, as above
+    dx, dw, pre = ctx.saved_tensors
+    factor = grad_out5[0:1].to(torch.float32) / pre
+    gx = _op_scale(dx, factor) if ctx.needs_input_grad[0] else None
+    gw = _op_scale(dw, factor) if ctx.needs_input_grad[2] else None
+    return gx, None, gw, None, None, None, None, None, None, None, None, None
+
+
+_op_forward_grads.register_autograd(_fg_autograd, setup_context=_fg_setup_context)
+
+
 def linear_cross_entropy(
     x,
     y,
@@ -473,12 +567,13 @@ def linear_cross_entropy(
 ):
     """Functional form (``ops.py:814-826``); returns ``(loss, z_reg, logit_max, logit_entropy, logit_norm)``.
 
-    While ``torch.compile`` / ``torch.export`` trace, the call goes through the registered operator
-    ``torch.ops.lce_amd.forward`` (loss in the forward, gradients by a backward that recomputes the logit
-    tiles), so it can sit inside a compiled region; in eager mode it goes through ``LinearXentImplementation``,
-    which computes the gradients along with the loss where it can (module docstring; with ``one_pass`` off:
-    the same device calls as the registered operator, bit-identical results, about 80 us less dispatch
-    overhead per forward+backward).  Under autocast ``x`` takes the weight's 16-bit dtype, or the autocast
+    While ``torch.compile`` / ``torch.export`` trace, the call goes through registered operators, so it can
+    sit inside a compiled region: ``torch.ops.lce_amd.forward_grads`` when an input needs a gradient (loss and
+    gradients from one evaluation of the logits, the upstream gradient multiplied in by ``lce_amd.scale`` in
+    the backward graph), else -- and with ``one_pass`` off at trace time -- ``torch.ops.lce_amd.forward`` (loss
+    in the forward, gradients by a backward that recomputes the logit tiles).  In eager mode it goes through
+    ``LinearXentImplementation``, which makes the same device calls with about 80 us less dispatch overhead
+    per forward+backward and bit-identical results.  Under autocast ``x`` takes the weight's 16-bit dtype, or the autocast
     dtype when the weight is fp32; an fp32 weight is read as is (no 16-bit copy) and gets an fp32 gradient.
     fp32 ``x`` with an fp32 weight (no autocast) is computed as bf16 pairs, accurate to about 1e-5 of the
     largest gradient entry, at three times the matrix work of 16-bit tensors.
@@ -490,8 +585,14 @@ def linear_cross_entropy(
             bool(monitoring))
         return loss, z_reg, logit_max, logit_ent, logit_norm
     x = _autocast_x(x, At)
-    out5, _, _ = _op_forward(x, y, At, int(ignore_index), float(z_regularization), float(logit_scale),
-                             int(N_chunk_size), bool(monitoring), _pack_mode())
+    route = _route_mode()
+    need_dx, need_dw = x.requires_grad, At.requires_grad
+    if route and torch.is_grad_enabled() and (need_dx or need_dw):
+        out5 = _op_forward_grads(x, y, At, int(ignore_index), float(z_regularization), float(logit_scale),
+                                 int(N_chunk_size), bool(monitoring), need_dx, need_dw, _pack_mode(), route == 2)[0]
+    else:
+        out5 = _op_forward(x, y, At, int(ignore_index), float(z_regularization), float(logit_scale),
+                           int(N_chunk_size), bool(monitoring), _pack_mode())[0]
     loss, z_reg, logit_max, logit_ent, logit_norm = out5.unbind(0)
     return loss, z_reg.detach(), logit_max.detach(), logit_ent.detach(), logit_norm.detach()
 

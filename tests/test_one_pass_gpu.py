@@ -76,6 +76,7 @@ def _both_routes(N, H, V, dt, n_chunk, ignore, z_reg=0.0, scale=1.0, pack=0, lay
                                   P(b["dx"]), P(b["dw"]), P(ws), ub, st)
     assert rc == 0, (rc, lib.lce_last_hip_error())
     torch.cuda.synchronize()
+    b["chunks"] = chunks
     for o in (a, b):
         o["dx"] = o["dx"][:, :H]
         o["dw"] = o["dw"][:, :H].t() if layout else o["dw"][:, :V]
@@ -321,3 +322,44 @@ def test_sums_over_chunks_kept_in_dw_stay_inside_dw(layout):
         assert (buf[:rows, cp:] == 7.0).all()
         results.append(buf[:rows, :cols].clone())
     assert torch.equal(results[0], results[1])
+
+
+@pytest.mark.pack_auto
+def test_forty_draws_over_chunks_packing_monitoring_and_layouts():
+    """Seeded draws over what the one-pass route varies at once -- the number of chunks (1 to 20), the three packing
+    modes with none to nine tenths of the labels ignored, the monitoring values, both weight layouts, a 16-bit or fp32
+    dW, z-regularisation and scale, shapes that the tiles do not divide -- each against the two-pass route and, where
+    the fp64 oracle is quick, against that."""
+    import random
+
+    rng = random.Random(9)
+    ran = several = 0
+    for it in range(40):
+        mon = rng.random() < 0.5
+        H = rng.choice([128, 256, 384, 512, 640]) if mon else rng.choice([64, 200, 256, 520, 768])
+        N = rng.choice([1500, 3000, 4096, 5000, 9000])
+        V = rng.choice([2048, 3000, 4096, 5000, 8200])
+        dt = rng.choice([torch.bfloat16, torch.float16])
+        n_chunk = rng.choice([512, 1024, 2048])
+        ign = rng.choice([0.0, 0.1, 0.5, 0.9])
+        z_reg = rng.choice([0.0, 1e-4, 1e-2])
+        scale = rng.choice([1.0, 0.5, 2.0])
+        pack, layout = rng.choice([0, 1, 2]), rng.choice([0, 1])
+        dw_dt = rng.choice([None, None, torch.float32])
+        print(f"draw {it}: N={N} H={H} V={V} {dt} n_chunk={n_chunk} ignored={ign} z_reg={z_reg} scale={scale} pack={pack} "
+              f"layout={layout} monitoring={mon} dW={dw_dt}", flush=True)
+        try:
+            inputs, a, b = _both_routes(N, H, V, dt, n_chunk, ign, z_reg, scale, pack, layout, dw_dt=dw_dt, mon=mon,
+                                        seed=100 + it)
+        except AssertionError as e:
+            if "meant to take the one-pass route" not in str(e):
+                raise
+            continue  # (the bound of this draw leaves no room for the route)
+        ran += 1
+        several += b["chunks"] > 1
+        _check(inputs, a, b, z_reg, scale, 1.0, fp64=N * V <= 4096 * 8192)
+        if mon:
+            assert a["out5"][2].item() == b["out5"][2].item()
+            for i in (3, 4):
+                assert abs(a["out5"][i].item() - b["out5"][i].item()) <= 5e-5 * abs(a["out5"][i].item()) + 1e-7, (i, a["out5"], b["out5"])
+    assert ran >= 25 and several >= 20, (ran, several)

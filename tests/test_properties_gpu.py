@@ -522,17 +522,17 @@ def _fp64_model_grads(head, body, x, y):
     return loss.detach(), wh.grad, wb.grad
 
 
-def _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise):
-    # (the registered operator that a traced call goes through computes the loss alone in its forward; eager
-    # calls do the same with one_pass off, and those two are compared bit for bit)
+def _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise, one_pass=False):
+    # (`one_pass` off: the operator that a traced call goes through computes the loss alone in its forward and
+    # recomputes the logits in its backward; "always": loss and gradients come from lce_amd.forward_grads and the
+    # upstream gradient is multiplied in by lce_amd.scale.  Eager calls make the same device calls under the same
+    # setting, and the two are compared bit for bit.  The setting in force while tracing is baked into the graph; the
+    # autouse fixture of conftest.py puts the default back.)
     from linear_cross_entropy_loss_amd import ops
 
-    token = ops.one_pass.set(False)
-    try:
-        loss = model(x, y)
-        loss.backward()
-    finally:
-        ops.one_pass.reset(token)
+    ops.one_pass.set(one_pass)
+    loss = model(x, y)
+    loss.backward()
     ref = (loss.detach().clone(), head.weight.grad.clone(), body.weight.grad.clone())
     want_loss, want_wh, want_wb = _fp64_model_grads(head, body, x, y)
     for _ in range(2):
@@ -553,27 +553,29 @@ def _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise):
     body.weight.grad = None
 
 
-def test_torch_compile_matches_eager_and_fp64():
-    print("torch.compile aot_eager", flush=True)
+@pytest.mark.parametrize("one_pass", [False, "always", True])
+def test_torch_compile_matches_eager_and_fp64(one_pass):
+    print(f"torch.compile aot_eager, one_pass={one_pass}", flush=True)
     head, body, model = _head_model(256, 5000, torch.bfloat16)
     x = torch.randn(4, 150, 256, device="cuda", dtype=torch.bfloat16)
     y = torch.randint(0, 5000, (4, 150), device="cuda")
     y[0, :7] = -1
     compiled = torch.compile(model, backend="aot_eager", fullgraph=True)
-    _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise=True)
+    _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise=True, one_pass=one_pass)
 
 
-def test_torch_compile_odd_shapes_and_strided_weight():
+@pytest.mark.parametrize("one_pass", [False, "always"])
+def test_torch_compile_odd_shapes_and_strided_weight(one_pass):
     """in_features and out_features that are not multiples of 8 (the host makes padded copies for the kernels)
     and a head weight that is a strided view: the fake kernels of the registered operator must describe what
     the real ones return (shapes, dtypes, contiguity), or the traced backward would not line up."""
-    print("torch.compile aot_eager, odd shapes", flush=True)
+    print(f"torch.compile aot_eager, odd shapes, one_pass={one_pass}", flush=True)
     head, body, model = _head_model(100, 1001, torch.float16, hidden=72)
     x = torch.randn(3, 50, 72, device="cuda", dtype=torch.float16)
     y = torch.randint(0, 1001, (3, 50), device="cuda")
     y[1, :5] = -1
     compiled = torch.compile(model, backend="aot_eager", fullgraph=True)
-    _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise=True)
+    _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise=True, one_pass=one_pass)
     # the functional form on a transposed (V, H) -> (H, V) view of a weight, compiled, against the oracle
     from linear_cross_entropy_loss_amd import linear_cross_entropy
     from oracle import lce_forward_backward_fp64
@@ -594,11 +596,12 @@ def test_torch_compile_odd_shapes_and_strided_weight():
     assert A.grad.shape == A.shape
 
 
-def test_torch_compile_inductor_around_the_operator():
+@pytest.mark.parametrize("one_pass", [False, "always"])
+def test_torch_compile_inductor_around_the_operator(one_pass):
     """The default backend (inductor, what the reference's own probe uses: variants/compile_tests_NV5.py:535
     compiles with mode="max-autotune") generates the kernels of the surrounding Linear + gelu; the fused loss
     stays an opaque registered operator inside the compiled graph, forward and backward."""
-    print("torch.compile inductor", flush=True)
+    print(f"torch.compile inductor, one_pass={one_pass}", flush=True)
     head, body, model = _head_model(256, 4096, torch.bfloat16)
     x = torch.randn(2, 256, 256, device="cuda", dtype=torch.bfloat16)
     y = torch.randint(0, 4096, (2, 256), device="cuda")
@@ -606,7 +609,7 @@ def test_torch_compile_inductor_around_the_operator():
     compiled = torch.compile(model, fullgraph=True)
     # inductor fuses bias + gelu its own way, so the activations handed to the loss differ from eager's in the
     # last bit: checked against fp64, not bitwise against eager
-    _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise=False)
+    _run_compiled_and_check(model, compiled, head, body, x, y, eager_bitwise=False, one_pass=one_pass)
 
 
 def test_registered_backward_operator_passes_opcheck():
@@ -620,6 +623,53 @@ def test_registered_backward_operator_passes_opcheck():
         torch.library.opcheck(torch.ops.lce_amd.backward.default,
                               (x, y, w, lse, n_valid, g, -1, 1e-4, 1.0, 512, need_dx, need_dw),
                               test_utils=("test_schema", "test_faketensor"))
+
+
+def test_operators_of_the_one_pass_route_pass_opcheck_and_equal_the_eager_function():
+    """lce_amd.forward_grads (loss and gradients in one call) and lce_amd.scale: schema, fake kernels and autograd
+    registration; and, taken wherever the route fits, bit for bit what LinearXentImplementation gives in eager mode,
+    also for an upstream gradient other than 1, a weight stored (V, H) and a second backward over the same graph."""
+    from linear_cross_entropy_loss_amd import LinearXentImplementation, ops
+
+    print("opcheck forward_grads / scale", flush=True)
+    x, y, w = make_inputs(600, 104, 3001, torch.bfloat16, seed=13, ignore_frac=0.1, device="cuda")
+    for need_dx, need_dw in ((True, True), (True, False), (False, True)):
+        args = (x.clone().requires_grad_(need_dx), y, w.clone().requires_grad_(need_dw), -1, 1e-4, 0.5, 512, True,
+                need_dx, need_dw, 0, True)
+        torch.library.opcheck(torch.ops.lce_amd.forward_grads.default, args,
+                              test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+    f = torch.full((1,), 0.37, device="cuda")
+    torch.library.opcheck(torch.ops.lce_amd.scale.default, (w, f), test_utils=("test_schema", "test_faketensor"))
+    torch.library.opcheck(torch.ops.lce_amd.scale.default, (w.t(), f), test_utils=("test_schema", "test_faketensor"))
+    assert torch.equal(torch.ops.lce_amd.scale(w.t(), f), (w.t().float() * 0.37).to(w.dtype))
+    assert torch.equal(torch.ops.lce_amd.scale(x[:7, :3].contiguous(), f), (x[:7, :3].float() * 0.37).to(x.dtype))
+
+    ops.one_pass.set("always")
+    for dt in (torch.bfloat16, torch.float16):
+        for vh in (False, True):
+            # (a hidden size that is a multiple of 128: with the monitoring values, others take two passes, where the
+            # eager function folds the upstream gradient into its backward kernels and the operator rounds twice)
+            x, y, w = make_inputs(2000, 256, 5000, dt, seed=14, ignore_frac=0.1, device="cuda")
+            res = []
+            for via_op in (False, True):
+                xi = x.clone().requires_grad_(True)
+                wi = (w.t().contiguous() if vh else w.clone()).requires_grad_(True)
+                wv = wi.t() if vh else wi
+                if via_op:
+                    out = torch.ops.lce_amd.forward_grads(xi, y, wv, -1, 1e-4, 0.5, 1024, True, True, True,
+                                                          int(ops.pack_rows.get()), True)[0].unbind(0)
+                else:
+                    out = LinearXentImplementation.apply(xi, y, wv, -1, 1e-4, 0.5, 1024, True)
+                (out[0] * 3.0).backward(retain_graph=True)
+                first = (xi.grad.clone(), wi.grad.clone())
+                xi.grad = wi.grad = None
+                (out[0] * 3.0).backward()  # the eager function recomputes here; the operator scales its saved gradients again
+                res.append((torch.stack([o.detach() for o in out]), first, (xi.grad, wi.grad)))
+            assert torch.equal(res[0][0], res[1][0])
+            for a, b in zip(res[0][1], res[1][1]):
+                assert torch.equal(a, b), (dt, vh)
+            for a, b in zip(res[0][2], res[1][2]):  # (recomputed against saved: rounding only)
+                assert max(rel_errors(b, a)) <= 1.5e-2, (dt, vh)
 
 
 def test_autocast_follows_a_16_bit_weight_and_mismatched_dtypes_are_named():
