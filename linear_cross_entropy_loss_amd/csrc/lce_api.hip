@@ -424,8 +424,8 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     // (per chunk, besides the tile kernels: the row merge, the kernel that adds dx's K segments, launch gaps -- about 25 units)
     const double cost = (double)(chunks - 1) * chunk_cost((double)t_even) + chunk_cost((double)t_last) + 25.0 * (double)chunks;
     if (first == 0) first = chunks;
-    // (what the chunks do not change: the pass over the stage at 4 bytes per logit, the plane's way out at
-    // 6 bytes per element of dW -- about 8 MB of memory traffic per unit)
+    // (what the chunks do not change: the pass over the stage at 4 bytes per logit -- about 8 MB of memory traffic
+    // per unit)
     if (!f->ok || cost < best) {
       best = cost;
       *f = cand;
@@ -439,8 +439,7 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
   // scratch bound leaves only short chunks (every chunk adds a round trip of the whole fp32 plane of dW).
   BwdPlan b;
   if (p->route == LCE_ROUTE_AUTO && plan_bwd(p, &b) == LCE_OK) {
-    const double fixed = (double)Np * (double)Vp * 4.0 / 8.0e6 +
-                         (f->chunks > 1 && want_dw && !f->dw_direct ? (double)Hp * (double)Vp * 6.0 / 8.0e6 : 0.0);
+    const double fixed = (double)Np * (double)Vp * 4.0 / 8.0e6;
     const double two = kernel_cost((double)tiles * tv, (double)(lce::padded_k(p->H) / 64), 4.0, false) + b.cost;
     if (best + fixed > two) {
       f->ok = false;
@@ -708,9 +707,8 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
       a.y = y + row0;
       a.dx = dx ? (char*)dx + (size_t)row0 * (size_t)p->lddx * dxes : nullptr;
     }
-    // dW over the chunks: the plane (1: store, 2: add), or -- fp32 dW -- the caller's buffer itself (3: store, 4: add)
-    a.dw_acc = f.chunks == 1 ? 0 : (f.dw_direct ? (c == 0 ? 3 : 4) : (c == 0 ? 1 : 2));
-    a.last_chunk = c == f.chunks - 1;
+    // dW over the chunks: as halves (1: store, 2: add, 5: add and store dW), or -- fp32 dW -- in the caller's buffer itself (3: store, 4: add)
+    a.dw_acc = f.chunks == 1 ? 0 : (f.dw_direct ? (c == 0 ? 3 : 4) : (c == 0 ? 1 : (c == f.chunks - 1 ? 5 : 2)));
     if (f.pack && (ph & (LCE_PHASE_PACK | LCE_PHASE_FWD_TILES | LCE_PHASE_BWD_DW))) {
       e = lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, perm + row0, chunk_rows + (all_rows ? 1024 : 0) + c, p->N,
                                   base + f.xc, k.ldxc * 2, nullptr, nullptr, num_cus, s, true);

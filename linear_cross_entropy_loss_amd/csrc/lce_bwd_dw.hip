@@ -201,7 +201,7 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
 // wave keeps to the 128 rows x 256 bytes of its own quarter of the tile's results, and within those the eight
 // pairs of one block row of results (32 rows) to the 32 rows x 256 bytes that these results will take: pair
 // j = 2 * column block + rq / 2 of a block row is 4 rows, a lane's 16 bytes at row 4 j + lane / 16, byte
-// (lane % 16) * 16.  So dw_plane_split_out_kernel can turn the sums into dW in place, 32 rows at a time.
+// (lane % 16) * 16.  So the last chunk can turn the sums into dW in place, 32 rows at a time (dw_plane_split_final).
 // (Hardware fp32 atomic adds into an fp32 plane instead of load - add - store were measured at the headline
 // shape: the 268 M atomics of a chunk take longer than the chunk's matrix work, 30.6 ms a step against 22.3.)
 constexpr unsigned kSelLow = 0x05040100u, kSelHigh = 0x07060302u;  // v_perm selectors: the lower / upper halves of (S0, S1)
@@ -272,6 +272,79 @@ LCE_DEV void dw_plane_split_io(char* hi, int hi_stride, char* lo, f32x16_t (&acc
     }
     __builtin_amdgcn_sched_barrier(0);  // (one batch in registers at a time: an operand tile is in flight)
   }
+}
+
+// The last chunk of a 16-bit dW summed over chunks: the tile's sums are added to those of the earlier chunks and leave
+// as dW at once -- scaled, rounded, as whole 256-byte rows -- instead of going back to the halves.  A wave takes the
+// 32 rows of one block row of its results at a time: the 8 KiB of upper halves come from exactly the 32 rows x 256
+// bytes of dW that these results will take (dw_plane_split_io), so all of them are loaded before the first row is
+// stored; the values pass through the wave's slice of `scratch` (main-loop stage 1, idle during an epilogue; rows of
+// the slice are 272 bytes apart: 16-byte pieces stay aligned, lanes on consecutive rows use different banks).
+template <class T, bool WVH>
+LCE_DEV void dw_plane_split_final(const BwdArgs& a, const char* hi, int hi_stride, const char* lo, f32x16_t (&acc)[kNB][kNB],
+                                  int tp, int tq, char* scratch) {
+  typedef typename elem_of<T>::type E;
+  constexpr int kRowBytes = 256 + 16;
+  static_assert(kBlk * kRowBytes <= kDwSliceBytes, "a block row of results fits a wave's slice");
+  const DwTileGeom<WVH> g(a, tp, tq);
+  const float coef = final_factor_of(a);
+  const int tid = opaque_tid();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wp = wave & 1, wq = wave >> 1, half = lane >> 5;
+  const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
+  const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(hi), 0, 255 * hi_stride + 512, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rl = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(lo), 0, kTile * kTile * 2, 0x00020000);
+  const int vh = (w_row * kWaveTile + (lane >> 4)) * hi_stride + w_col * 256 + (lane & 15) * 16;
+  const int vl = tid * 16;
+  char* my = scratch + wave * kDwSliceBytes;
+  E* out = reinterpret_cast<E*>(a.dw);
+#pragma unroll
+  for (int rb = 0; rb < kNB; ++rb) {
+    u32x4_t h[8], l[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int cb = j >> 1, i = WVH ? cb : rb, k = WVH ? rb : cb;  // the pair is of block acc[i][k]
+      h[j] = __builtin_amdgcn_raw_buffer_load_b128(rh, vh, (rb * kBlk + j * 4) * hi_stride, 0);
+      l[j] = __builtin_amdgcn_raw_buffer_load_b128(rl, vl, ((i * 4 + k) * 2 + (j & 1)) * 4096, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int cb = j >> 1, i = WVH ? cb : rb, k = WVH ? rb : cb;
+#pragma unroll
+      for (int qq = 0; qq < 2; ++qq) {
+        float v[4];
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+          float a0, a1;
+          // (volatile reads: the compiler would otherwise read all 256 accumulator registers before the first load)
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a0) : "a"(acc[i][k][(j & 1) * 8 + qq * 4 + 2 * d]));
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a1) : "a"(acc[i][k][(j & 1) * 8 + qq * 4 + 2 * d + 1]));
+          v[2 * d] = (a0 + __builtin_bit_cast(float, __builtin_amdgcn_perm(h[j][2 * qq + d], l[j][2 * qq + d], kSelLow))) * coef;
+          v[2 * d + 1] = (a1 + __builtin_bit_cast(float, __builtin_amdgcn_perm(h[j][2 * qq + d], l[j][2 * qq + d], kSelHigh))) * coef;
+        }
+        const int rq = (j & 1) * 2 + qq;
+        u32x2_t o;
+        o[0] = pack2<T>(v[0], v[1]);
+        o[1] = pack2<T>(v[2], v[3]);
+        *reinterpret_cast<u32x2_t*>(my + (lane & 31) * kRowBytes + (cb * kBlk + 8 * rq + 4 * half) * 2) = o;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int r = it * 4 + (lane >> 4), piece = lane & 15;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(my + r * kRowBytes + piece * 16);
+      const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + r;
+      const int64_t col = g.col0 + w_col * kWaveTile + piece * 8;
+      // pieces that start at or past the last column are not stored; one that it cuts through is written whole,
+      // into the stride padding of its row
+      if (row < g.row_limit && col < g.col_limit)
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + row * a.lddw + col));
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_sched_barrier(0);  // (one block row in registers at a time: an operand tile is in flight)
+  }
+  __syncthreads();  // scratch is handed back to the main loop
 }
 
 // fp32 dW summed over chunks of token rows in the caller's buffer itself (BwdArgs::dw_acc 3 / 4): the tile's sum times
@@ -445,7 +518,8 @@ template <class T, bool WVH, int MODE, int ACC = 0> struct DwProblem {
       int stride;
       char* hi = dw_hi_block<WVH>(a, tp, tq, stride);
       char* lo = reinterpret_cast<char*>(a.dw_plane) + ((int64_t)tq * tiles_p + tp) * (kTile * kTile * 2);
-      dw_plane_split_io<ACC == 2, WVH>(hi, stride, lo, acc);
+      if constexpr (ACC == 5) dw_plane_split_final<T, WVH>(a, hi, stride, lo, acc, tp, tq, scratch);
+      else dw_plane_split_io<ACC == 2, WVH>(hi, stride, lo, acc);
       return;
     }
     if (MODE == kDwStaged || MODE == kDwStaged32) {
@@ -511,80 +585,10 @@ template <class T, bool WVH, int MODE, int ACC = 0> hipError_t launch_tiles(cons
   return hipGetLastError();
 }
 
-// The sums over chunks of token rows become dW: one workgroup per tile, each wave on the 128 x 128 quarter whose
-// sums its threads stored (dw_plane_split_io).  A wave takes 32 rows of the stored matrix at a time: the 8 KiB of
-// upper halves come from exactly the 32 rows x 256 bytes that the results will take, the lower halves from the
-// plane; the sums are put together, scaled, rounded and written to the wave's slice of LDS where dw_epilogue would
-// have put them in memory, and leave as whole 256-byte rows, four rows per store instruction -- all loads of the
-// 32 rows are done before their first store.  (Rows of the slice are 272 bytes apart: 16-byte pieces stay aligned,
-// and lanes on consecutive rows use different banks.)
-template <class T, bool WVH>
-__global__ __launch_bounds__(256) void dw_plane_split_out_kernel(const BwdArgs a) {
-  typedef typename elem_of<T>::type E;
-  constexpr int kRowBytes = 256 + 16;
-  __shared__ __attribute__((aligned(16))) char sh[4][kBlk * kRowBytes];
-  const int tiles_p = (int)(a.Hp / kTile);
-  const int tq = (int)blockIdx.x / tiles_p, tp = (int)blockIdx.x % tiles_p;
-  const DwTileGeom<WVH> g(a, tp, tq);
-  const float coef = final_factor_of(a);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wp = wave & 1, wq = wave >> 1, half = lane >> 5;
-  const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
-  int stride;
-  const char* hi = dw_hi_block<WVH>(a, tp, tq, stride) + (int64_t)(w_row * kWaveTile + (lane >> 4)) * stride + w_col * 256 +
-                   (lane & 15) * 16;
-  const char* lo = reinterpret_cast<const char*>(a.dw_plane) + (int64_t)blockIdx.x * (kTile * kTile * 2) + threadIdx.x * 16;
-  char* my = sh[wave];
-  E* out = reinterpret_cast<E*>(a.dw);
-#pragma unroll 1
-  for (int rb = 0; rb < kNB; ++rb) {
-    u32x4_t h[8], l[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int cb = j >> 1, i = WVH ? cb : rb, k = WVH ? rb : cb;  // the pair is of block acc[i][k] of the tile kernel
-      h[j] = *reinterpret_cast<const u32x4_t*>(hi + (int64_t)(rb * kBlk + j * 4) * stride);
-      l[j] = *reinterpret_cast<const u32x4_t*>(lo + ((i * 4 + k) * 2 + (j & 1)) * 4096);
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-#pragma unroll
-      for (int qq = 0; qq < 2; ++qq) {
-        float v[4];
-#pragma unroll
-        for (int d = 0; d < 2; ++d) {
-          v[2 * d] = __builtin_bit_cast(float, __builtin_amdgcn_perm(h[j][2 * qq + d], l[j][2 * qq + d], kSelLow)) * coef;
-          v[2 * d + 1] = __builtin_bit_cast(float, __builtin_amdgcn_perm(h[j][2 * qq + d], l[j][2 * qq + d], kSelHigh)) * coef;
-        }
-        const int rq = (j & 1) * 2 + qq;
-        u32x2_t o;
-        o[0] = pack2<T>(v[0], v[1]);
-        o[1] = pack2<T>(v[2], v[3]);
-        *reinterpret_cast<u32x2_t*>(my + (lane & 31) * kRowBytes + ((j >> 1) * kBlk + 8 * rq + 4 * half) * 2) = o;
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int r = it * 4 + (lane >> 4), piece = lane & 15;
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(my + r * kRowBytes + piece * 16);
-      const int64_t row = g.row0 + w_row * kWaveTile + rb * kBlk + r;
-      const int64_t col = g.col0 + w_col * kWaveTile + piece * 8;
-      // pieces that start at or past the last column are not stored; one that it cuts through is written whole,
-      // into the stride padding of its row
-      if (row < g.row_limit && col < g.col_limit)
-        __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(out + row * a.lddw + col));
-    }
-    __builtin_amdgcn_wave_barrier();
-  }
-}
-
 // Whole tiles that meet the plane of sums over chunks of token rows (nothing is split along K then).
 template <class T, bool WVH, int MODE> hipError_t launch_plane(const BwdArgs& a, hipStream_t s) {
-  hipError_t e = a.dw_acc == 1 ? launch_tiles<T, WVH, MODE, 1>(a, s) : launch_tiles<T, WVH, MODE, 2>(a, s);
-  if (e != hipSuccess || !a.last_chunk) return e;
-  const dim3 grid((unsigned)((a.vs / kTile) * (a.Hp / kTile)));
-  hipLaunchKernelGGL((dw_plane_split_out_kernel<T, WVH>), grid, dim3(256), 0, s, a);
-  return hipGetLastError();
+  if (a.dw_acc == 5) return launch_tiles<T, WVH, MODE, 5>(a, s);  // the last chunk: the sums leave as dW at once
+  return a.dw_acc == 1 ? launch_tiles<T, WVH, MODE, 1>(a, s) : launch_tiles<T, WVH, MODE, 2>(a, s);
 }
 
 template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
@@ -595,7 +599,7 @@ template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipS
   if (a.dw_acc != 0) {
     // (16-bit dW only, and a place for the upper halves of the tiles that the edge of the matrix cuts)
     const bool cut = a.Hp != a.H || a.v0 + a.vs != a.V;
-    if (a.dw_plane == nullptr || a.dw_part != nullptr || a.dw_acc > 2 || a.dw_dtype == DT_F32 || (cut && a.dw_plane_hi == nullptr))
+    if (a.dw_plane == nullptr || a.dw_part != nullptr || (a.dw_acc > 2 && a.dw_acc != 5) || a.dw_dtype == DT_F32 || (cut && a.dw_plane_hi == nullptr))
       return hipErrorInvalidValue;
     return launch_plane<T, WVH, kDwAll>(a, s);
   }

@@ -168,11 +168,11 @@ struct BwdArgs {
   // itself, the lower ones in dw_plane (one block of 256 x 256 halves per tile of dW); dw_plane_hi takes the upper
   // halves of the tiles that the edge of the matrix cuts (null if there is none) -- see lce_bwd_dw.hip.
   // dw_acc: 0 = no sums over chunks (dW is stored as it comes), 1 = the sums are stored (first chunk), 2 = added
-  // to; last_chunk: they are then scaled and stored as dW.
+  // to, 5 = added to, and the result scaled and stored as dW (last chunk).
   // fp32 dW: 3 = the sums times the final factor are stored to dw itself (first chunk), 4 = added to it.
   void* dw_plane;
   void* dw_plane_hi;
-  int dw_acc, last_chunk;
+  int dw_acc;
 };
 
 // Element offset of block (row tile, column group) of a dz stage that is `vs` columns wide.
