@@ -100,7 +100,7 @@ def time_phases_one_pass(cfg, x, y, w, prob, chunks, torch, reps):
         # 2 bytes read and 2 written per logit: bound by memory traffic, not by matrix instructions
         ("stage_scale", _lib.PHASE_BWD_DZ, 0.0, 4.0 * rows * V / chunks),
         ("bwd_dx", _lib.PHASE_BWD_DX, 2.0 * rows * H * V / chunks, 0.0),
-        # (with more than one chunk: the tile kernel adding into the fp32 plane, and after the last chunk the pass that stores dW)
+        # (with more than one chunk: the tile kernel adds into the fp32 sums of dW that are kept over the chunks; the last chunk's launch stores dW)
         ("bwd_dw", _lib.PHASE_BWD_DW, 2.0 * rows * H * V / chunks, 0.0),
         ("pack", _lib.PHASE_PACK, 0.0, 0.0),
     ):

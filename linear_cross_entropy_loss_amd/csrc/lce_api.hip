@@ -436,7 +436,7 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
   }
   if (!f->ok) return false;
   // The two-pass route by the same model: the forward over all tokens, then the backward's plan.  It wins where the
-  // scratch bound leaves only short chunks (every chunk adds a round trip of the whole fp32 plane of dW).
+  // scratch bound leaves only short chunks (every chunk adds a round trip of all the fp32 sums of dW).
   BwdPlan b;
   if (p->route == LCE_ROUTE_AUTO && plan_bwd(p, &b) == LCE_OK) {
     const double fixed = (double)Np * (double)Vp * 4.0 / 8.0e6;
