@@ -20,6 +20,9 @@ files.  Sweep ranges are the reference's: H 2^8..2^13, V 2^8..2^17, N 2^8..2^16
 
 Usage:  python -m linear_cross_entropy_loss_amd.sweep --out DIR
             [--kind speed mem acc] [--acc bf16 fp16 fp16-mixed] [--vars N V H] [--quick]
+        python -m linear_cross_entropy_loss_amd.sweep --out DIR --heads
+            (not one of the reference's protocols: output layers of the sizes of public language models, bf16,
+            time and peak memory of a fwd+bwd step beside eager, and the route the library takes; writes DIR/heads.txt)
 """
 from __future__ import annotations
 
@@ -228,6 +231,70 @@ def run(out, kinds, accs, variables, quick=False, log=print):
     return written
 
 
+# Output layers (hidden size, vocabulary) of the sizes of some public language models, with a token count per step.
+HEADS = [
+    ("gpt2-small", 8192, 768, 50257), ("gpt2-xl", 8192, 1600, 50257), ("llama-2-7b", 16384, 4096, 32000),
+    ("mistral-7b", 16384, 4096, 32768), ("phi-3-mini", 8192, 3072, 32064), ("llama-3-8b", 16384, 4096, 128256),
+    ("llama-3-70b", 8192, 8192, 128256), ("qwen-2.5-7b", 8192, 3584, 152064), ("gemma-2b", 8192, 2048, 256000),
+    ("gemma-2-9b", 8192, 3584, 256000),
+]
+
+
+def run_heads(out, chunk_sizes=(4096, 8192), log=print):
+    """fwd+bwd of each output layer in HEADS, bf16, 5 % of the labels ignored: this package at each N_chunk_size
+    (route, ms, peak GiB beyond the inputs) beside eager F.linear + F.cross_entropy (bench_fusions.py:31-33)."""
+    import torch
+    import torch.nn.functional as F
+
+    from . import _lib, linear_cross_entropy
+
+    lines = [f"{'head':<13}{'N':>7}{'H':>6}{'V':>8} | {'eager ms':>9}{'GiB':>7} | "
+             + " | ".join(f"{'N_chunk ' + str(c):>13}{'ms':>8}{'GiB':>7}{'x eager':>8}" for c in chunk_sizes)]
+    for name, N, H, V in HEADS:
+        torch.manual_seed(0)
+        dt = torch.bfloat16
+        x = torch.randn(N, H, device="cuda", dtype=dt).requires_grad_(True)
+        w = (torch.randn(H, V, device="cuda") / math.sqrt(H)).to(dt).requires_grad_(True)
+        y = torch.randint(0, V, (N,), device="cuda")
+        y[torch.rand(N, device="cuda") < 0.05] = -100
+
+        def measure(step):
+            def run():
+                x.grad = w.grad = None
+                step()
+            ms = _median_ms(torch, run, 3, 10)
+            x.grad = w.grad = None
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+            torch.cuda.reset_peak_memory_stats()
+            initial = torch.cuda.memory_allocated()
+            step()
+            torch.cuda.synchronize()
+            return ms, (torch.cuda.max_memory_allocated() - initial) / 1024**3
+
+        try:
+            e_ms, e_gib = measure(lambda: F.cross_entropy(F.linear(x, w.t()).float(), y).backward())
+        except (RuntimeError, torch.OutOfMemoryError):
+            e_ms = e_gib = float("nan")
+        cells = []
+        for c in chunk_sizes:
+            ldw = V + (-V) % 8
+            prob = _lib.make_problem(N, H, V, H, ldw, H, ldw, dt, dt, dt, dt, -100, 1.0, 0.0, c, False)
+            chunks, rows = _lib.forward_backward_plan(prob)
+            route = f"one, {chunks}x{rows}" if chunks else "two passes"
+            ms, gib = measure(lambda: linear_cross_entropy(x, y, w, N_chunk_size=c)[0].backward())
+            cells.append(f"{route:>13}{ms:>8.2f}{gib:>7.2f}{e_ms / ms:>8.2f}")
+        lines.append(f"{name:<13}{N:>7}{H:>6}{V:>8} | {e_ms:>9.2f}{e_gib:>7.2f} | " + " | ".join(cells))
+        log(lines[-1])
+        del x, w, y
+        torch.cuda.empty_cache()
+    os.makedirs(out, exist_ok=True)
+    path = os.path.join(out, "heads.txt")
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    return path
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--out", required=True)
@@ -235,7 +302,11 @@ def main(argv=None):
     ap.add_argument("--acc", nargs="+", default=["fp16", "bf16", "fp16-mixed"], choices=["fp16", "bf16", "fp16-mixed"])
     ap.add_argument("--vars", nargs="+", default=["H", "N", "V"], choices=["H", "N", "V"])
     ap.add_argument("--quick", action="store_true", help="every third point, fewer repetitions")
+    ap.add_argument("--heads", action="store_true", help="output layers of the sizes of public language models instead")
     args = ap.parse_args(argv)
+    if args.heads:
+        print("wrote", run_heads(args.out, log=lambda m: print(m, flush=True)), flush=True)
+        return 0
     for p in run(args.out, args.kind, args.acc, args.vars, args.quick, log=lambda m: print(m, flush=True)):
         print("wrote", p, flush=True)
     return 0
