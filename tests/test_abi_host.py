@@ -245,6 +245,16 @@ def test_null_and_small_workspace_are_rejected_without_touching_the_gpu(lib):
     assert rc == _lib.LCE_EWORKSPACE
     rc = lib.lce_backward(ctypes.byref(p), one, one, one, one, one, one, ctypes.c_void_p(260), one, one, 1 << 40, None)
     assert rc == _lib.LCE_EINVAL_ARG  # misaligned dx
+    # lce_forward_backward, on its one-pass route (a bf16 problem that it covers) and on the two calls it makes otherwise
+    f32 = dict(x_dtype=torch.float32, w_dtype=torch.float32, dx_dtype=torch.float32, dw_dtype=torch.float32)
+    for kw in (dict(), f32):
+        q = _prob(**kw)
+        args = lambda ws, n, dx=one: (ctypes.byref(q), one, one, one, one, one, one, one, dx, one, ws, n, None)
+        assert lib.lce_forward_backward(*args(None, 0)) == _lib.LCE_EWORKSPACE
+        assert lib.lce_forward_backward(*args(one, 16)) == _lib.LCE_EWORKSPACE
+        assert lib.lce_forward_backward(*args(one, 1 << 40, ctypes.c_void_p(260))) == _lib.LCE_EINVAL_ARG
+        assert lib.lce_forward_backward(ctypes.byref(q), one, one, one, None, one, one, one, one, one, one, 1 << 40,
+                                        None) == _lib.LCE_EINVAL_ARG  # no upstream gradient
 
 
 def test_python_surface_mirrors_reference():
