@@ -363,3 +363,45 @@ def test_forty_draws_over_chunks_packing_monitoring_and_layouts():
             for i in (3, 4):
                 assert abs(a["out5"][i].item() - b["out5"][i].item()) <= 5e-5 * abs(a["out5"][i].item()) + 1e-7, (i, a["out5"], b["out5"])
     assert ran >= 25 and several >= 20, (ran, several)
+
+
+@pytest.mark.pack_auto
+@pytest.mark.parametrize("layout", [0, 1])
+def test_one_pass_is_deterministic_at_the_headline_shape(layout):
+    """N=16384, H=2048, V=131072, bf16, four chunks on all compute units: three calls on a workspace that is overwritten
+    in between give the same loss, lse, dx and dW bit for bit (the sums of dW over the chunks are added in chunk order,
+    dx's K segments in segment order, and dW's upper halves are replaced in place by the results of the last chunk)."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    lib = _lib.load()
+    N, H, V, dt = 16384, 2048, 131072, torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(N, H, device="cuda", generator=g).to(dt)
+    w = (torch.randn((V, H) if layout else (H, V), device="cuda", generator=g) / H ** 0.5).to(dt)
+    y = torch.randint(0, V, (N,), device="cuda", generator=g)
+    y[torch.rand(N, device="cuda", generator=g) < 0.05] = -1
+    ldw = H if layout else V
+    prob = _lib.make_problem(N, H, V, H, ldw, H, ldw, dt, dt, dt, dt, -1, 1.0, 1e-4, 4096, False, 0, 0, 0, layout,
+                             _lib.ROUTE_ONE_PASS)
+    chunks, rows = _lib.forward_backward_plan(prob)
+    print(f"layout={layout}: {chunks} chunks of {rows} rows", flush=True)
+    assert chunks >= 3
+    ub = _lib.forward_backward_workspace_bytes(prob)
+    ws = torch.empty(ub, dtype=torch.uint8, device="cuda")
+    one = torch.ones(1, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    runs = []
+    for fill in (0x00, 0x5a, 0xff):
+        ws.fill_(fill)
+        o = dict(lse=torch.empty(N, device="cuda"), out5=torch.empty(5, device="cuda"),
+                 nv=torch.empty(1, dtype=torch.int64, device="cuda"), dx=torch.full((N, H), 3.0, dtype=dt, device="cuda"),
+                 dw=torch.full(w.shape, float(fill), dtype=dt, device="cuda"))
+        rc = lib.lce_forward_backward(ctypes.byref(prob), P(x), P(w), P(y), P(one), P(o["lse"]), P(o["out5"]), P(o["nv"]),
+                                      P(o["dx"]), P(o["dw"]), P(ws), ub, st)
+        assert rc == 0, (rc, lib.lce_last_hip_error())
+        torch.cuda.synchronize()
+        runs.append(o)
+    assert torch.isfinite(runs[0]["dw"]).all() and torch.isfinite(runs[0]["dx"]).all()
+    for o in runs[1:]:
+        for k in o:
+            assert torch.equal(o[k], runs[0][k]), k
