@@ -299,8 +299,7 @@ enum {
  *
  * Problems this route does not cover take the two calls above, one after the
  * other on the same workspace, inside this entry point: fp32 activations, a
- * weight that is neither of x's dtype nor fp32, monitoring != 0 with a hidden
- * size that is not a multiple of 128, and shapes whose sums of dW leave no
+ * weight that is neither of x's dtype nor fp32, and shapes whose sums of dW leave no
  * room for a chunk within the bound (a 16-bit dW with H near 2 * n_chunk or
  * above; lce_forward_backward_plan then reports 0 chunks).  `phases` selects kernels of either route; on the one-pass
  * route LCE_PHASE_FWD_TILES is the logit kernel and LCE_PHASE_BWD_DZ the pass

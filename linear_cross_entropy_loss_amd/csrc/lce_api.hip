@@ -344,8 +344,6 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
   memset(f, 0, sizeof(*f));
   const bool x16 = p->x_dtype == LCE_BF16 || p->x_dtype == LCE_F16;
   if (!x16 || (p->w_dtype != p->x_dtype && p->w_dtype != LCE_F32) || p->route == LCE_ROUTE_TWO_PASS) return false;
-  // (the logit kernel of this route has no variant with both the monitoring sums and a K mask: lce_bwd_dz.hip)
-  if (p->monitoring && lce::padded_k(p->H) != p->H) return false;
   const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V), Hp = (size_t)lce::padded_hidden(p->H);
   const size_t dxes = p->dx_dtype == LCE_F32 ? 4 : 2;
   // (packed rows of dx go to their tokens through 32-bit offsets into dx)

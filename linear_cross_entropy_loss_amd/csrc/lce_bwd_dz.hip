@@ -297,7 +297,8 @@ LCE_DEV void dz_epilogue_impl(const BwdArgs& a, const int (&pf_y)[kNB], const fl
 // both arms above it and needs every vector register at once.
 // The launch covers `tiles_p` tile columns of the slab starting at column tile
 // `tp0`: all the full ones, or (VTAIL) those from the one straddling the end
-// of the vocabulary to the end of the padded slab.
+// of the vocabulary to the end of the padded slab -- or, with BwdArgs::vtail_all, every column (the VTAIL code
+// is right for full columns too, only slower).
 // WVH: the weight is stored (V, H) row-major, so that the P operand runs along K in memory like x does.
 template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH, bool FUSE = false> struct DzProblem {
   typedef typename elem_of<T>::type E;
@@ -311,8 +312,8 @@ template <class T, bool ZREG, bool VTAIL, bool KMASK, bool SPLIT, bool WVH, bool
   const E* x;
   int tp0, tiles_p, tiles_q;
   LCE_DEV DzProblem(const BwdArgs& a_)
-      : a(a_), tp0(VTAIL ? (int)(a_.vw / kTile) : 0),
-        tiles_p(VTAIL ? (int)(a_.vs / kTile - a_.vw / kTile) : (int)(a_.vw / kTile)) {
+      : a(a_), tp0(VTAIL && !a_.vtail_all ? (int)(a_.vw / kTile) : 0),
+        tiles_p(VTAIL ? (int)(a_.vs / kTile) - (a_.vtail_all ? 0 : (int)(a_.vw / kTile)) : (int)(a_.vw / kTile)) {
     rows = packed_rows(a.n_rows, a.N);
     const bool packed = rows != a.N;
     x = reinterpret_cast<const E*>(packed ? a.xc : a.x);
@@ -390,9 +391,13 @@ hipError_t launch_persistent_z(const BwdArgs& a, hipStream_t s) {
   if (full > 0) {
     hipError_t e;
     if constexpr (FUSE && ZREG) {
-      // (the monitoring sums on top of the K mask do not fit the registers; such problems -- a hidden size that is not
-      // a multiple of 128 -- take two passes, lce_api.hip)
-      if (!exact_k) return hipErrorInvalidValue;
+      // (the monitoring sums on top of the K mask do not fit the registers in the kernel for full columns: a hidden
+      // size that is not a multiple of 128 sends every column through the kernel for the last one, which has both)
+      if (!exact_k) {
+        BwdArgs all = a;
+        all.vtail_all = 1;
+        return launch_one<T, ZREG, true, true, SPLIT, WVH, FUSE>(all, (a.vs / kTile) * tq, s);
+      }
       e = launch_one<T, ZREG, false, false, SPLIT, WVH, FUSE>(a, full * tq, s);
     } else {
       e = exact_k ? launch_one<T, ZREG, false, false, SPLIT, WVH, FUSE>(a, full * tq, s)

@@ -173,6 +173,7 @@ struct BwdArgs {
   void* dw_plane;
   void* dw_plane_hi;
   int dw_acc;
+  int vtail_all;  // the logit kernel for the tile column that straddles the end of the vocabulary takes every column
 };
 
 // Element offset of block (row tile, column group) of a dz stage that is `vs` columns wide.

@@ -507,15 +507,18 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
     prob = _lib.make_problem(16384, 2048, 131072, 2048, 131072, 2048, 131072, torch.bfloat16, torch.bfloat16,
                              torch.bfloat16, torch.bfloat16, -1, 1.0, 0.0, 4096, False)
     assert _lib.forward_backward_plan(prob) == (4, 4096)
-    # no one-pass route for fp32 activations, nor for the monitoring values with a hidden size that needs the K mask
-    for kw in (dict(x=torch.float32, w=torch.float32), dict(mon=True, H=520)):
+    # no one-pass route for fp32 activations
+    for kw in (dict(x=torch.float32, w=torch.float32),):
         xd, wd, Hh = kw.get("x", torch.bfloat16), kw.get("w", torch.bfloat16), kw.get("H", 512)
         prob = _lib.make_problem(4096, Hh, 8192, Hh, 8192, Hh, 8192, xd, wd, xd, wd, -1, 1.0, 0.0, 4096,
                                  kw.get("mon", False), route=_lib.ROUTE_ONE_PASS)
         assert _lib.forward_backward_plan(prob) == (0, 0), kw
     prob = _lib.make_problem(4096, 512, 8192, 512, 8192, 512, 8192, torch.bfloat16, torch.bfloat16, torch.bfloat16,
                              torch.bfloat16, -1, 1.0, 0.0, 4096, True, route=_lib.ROUTE_ONE_PASS)
-    assert _lib.forward_backward_plan(prob)[0] > 0  # monitoring with H a multiple of 128: covered
+    assert _lib.forward_backward_plan(prob)[0] > 0  # the monitoring values are covered
+    prob = _lib.make_problem(4096, 520, 8192, 520, 8192, 520, 8192, torch.bfloat16, torch.bfloat16, torch.bfloat16,
+                             torch.bfloat16, -1, 1.0, 0.0, 4096, True, route=_lib.ROUTE_ONE_PASS)
+    assert _lib.forward_backward_plan(prob)[0] > 0  # also with a hidden size that is no multiple of 128
     # a 16-bit dW whose rows are 8 MiB apart or more: its sums over chunks cannot live in it (32-bit offsets over the
     # 256 rows of a tile), so more than one chunk is not planned; an fp32 dW is summed in place and may
     V = 1 << 22

@@ -156,6 +156,10 @@ MON_CASES = [
     (4096, 512, 4096, torch.bfloat16, 1024, 0.7, 1e-4, 1.0, 1, 0),
     (6000, 256, 3000, torch.float16, 1024, 0.45, 0.0, 0.5, 1, 1),    # 6 chunks, the edge of dW cuts tiles, (V, H)
     (4096, 512, 4096, torch.float16, 1024, 0.97, 0.0, 1.0, 1, 0),    # kept rows in the first chunk only
+    # hidden sizes that are no multiple of 128: the K mask and the monitoring sums together
+    (3000, 520, 5000, torch.bfloat16, 1024, 0.1, 1e-4, 1.0, 1, 0),
+    (3000, 200, 4096, torch.float16, 1024, 0.3, 0.0, 0.5, 2, 1),
+    (700, 72, 777, torch.bfloat16, 4096, 0.0, 1e-3, 2.0, 0, 0),
 ]
 
 
@@ -336,7 +340,7 @@ def test_forty_draws_over_chunks_packing_monitoring_and_layouts():
     ran = several = 0
     for it in range(40):
         mon = rng.random() < 0.5
-        H = rng.choice([128, 256, 384, 512, 640]) if mon else rng.choice([64, 200, 256, 520, 768])
+        H = rng.choice([64, 200, 256, 520, 768, 128, 384, 640])
         N = rng.choice([1500, 3000, 4096, 5000, 9000])
         V = rng.choice([2048, 3000, 4096, 5000, 8200])
         dt = rng.choice([torch.bfloat16, torch.float16])

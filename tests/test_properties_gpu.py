@@ -647,8 +647,8 @@ def test_operators_of_the_one_pass_route_pass_opcheck_and_equal_the_eager_functi
     ops.one_pass.set("always")
     for dt in (torch.bfloat16, torch.float16):
         for vh in (False, True):
-            # (a hidden size that is a multiple of 128: with the monitoring values, others take two passes, where the
-            # eager function folds the upstream gradient into its backward kernels and the operator rounds twice)
+            # (a problem that the one-pass route covers: on others the eager function folds the upstream gradient into
+            # its backward kernels, while the operator rounds twice)
             x, y, w = make_inputs(2000, 256, 5000, dt, seed=14, ignore_frac=0.1, device="cuda")
             res = []
             for via_op in (False, True):
