@@ -287,6 +287,11 @@ enum {
  * as two 16-bit halves per sum, the upper halves in the caller's dw -- which
  * holds no meaningful values until the call is done --, the lower halves in
  * H * V * 2 bytes of the workspace (nothing of this with a single chunk).
+ * Where the bound has no room for those (H near 2 * n_chunk and above), one
+ * byte of each lower half is kept instead (H * V bytes): the sums are then
+ * rounded to nearest at 24 bits, 16 of mantissa, each time they go back to
+ * memory -- with C chunks a relative error of at most C * 2^-17 before the
+ * final rounding to the 16-bit dW.
  * The chunks are as long as n_chunk * V * 4 bytes allow, or shorter where the
  * library's model of its kernels finds that faster.  8*N*H*V FLOPs become
  * 6*N*H*V.
@@ -300,7 +305,7 @@ enum {
  * Problems this route does not cover take the two calls above, one after the
  * other on the same workspace, inside this entry point: fp32 activations, a
  * weight that is neither of x's dtype nor fp32, and shapes whose sums of dW leave no
- * room for a chunk within the bound (a 16-bit dW with H near 2 * n_chunk or
+ * room for a chunk within the bound (a 16-bit dW with H near 4 * n_chunk or
  * above; lce_forward_backward_plan then reports 0 chunks).  `phases` selects kernels of either route; on the one-pass
  * route LCE_PHASE_FWD_TILES is the logit kernel and LCE_PHASE_BWD_DZ the pass
  * that turns e into dz.

@@ -338,10 +338,23 @@ struct FusedPlan {
   int64_t ld16;    // row stride of the 16-bit copy of an fp32 weight
   bool parts_on;
   bool dw_direct;  // fp32 dW: the chunks' terms are added in the caller's buffer, there is no plane
+  bool lo8;        // the lower halves of a 16-bit dW's sums are cut to a byte (no room for more: lce_bwd_dw.hip)
 };
 
+bool plan_fused_with(const lce_problem* p, bool want_dx, bool want_dw, bool lo8, FusedPlan* f);
+
+// The lower halves of the fp32 sums of a 16-bit dW at 16 bits where that fits the bound (the sums are then exact
+// fp32), else at 8 (sums of 24 bits).
 bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) {
+  if (plan_fused_with(p, want_dx, want_dw, false, f)) return true;
+  // (only where no plan at all fits: a plan that fits and loses to two passes by the model stays lost)
+  if (f->chunks != 0 || !want_dw || p->dw_dtype == LCE_F32) return false;
+  return plan_fused_with(p, want_dx, want_dw, true, f);
+}
+
+bool plan_fused_with(const lce_problem* p, bool want_dx, bool want_dw, bool lo8, FusedPlan* f) {
   memset(f, 0, sizeof(*f));
+  f->lo8 = lo8;
   const bool x16 = p->x_dtype == LCE_BF16 || p->x_dtype == LCE_F16;
   if (!x16 || (p->w_dtype != p->x_dtype && p->w_dtype != LCE_F32) || p->route == LCE_ROUTE_TWO_PASS) return false;
   const size_t Np = (size_t)lce::padded_tokens(p->N), Vp = (size_t)lce::padded_vocab(p->V), Hp = (size_t)lce::padded_hidden(p->H);
@@ -387,7 +400,7 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     out->part = t; t += pb;
     out->parts_on = pb != 0;
     out->plane = t;
-    if (chunks > 1 && want_dw && !f->dw_direct) t += align_up(Hp * Vp * 2);
+    if (chunks > 1 && want_dw && !f->dw_direct) t += align_up(Hp * Vp * (lo8 ? 1 : 2));
     // (upper halves of the tiles that the edge of dW cuts: the last tile row over h, the last over v)
     out->plane_hi = t;
     if (chunks > 1 && want_dw && !f->dw_direct)
@@ -440,7 +453,7 @@ bool plan_fused(const lce_problem* p, bool want_dx, bool want_dw, FusedPlan* f) 
     const double fixed = (double)Np * (double)Vp * 4.0 / 8.0e6;
     const double two = kernel_cost((double)tiles * tv, (double)(lce::padded_k(p->H) / 64), 4.0, false) + b.cost;
     if (best + fixed > two) {
-      f->ok = false;
+      f->ok = false;  // (f->chunks stays: a plan fitted)
       return false;
     }
   }
@@ -705,8 +718,10 @@ int fused_impl(const lce_problem* p, const FusedPlan& f, const void* x, const vo
       a.y = y + row0;
       a.dx = dx ? (char*)dx + (size_t)row0 * (size_t)p->lddx * dxes : nullptr;
     }
-    // dW over the chunks: as halves (1: store, 2: add, 5: add and store dW), or -- fp32 dW -- in the caller's buffer itself (3: store, 4: add)
-    a.dw_acc = f.chunks == 1 ? 0 : (f.dw_direct ? (c == 0 ? 3 : 4) : (c == 0 ? 1 : (c == f.chunks - 1 ? 5 : 2)));
+    // dW over the chunks: as halves (1: store, 2: add, 5: add and store dW; 6, 7, 8 with the lower halves cut to a byte), or
+    // -- fp32 dW -- in the caller's buffer itself (3: store, 4: add)
+    const bool last = c == f.chunks - 1;
+    a.dw_acc = f.chunks == 1 ? 0 : f.dw_direct ? (c == 0 ? 3 : 4) : f.lo8 ? (c == 0 ? 6 : last ? 8 : 7) : (c == 0 ? 1 : last ? 5 : 2);
     if (f.pack && (ph & (LCE_PHASE_PACK | LCE_PHASE_FWD_TILES | LCE_PHASE_BWD_DW))) {
       e = lce::launch_gather_rows(x, p->ldx * 2, p->H * 2, perm + row0, chunk_rows + (all_rows ? 1024 : 0) + c, p->N,
                                   base + f.xc, k.ldxc * 2, nullptr, nullptr, num_cus, s, true);

@@ -201,7 +201,22 @@ LCE_DEV void dw_epilogue(const BwdArgs& a, float* part, f32x16_t (&acc)[kNB][kNB
 // (lane % 16) * 16.  So the last chunk can turn the sums into dW in place, 32 rows at a time (dw_plane_split_final).
 // (Hardware fp32 atomic adds into an fp32 plane instead of load - add - store were measured at the headline
 // shape: the 268 M atomics of a chunk take longer than the chunk's matrix work, 30.6 ms a step against 22.3.)
+//   LO8 (BwdArgs::dw_acc 6 to 8), for problems whose scratch bound has no room for H * V * 2 bytes of lower halves: only
+// the upper byte of each lower half is kept (H * V bytes; pair p of thread t at byte p * 2048 + t * 8 of a 64 KiB
+// block), and a sum is rounded to nearest at those 24 bits -- 16 of mantissa -- every time it goes back to memory:
+// with C chunks a relative error of at most C * 2^-17 before the final rounding to the 16-bit dW.
 constexpr unsigned kSelLow = 0x05040100u, kSelHigh = 0x07060302u;  // v_perm selectors: the lower / upper halves of (S0, S1)
+
+// Sum number e (0..7) of a pair from the dword of upper halves that holds its upper half and the lower parts.
+template <bool LO8, class L> LCE_DEV float dw_sum_of(const u32x4_t& h, const L& l, int e) {
+  if constexpr (LO8) {
+    // bytes (0, lower part e % 4 of dword e / 4, the two bytes of upper half e % 2 of dword e / 2)
+    const unsigned sel = ((5u + 2u * (e & 1)) << 24) | ((4u + 2u * (e & 1)) << 16) | ((unsigned)(e & 3) << 8) | 0x0cu;
+    return __builtin_bit_cast(float, __builtin_amdgcn_perm(h[e >> 1], l[e >> 2], sel));
+  } else {
+    return __builtin_bit_cast(float, __builtin_amdgcn_perm(h[e >> 1], l[e >> 1], (e & 1) ? kSelHigh : kSelLow));
+  }
+}
 
 // Where the upper halves of tile (tp, tq) lie, and the distance of their rows in bytes.
 template <bool WVH>
@@ -219,54 +234,65 @@ LCE_DEV char* dw_hi_block(const BwdArgs& a, int tp, int tq, int& stride) {
   return reinterpret_cast<char*>(a.dw_plane_hi) + (int64_t)e * (kTile * kTile * 2);
 }
 
-template <bool LOAD, bool WVH>
+template <bool LOAD, bool WVH, bool LO8>
 LCE_DEV void dw_plane_split_io(char* hi, int hi_stride, char* lo, f32x16_t (&acc)[kNB][kNB]) {
+  typedef typename std::conditional<LO8, u32x2_t, u32x4_t>::type L;
+  constexpr int kLoBytes = LO8 ? 8 : 16;  // of a pair and thread
   // one descriptor per block, the thread's place as the vector offset, the pair as a scalar offset: no 64-bit
   // address per pair
   const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(hi, 0, 255 * hi_stride + 512, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rl = __builtin_amdgcn_make_buffer_rsrc(lo, 0, kTile * kTile * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rl = __builtin_amdgcn_make_buffer_rsrc(lo, 0, 32 * kThreads * kLoBytes, 0x00020000);
   const int tid = opaque_tid();
   const int lane = tid & 63, wave = tid >> 6;
   const int wp = wave & 1, wq = wave >> 1;
   const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
   const int vh = (w_row * kWaveTile + (lane >> 4)) * hi_stride + w_col * 256 + (lane & 15) * 16;
-  const int vl = tid * 16;
+  const int vl = tid * kLoBytes;
   // kBatch pairs are fetched together before any is used: their loads are in flight together (2, 8 and 16 pairs
   // measured the same)
   constexpr int kBatch = 8;
 #pragma unroll
   for (int p0 = 0; p0 < 32; p0 += kBatch) {
-    u32x4_t oh[kBatch], ol[kBatch];
+    u32x4_t oh[kBatch];
+    L ol[kBatch];
     if (LOAD) {
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
         const int p = p0 + u, i = p >> 3, k = (p >> 1) & 3, rb = WVH ? k : i, cb = WVH ? i : k;
         oh[u] = __builtin_amdgcn_raw_buffer_load_b128(rh, vh, (rb * kBlk + (cb * 2 + (p & 1)) * 4) * hi_stride, 0);
-        ol[u] = __builtin_amdgcn_raw_buffer_load_b128(rl, vl, p * 4096, 0);
+        if constexpr (LO8) ol[u] = __builtin_amdgcn_raw_buffer_load_b64(rl, vl, p * (kThreads * kLoBytes), 0);
+        else ol[u] = __builtin_amdgcn_raw_buffer_load_b128(rl, vl, p * (kThreads * kLoBytes), 0);
       }
     }
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
       const int p = p0 + u, i = p >> 3, k = (p >> 1) & 3, rb = WVH ? k : i, cb = WVH ? i : k;
-      float f[8];
+      unsigned r[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         // (a volatile read: the compiler would otherwise read all 256 accumulator registers before the first load)
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(f[j]) : "a"(acc[i][k][(p & 1) * 8 + j]));
+        float f;
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(f) : "a"(acc[i][k][(p & 1) * 8 + j]));
+        if (LOAD) f += dw_sum_of<LO8>(oh[u], ol[u], j);
+        r[j] = __builtin_bit_cast(unsigned, f);
+        if constexpr (LO8) r[j] += 0x7fu + ((r[j] >> 8) & 1u);  // to nearest (even) at 24 bits; the last byte is dropped below
       }
-      u32x4_t nh, nl;
+      u32x4_t nh;
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        if (LOAD) {
-          f[2 * d] += __builtin_bit_cast(float, __builtin_amdgcn_perm(oh[u][d], ol[u][d], kSelLow));
-          f[2 * d + 1] += __builtin_bit_cast(float, __builtin_amdgcn_perm(oh[u][d], ol[u][d], kSelHigh));
-        }
-        const unsigned f0 = __builtin_bit_cast(unsigned, f[2 * d]), f1 = __builtin_bit_cast(unsigned, f[2 * d + 1]);
-        nh[d] = __builtin_amdgcn_perm(f1, f0, kSelHigh);
-        nl[d] = __builtin_amdgcn_perm(f1, f0, kSelLow);
-      }
+      for (int d = 0; d < 4; ++d) nh[d] = __builtin_amdgcn_perm(r[2 * d + 1], r[2 * d], kSelHigh);
       __builtin_amdgcn_raw_buffer_store_b128(nh, rh, vh, (rb * kBlk + (cb * 2 + (p & 1)) * 4) * hi_stride, 0);
-      __builtin_amdgcn_raw_buffer_store_b128(nl, rl, vl, p * 4096, 0);
+      if constexpr (LO8) {
+        u32x2_t nl;
+#pragma unroll
+        for (int w = 0; w < 2; ++w)  // byte 1 of four sums
+          nl[w] = __builtin_amdgcn_perm(r[4 * w + 1], r[4 * w], 0x0c0c0501u) | __builtin_amdgcn_perm(r[4 * w + 3], r[4 * w + 2], 0x05010c0cu);
+        __builtin_amdgcn_raw_buffer_store_b64(nl, rl, vl, p * (kThreads * kLoBytes), 0);
+      } else {
+        u32x4_t nl;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) nl[d] = __builtin_amdgcn_perm(r[2 * d + 1], r[2 * d], kSelLow);
+        __builtin_amdgcn_raw_buffer_store_b128(nl, rl, vl, p * (kThreads * kLoBytes), 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);  // (one batch in registers at a time: an operand tile is in flight)
   }
@@ -278,10 +304,12 @@ LCE_DEV void dw_plane_split_io(char* hi, int hi_stride, char* lo, f32x16_t (&acc
 // bytes of dW that these results will take (dw_plane_split_io), so all of them are loaded before the first row is
 // stored; the values pass through the wave's slice of `scratch` (main-loop stage 1, idle during an epilogue; rows of
 // the slice are 272 bytes apart: 16-byte pieces stay aligned, lanes on consecutive rows use different banks).
-template <class T, bool WVH>
+template <class T, bool WVH, bool LO8>
 LCE_DEV void dw_plane_split_final(const BwdArgs& a, const char* hi, int hi_stride, const char* lo, f32x16_t (&acc)[kNB][kNB],
                                   int tp, int tq, char* scratch) {
   typedef typename elem_of<T>::type E;
+  typedef typename std::conditional<LO8, u32x2_t, u32x4_t>::type L;
+  constexpr int kLoBytes = LO8 ? 8 : 16;
   constexpr int kRowBytes = 256 + 16;
   static_assert(kBlk * kRowBytes <= kDwSliceBytes, "a block row of results fits a wave's slice");
   const DwTileGeom<WVH> g(a, tp, tq);
@@ -291,19 +319,21 @@ LCE_DEV void dw_plane_split_final(const BwdArgs& a, const char* hi, int hi_strid
   const int wp = wave & 1, wq = wave >> 1, half = lane >> 5;
   const int w_row = WVH ? wq : wp, w_col = WVH ? wp : wq;
   const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(hi), 0, 255 * hi_stride + 512, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rl = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(lo), 0, kTile * kTile * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rl = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(lo), 0, 32 * kThreads * kLoBytes, 0x00020000);
   const int vh = (w_row * kWaveTile + (lane >> 4)) * hi_stride + w_col * 256 + (lane & 15) * 16;
-  const int vl = tid * 16;
+  const int vl = tid * kLoBytes;
   char* my = scratch + wave * kDwSliceBytes;
   E* out = reinterpret_cast<E*>(a.dw);
 #pragma unroll
   for (int rb = 0; rb < kNB; ++rb) {
-    u32x4_t h[8], l[8];
+    u32x4_t h[8];
+    L l[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int cb = j >> 1, i = WVH ? cb : rb, k = WVH ? rb : cb;  // the pair is of block acc[i][k]
       h[j] = __builtin_amdgcn_raw_buffer_load_b128(rh, vh, (rb * kBlk + j * 4) * hi_stride, 0);
-      l[j] = __builtin_amdgcn_raw_buffer_load_b128(rl, vl, ((i * 4 + k) * 2 + (j & 1)) * 4096, 0);
+      if constexpr (LO8) l[j] = __builtin_amdgcn_raw_buffer_load_b64(rl, vl, ((i * 4 + k) * 2 + (j & 1)) * (kThreads * kLoBytes), 0);
+      else l[j] = __builtin_amdgcn_raw_buffer_load_b128(rl, vl, ((i * 4 + k) * 2 + (j & 1)) * (kThreads * kLoBytes), 0);
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -317,8 +347,8 @@ LCE_DEV void dw_plane_split_final(const BwdArgs& a, const char* hi, int hi_strid
           // (volatile reads: the compiler would otherwise read all 256 accumulator registers before the first load)
           asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a0) : "a"(acc[i][k][(j & 1) * 8 + qq * 4 + 2 * d]));
           asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a1) : "a"(acc[i][k][(j & 1) * 8 + qq * 4 + 2 * d + 1]));
-          v[2 * d] = (a0 + __builtin_bit_cast(float, __builtin_amdgcn_perm(h[j][2 * qq + d], l[j][2 * qq + d], kSelLow))) * coef;
-          v[2 * d + 1] = (a1 + __builtin_bit_cast(float, __builtin_amdgcn_perm(h[j][2 * qq + d], l[j][2 * qq + d], kSelHigh))) * coef;
+          v[2 * d] = (a0 + dw_sum_of<LO8>(h[j], l[j], qq * 4 + 2 * d)) * coef;
+          v[2 * d + 1] = (a1 + dw_sum_of<LO8>(h[j], l[j], qq * 4 + 2 * d + 1)) * coef;
         }
         const int rq = (j & 1) * 2 + qq;
         u32x2_t o;
@@ -515,9 +545,10 @@ template <class T, bool WVH, int MODE, int ACC = 0> struct DwProblem {
     } else if constexpr (ACC != 0) {
       int stride;
       char* hi = dw_hi_block<WVH>(a, tp, tq, stride);
-      char* lo = reinterpret_cast<char*>(a.dw_plane) + ((int64_t)tq * tiles_p + tp) * (kTile * kTile * 2);
-      if constexpr (ACC == 5) dw_plane_split_final<T, WVH>(a, hi, stride, lo, acc, tp, tq, scratch);
-      else dw_plane_split_io<ACC == 2, WVH>(hi, stride, lo, acc);
+      constexpr bool kLo8 = ACC >= 6;
+      char* lo = reinterpret_cast<char*>(a.dw_plane) + ((int64_t)tq * tiles_p + tp) * (kTile * kTile * (kLo8 ? 1 : 2));
+      if constexpr (ACC == 5 || ACC == 8) dw_plane_split_final<T, WVH, kLo8>(a, hi, stride, lo, acc, tp, tq, scratch);
+      else dw_plane_split_io<ACC == 2 || ACC == 7, WVH, kLo8>(hi, stride, lo, acc);
       return;
     }
     if (MODE == kDwStaged || MODE == kDwStaged32) {
@@ -535,7 +566,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dw_persistent_kernel(const BwdAr
   typedef typename elem_of<T>::type E;
   DwProblem<T, WVH, MODE, ACC> prob(a);
   // (a chunk without a kept row adds nothing to the sums of the earlier chunks)
-  if ((ACC == 2 || ACC == 4) && prob.rows == 0) return;
+  if ((ACC == 2 || ACC == 4 || ACC == 7) && prob.rows == 0) return;
   Pipe3<T, E, false, E, false, DwProblem<T, WVH, MODE, ACC>> pipe(prob);
   pipe.run(prob.ldx, a.vs / kBK, prob.plan.kt, lds);
 }
@@ -585,8 +616,15 @@ template <class T, bool WVH, int MODE, int ACC = 0> hipError_t launch_tiles(cons
 
 // Whole tiles that meet the plane of sums over chunks of token rows (nothing is split along K then).
 template <class T, bool WVH, int MODE> hipError_t launch_plane(const BwdArgs& a, hipStream_t s) {
-  if (a.dw_acc == 5) return launch_tiles<T, WVH, MODE, 5>(a, s);  // the last chunk: the sums leave as dW at once
-  return a.dw_acc == 1 ? launch_tiles<T, WVH, MODE, 1>(a, s) : launch_tiles<T, WVH, MODE, 2>(a, s);
+  switch (a.dw_acc) {
+    case 1: return launch_tiles<T, WVH, MODE, 1>(a, s);
+    case 2: return launch_tiles<T, WVH, MODE, 2>(a, s);
+    case 5: return launch_tiles<T, WVH, MODE, 5>(a, s);  // the last chunk: the sums leave as dW at once
+    case 6: return launch_tiles<T, WVH, MODE, 6>(a, s);  // the same three with the lower halves cut to a byte
+    case 7: return launch_tiles<T, WVH, MODE, 7>(a, s);
+    case 8: return launch_tiles<T, WVH, MODE, 8>(a, s);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipStream_t s) {
@@ -597,7 +635,7 @@ template <class T, bool WVH> hipError_t launch_persistent(const BwdArgs& a, hipS
   if (a.dw_acc != 0) {
     // (16-bit dW only, and a place for the upper halves of the tiles that the edge of the matrix cuts)
     const bool cut = a.Hp != a.H || a.v0 + a.vs != a.V;
-    if (a.dw_plane == nullptr || a.dw_part != nullptr || (a.dw_acc > 2 && a.dw_acc != 5) || a.dw_dtype == DT_F32 || (cut && a.dw_plane_hi == nullptr))
+    if (a.dw_plane == nullptr || a.dw_part != nullptr || a.dw_dtype == DT_F32 || (cut && a.dw_plane_hi == nullptr))
       return hipErrorInvalidValue;
     return launch_plane<T, WVH, kDwAll>(a, s);
   }

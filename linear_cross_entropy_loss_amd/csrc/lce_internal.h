@@ -168,7 +168,8 @@ struct BwdArgs {
   // itself, the lower ones in dw_plane (one block of 256 x 256 halves per tile of dW); dw_plane_hi takes the upper
   // halves of the tiles that the edge of the matrix cuts (null if there is none) -- see lce_bwd_dw.hip.
   // dw_acc: 0 = no sums over chunks (dW is stored as it comes), 1 = the sums are stored (first chunk), 2 = added
-  // to, 5 = added to, and the result scaled and stored as dW (last chunk).
+  // to, 5 = added to, and the result scaled and stored as dW (last chunk); 6, 7, 8 = the same three with only the
+  // upper byte of each lower half kept (dw_plane: 256 x 256 bytes per tile; the sums are rounded at 24 bits).
   // fp32 dW: 3 = the sums times the final factor are stored to dw itself (first chunk), 4 = added to it.
   void* dw_plane;
   void* dw_plane_hi;

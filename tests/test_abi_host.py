@@ -500,8 +500,8 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
         assert rows % 256 == 0 and rows > 0
         assert chunks * rows >= N and (chunks - 1) * rows < N + 255
         assert total <= n_chunk * V * 4, (N, H, V, n_chunk, total)
-        if chunks > 1:  # the lower halves of the fp32 sums of dW are part of it (the upper halves lie in dW itself)
-            assert total >= (H + (-H) % 256) * (V + (-V) % 256) * 2
+        if chunks > 1:  # the lower halves of the fp32 sums of dW are part of it (the upper halves lie in dW itself),
+            assert total >= (H + (-H) % 256) * (V + (-V) % 256)  # cut to a byte each where two do not fit the bound
     assert took > 50
     # the benchmark's default shape: four chunks of 16 token tiles
     prob = _lib.make_problem(16384, 2048, 131072, 2048, 131072, 2048, 131072, torch.bfloat16, torch.bfloat16,
@@ -519,6 +519,12 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
     prob = _lib.make_problem(4096, 520, 8192, 520, 8192, 520, 8192, torch.bfloat16, torch.bfloat16, torch.bfloat16,
                              torch.bfloat16, -1, 1.0, 0.0, 4096, True, route=_lib.ROUTE_ONE_PASS)
     assert _lib.forward_backward_plan(prob)[0] > 0  # also with a hidden size that is no multiple of 128
+    # H = 2 * N_chunk_size: the lower halves of a 16-bit dW's sums alone are the bound, a byte of each fits
+    prob = _lib.make_problem(16384, 8192, 131072, 8192, 131072, 8192, 131072, torch.bfloat16, torch.bfloat16,
+                             torch.bfloat16, torch.bfloat16, -1, 1.0, 0.0, 4096, False, route=_lib.ROUTE_ONE_PASS)
+    chunks, rows = _lib.forward_backward_plan(prob)
+    total = _lib.forward_backward_workspace_bytes(prob)
+    assert chunks > 1 and 8192 * 131072 + rows * 131072 * 2 <= total <= 4096 * 131072 * 4 < 8192 * 131072 * 2 + rows * 131072 * 2
     # a 16-bit dW whose rows are 8 MiB apart or more: its sums over chunks cannot live in it (32-bit offsets over the
     # 256 rows of a tile), so more than one chunk is not planned; an fp32 dW is summed in place and may
     V = 1 << 22
