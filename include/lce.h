@@ -114,8 +114,10 @@ enum {
 
 /*
  * Arithmetic.  16-bit x: products of 16-bit operands (an fp32 master weight is
- * rounded to the type of x), fp32 accumulation; dz is rounded once to the type
- * of x before the two gradient contractions, as the reference casts it
+ * rounded to the type of x), fp32 accumulation (one exception, described at
+ * lce_forward_backward: a 16-bit dW's sums over chunks of token rows at 24
+ * bits where the scratch bound has no room for 32); dz is rounded once to the
+ * type of x before the two gradient contractions, as the reference casts it
  * (ops.py:314, 422).  fp32 x (with an fp32 w): every operand of every
  * contraction, dz included, is carried as a PAIR of bf16 numbers hi + lo
  * (16 bits of mantissa) and each product as hi*hi + hi*lo + lo*hi with fp32
