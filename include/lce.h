@@ -91,7 +91,7 @@ typedef struct lce_problem {
   int32_t pack_rows;    /* LCE_PACK_AUTO | LCE_PACK_ALWAYS | LCE_PACK_NEVER: see below        */
   int32_t max_workgroups; /* profiling aid: cap on the persistent workgroups of the tile kernels (0 = one per compute unit) */
   int32_t w_layout;     /* LCE_W_HV (0) | LCE_W_VH: how w and dw are stored, see below */
-  int32_t route;        /* lce_forward_backward only: LCE_ROUTE_AUTO (0) | LCE_ROUTE_ONE_PASS | LCE_ROUTE_TWO_PASS, see there */
+  int32_t route;        /* lce_forward_backward only: LCE_ROUTE_AUTO (0) | LCE_ROUTE_ONE_PASS | LCE_ROUTE_TWO_PASS, [+ LCE_ROUTE_EXACT_SUMS], see there */
 } lce_problem;
 
 /*
@@ -266,7 +266,9 @@ int lce_backward(const lce_problem* p, const void* x, const void* w, const int64
 enum {
   LCE_ROUTE_AUTO = 0,
   LCE_ROUTE_ONE_PASS = 1,
-  LCE_ROUTE_TWO_PASS = 2
+  LCE_ROUTE_TWO_PASS = 2,
+  /* a flag, to be or-ed to one of the above: a 16-bit dW's sums over chunks are never kept at fewer than 32 bits */
+  LCE_ROUTE_EXACT_SUMS = 4
 };
 
 /*
@@ -289,11 +291,15 @@ enum {
  * as two 16-bit halves per sum, the upper halves in the caller's dw -- which
  * holds no meaningful values until the call is done --, the lower halves in
  * H * V * 2 bytes of the workspace (nothing of this with a single chunk).
- * Where the bound has no room for those (H near 2 * n_chunk and above), one
- * byte of each lower half is kept instead (H * V bytes): the sums are then
- * rounded to nearest at 24 bits, 16 of mantissa, each time they go back to
- * memory -- with C chunks a relative error of at most C * 2^-17 before the
- * final rounding to the 16-bit dW.
+ * Where the bound has no room for those (H near 2 * n_chunk and above), or
+ * where they leave so little room for the chunks that the library's model of
+ * its kernels finds the alternative at least 3 % faster (typically H near
+ * n_chunk and above), one byte of each lower half is kept instead (H * V
+ * bytes): the sums are then rounded to nearest at 24 bits, 16 of mantissa,
+ * each time they go back to memory -- with C chunks a relative error of at
+ * most C * 2^-17 before the final rounding to the 16-bit dW (2^-9 in bf16,
+ * 2^-12 in fp16).  LCE_ROUTE_EXACT_SUMS in lce_problem.route rules that out:
+ * the sums are then fp32 between chunks or the problem takes two passes.
  * The chunks are as long as n_chunk * V * 4 bytes allow, or shorter where the
  * library's model of its kernels finds that faster.  8*N*H*V FLOPs become
  * 6*N*H*V.

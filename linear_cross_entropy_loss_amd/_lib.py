@@ -14,6 +14,7 @@ LCE_OK = 0
 PHASE_FWD_TILES, PHASE_FWD_REDUCE, PHASE_BWD_DZ, PHASE_BWD_DX, PHASE_BWD_DW, PHASE_PACK = 1, 2, 4, 8, 16, 32
 PACK_AUTO, PACK_ALWAYS, PACK_NEVER = 0, 1, 2
 ROUTE_AUTO, ROUTE_ONE_PASS, ROUTE_TWO_PASS = 0, 1, 2  # lce_problem.route (lce_forward_backward)
+ROUTE_EXACT_SUMS = 4  # a flag for the same field: dW's sums over chunks never at fewer than 32 bits
 W_HV, W_VH = 0, 1  # lce_problem.w_layout: weight stored (H, V) / (V, H) row-major
 LCE_EINVAL_SHAPE, LCE_EINVAL_DTYPE, LCE_EINVAL_ARG, LCE_EWORKSPACE, LCE_EHIP, LCE_ESTATIC = -1, -2, -3, -4, -5, -6
 STATIC_SCRATCH_BYTES = 64 << 20

@@ -51,6 +51,12 @@ pack_rows: contextvars.ContextVar = contextvars.ContextVar("lce_pack_rows", defa
 # loss-only forward and the recomputing backward.
 one_pass: contextvars.ContextVar = contextvars.ContextVar("lce_one_pass", default=True)
 
+# On the one-pass route a 16-bit dW is summed over chunks of token rows in fp32 where that fits the scratch bound and
+# leaves room for chunks long enough; elsewhere the sums are kept at 24 bits between chunks (16 of mantissa, rounded to
+# nearest: include/lce.h).  True here rules the 24 bits out (LCE_ROUTE_EXACT_SUMS): such problems then run with shorter
+# chunks or take two passes.  Read when the device call is made.
+exact_dw_sums: contextvars.ContextVar = contextvars.ContextVar("lce_exact_dw_sums", default=False)
+
 
 @torch.compiler.assume_constant_result
 def _pack_mode() -> int:
@@ -230,7 +236,7 @@ def _one_pass_impl(x_in, y, At, ignore_index, z_regularization, logit_scale, N_c
         prob = _lib.make_problem(
             N, H, V, x.stride(0), w.stride(0), H + (-H) % 8, w_cols + (-w_cols) % 8, x.dtype, w.dtype, x.dtype, w.dtype,
             ignore_index, logit_scale, z_regularization, N_chunk_size, monitoring, 0, pack, 0, layout,
-            _lib.ROUTE_ONE_PASS if always else _lib.ROUTE_AUTO,
+            (_lib.ROUTE_ONE_PASS if always else _lib.ROUTE_AUTO) | (_lib.ROUTE_EXACT_SUMS if exact_dw_sums.get() else 0),
         )
         lib = _lib.load()
         _lib.raise_for_status(lib.lce_check_problem(ctypes.byref(prob)), "linear_cross_entropy")

@@ -468,7 +468,7 @@ def test_a_weight_that_cannot_be_read_in_place_is_copied_with_one_warning():
         ops._weight_rows(bad, ops._weight_layout(bad, torch.bfloat16))  # the second copy is silent
 
 
-def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
+def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens(lib):
     """lce_forward_backward_plan: chunks of whole token tiles that cover N, a workspace within n_chunk * V * 4
     bytes, and no one-pass route for fp32 tensors, monitoring, or a bound that the fp32 plane of dW alone fills."""
     import random
@@ -545,8 +545,16 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens():
     c16, r16 = _lib.forward_backward_plan(p16)
     c1632, r1632 = _lib.forward_backward_plan(p16_32)
     assert c32 > 1 and c16 > 1 and c1632 > 1
-    plane, copy = 1024 * 32768 * 4, 1024 * 32768 * 2
-    assert r1632 >= r16  # without the plane there is room for longer chunks
+    sums, copy = 1024 * 32768, 1024 * 32768 * 2  # (a 16-bit dW: at least a byte per sum in the workspace)
+    assert r1632 >= r16  # without them there is room for chunks at least as long
     assert _lib.forward_backward_workspace_bytes(p32) >= copy + r32 * 32768 * 2
-    assert _lib.forward_backward_workspace_bytes(p16) >= plane + r16 * 32768 * 2
-    assert _lib.forward_backward_workspace_bytes(p16_32) < plane + r1632 * 32768 * 2
+    assert _lib.forward_backward_workspace_bytes(p16) >= sums + r16 * 32768 * 2
+    # LCE_ROUTE_EXACT_SUMS: two bytes per sum there (the upper halves lie in dW), or no plan
+    p16x = _lib.make_problem(w_dtype=torch.bfloat16, dw_dtype=torch.bfloat16, **dict(kw, route=_lib.ROUTE_ONE_PASS | _lib.ROUTE_EXACT_SUMS))
+    c16x, r16x = _lib.forward_backward_plan(p16x)
+    assert c16x == 0 or (r16x <= r16 and _lib.forward_backward_workspace_bytes(p16x) >= 2 * sums + r16x * 32768 * 2)
+    # the flag goes with every route and with nothing else
+    for r in (0, 1, 2, 4, 5, 6):
+        assert lib.lce_check_problem(ctypes.byref(_lib.make_problem(**dict(kw, w_dtype=torch.bfloat16, dw_dtype=torch.bfloat16, route=r)))) == 0
+    for r in (3, 7, 8, -1):
+        assert lib.lce_check_problem(ctypes.byref(_lib.make_problem(**dict(kw, w_dtype=torch.bfloat16, dw_dtype=torch.bfloat16, route=r)))) == _lib.LCE_EINVAL_ARG

@@ -18,16 +18,17 @@ def P(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
 
-def _problem(N, H, V, x, w, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, phases=0, mon=False):
+def _problem(N, H, V, x, w, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, phases=0, mon=False, exact=False):
     from linear_cross_entropy_loss_amd import _lib
 
     hp, cols = H + (-H) % 8, (H if layout else V)
     return _lib.make_problem(N, H, V, x.stride(0), w.stride(0), hp, cols + (-cols) % 8, dt, w.dtype, dt, dw_dt, -1, scale,
-                             z_reg, n_chunk, mon, phases, pack, 0, layout, _lib.ROUTE_ONE_PASS)
+                             z_reg, n_chunk, mon, phases, pack, 0, layout,
+                             _lib.ROUTE_ONE_PASS | (_lib.ROUTE_EXACT_SUMS if exact else 0))
 
 
 def _both_routes(N, H, V, dt, n_chunk, ignore, z_reg=0.0, scale=1.0, pack=0, layout=0, dw_dt=None, grad_out=1.0,
-                 seed=7, want_chunks=None, w_dt=None, mon=False):
+                 seed=7, want_chunks=None, w_dt=None, mon=False, exact=False):
     """Runs the two routes on the same inputs; returns (inputs on the CPU, two-pass outputs, one-pass outputs)."""
     from linear_cross_entropy_loss_amd import _lib
 
@@ -45,7 +46,7 @@ def _both_routes(N, H, V, dt, n_chunk, ignore, z_reg=0.0, scale=1.0, pack=0, lay
         pad[:, :H] = xd
         xd = pad[:, :H]
     dw_dt = dw_dt or dt
-    prob = _problem(N, H, V, xd, wd, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, mon=mon)
+    prob = _problem(N, H, V, xd, wd, dt, dw_dt, z_reg, scale, n_chunk, pack, layout, mon=mon, exact=exact)
     chunks, rows = _lib.forward_backward_plan(prob)
     print(f"N={N} H={H} V={V} {dt} n_chunk={n_chunk} pack={pack} layout={layout}: {chunks} chunks of {rows} rows", flush=True)
     assert chunks > 0, "this case is meant to take the one-pass route"
@@ -206,6 +207,25 @@ def test_sums_of_dw_with_a_byte_of_each_lower_half(N, H, V, dt, n_chunk, ign, z_
     # of the 16-bit result (2^-9 in bf16, 2^-12 in fp16); the gradients differ by the staged dz's second rounding
     emax, el2 = rel_errors(b["dw"], a["dw"])
     assert el2 <= 3e-3
+
+
+@pytest.mark.pack_auto
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_exact_sums_flag_keeps_the_halves_and_changes_only_the_rounding(dt):
+    """N=8192, H=2048, V=16384 at N_chunk_size 2048 (H = N_chunk_size: the lower halves take half of the bound): the
+    library's plan keeps a byte per sum and runs longer chunks; with LCE_ROUTE_EXACT_SUMS it keeps both halves, in more
+    and shorter chunks.  Both agree with the two-pass route and with fp64, and with each other to the rounding of dz
+    and of the 24 bits."""
+    a_inputs, a2, fast = _both_routes(8192, 2048, 16384, dt, 2048, 0.1, 1e-4, 1.0, 1, 0, seed=21)
+    b_inputs, b2, exact = _both_routes(8192, 2048, 16384, dt, 2048, 0.1, 1e-4, 1.0, 1, 0, seed=21, exact=True)
+    assert fast["chunks"] > 1 and exact["chunks"] > fast["chunks"]
+    _check(a_inputs, a2, fast, 1e-4, 1.0, 1.0, fp64=True)
+    _check(b_inputs, b2, exact, 1e-4, 1.0, 1.0, fp64=True)
+    assert torch.equal(fast["lse"], exact["lse"]) or rel_errors(fast["lse"], exact["lse"])[0] <= 1e-6
+    for name in ("dx", "dw"):
+        emax, el2 = rel_errors(fast[name], exact[name])
+        print(f"  {name} bytes vs halves: max-rel {emax:.3e}  l2-rel {el2:.3e}", flush=True)
+        assert el2 <= 3e-3
 
 
 @pytest.mark.pack_auto
