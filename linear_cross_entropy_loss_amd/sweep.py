@@ -23,6 +23,9 @@ Usage:  python -m linear_cross_entropy_loss_amd.sweep --out DIR
         python -m linear_cross_entropy_loss_amd.sweep --out DIR --heads
             (not one of the reference's protocols: output layers of the sizes of public language models, bf16,
             time and peak memory of a fwd+bwd step beside eager, and the route the library takes; writes DIR/heads.txt)
+        python -m linear_cross_entropy_loss_amd.sweep --out DIR --routes
+            (lce_forward_backward at 25 shapes with the library's choice of route, with exact sums, forced onto one pass
+            and onto two; writes DIR/routes.txt)
 """
 from __future__ import annotations
 
@@ -295,6 +298,85 @@ def run_heads(out, chunk_sizes=(4096, 8192), log=print):
     return path
 
 
+# Shapes (N, H, V, N_chunk_size) on which the library's choice of route is timed against the alternatives.
+ROUTE_SHAPES = [
+    ("headline", 16384, 2048, 131072, 4096), ("config 3's", 16384, 4096, 131072, 4096),
+    ("llama-3-8b", 16384, 4096, 128256, 4096), ("llama-2-7b", 16384, 4096, 32000, 4096),
+    ("qwen-2.5-7b", 8192, 3584, 152064, 4096), ("phi-3-mini", 8192, 3072, 32064, 4096),
+    ("config 4", 16384, 2048, 32768, 2048), ("config 4", 16384, 2048, 65536, 2048), ("config 4", 16384, 2048, 131072, 2048),
+    ("config 4", 16384, 2048, 262144, 2048), ("config 4", 16384, 2048, 32768, 4096), ("config 4", 16384, 2048, 262144, 8192),
+    ("H = 8192", 16384, 8192, 131072, 4096), ("H = 1024", 16384, 1024, 131072, 4096), ("H = 512", 16384, 512, 131072, 4096),
+    ("H = 256", 16384, 256, 131072, 4096), ("V = 16384", 16384, 2048, 16384, 4096), ("V = 8192", 16384, 2048, 8192, 4096),
+    ("V = 4096", 16384, 2048, 4096, 4096), ("N = 65536", 65536, 2048, 131072, 4096), ("N = 4096", 4096, 2048, 131072, 4096),
+    ("N = 1024", 1024, 2048, 131072, 4096), ("small", 8192, 1024, 32768, 4096), ("small", 4096, 512, 4096, 1024),
+    ("small", 2048, 2048, 16384, 4096),
+]
+
+
+def run_routes(out, log=print):
+    """lce_forward_backward through the C ABI, bf16, 5 % of the labels ignored, at each shape of ROUTE_SHAPES with
+    lce_problem.route = LCE_ROUTE_AUTO (the library's choice), the same with LCE_ROUTE_EXACT_SUMS, LCE_ROUTE_ONE_PASS and
+    LCE_ROUTE_TWO_PASS: (chunks, rows per chunk) of the plan -- (0, 0) = two passes -- and ms per call."""
+    import ctypes
+    import time
+
+    import torch
+
+    from . import _lib
+
+    lib = _lib.load()
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    dt = torch.bfloat16
+    routes = (("library", _lib.ROUTE_AUTO), ("exact sums", _lib.ROUTE_AUTO | _lib.ROUTE_EXACT_SUMS),
+              ("one pass", _lib.ROUTE_ONE_PASS), ("two passes", _lib.ROUTE_TWO_PASS))
+    lines = [f"{'shape':<12}{'N':>7}{'H':>6}{'V':>8}{'N_chunk':>8} | "
+             + " | ".join(f"{name:>12}{'ms':>9}" for name, _ in routes) + " | library / fastest"]
+    for name, N, H, V, n_chunk in ROUTE_SHAPES:
+        g = torch.Generator(device="cuda").manual_seed(1)
+        x = torch.randn(N, H, device="cuda", generator=g).to(dt)
+        w = (torch.randn(H, V, device="cuda", generator=g) / math.sqrt(H)).to(dt)
+        y = torch.randint(0, V, (N,), device="cuda", generator=g)
+        y[torch.rand(N, device="cuda", generator=g) < 0.05] = -1
+        lse, out5 = torch.empty(N, device="cuda"), torch.empty(5, device="cuda")
+        nv = torch.empty(1, dtype=torch.int64, device="cuda")
+        dx, dw = torch.empty(N, H, dtype=dt, device="cuda"), torch.empty(H, V, dtype=dt, device="cuda")
+        one = torch.ones(1, device="cuda")
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        cells, times = [], []
+        for _, route in routes:
+            prob = _lib.make_problem(N, H, V, H, V, H, V, dt, dt, dt, dt, -1, 1.0, 0.0, n_chunk, False, route=route)
+            plan = _lib.forward_backward_plan(prob)
+            nbytes = _lib.forward_backward_workspace_bytes(prob)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+
+            def call():
+                rc = lib.lce_forward_backward(ctypes.byref(prob), ptr(x), ptr(w), ptr(y), ptr(one), ptr(lse), ptr(out5), ptr(nv),
+                                              ptr(dx), ptr(dw), ptr(ws), nbytes, stream)
+                _lib.raise_for_status(rc, "lce_forward_backward")
+
+            for _ in range(3):
+                call()
+            torch.cuda.synchronize()
+            reps = 10 if N * H * V < 3e13 else 4
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                call()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) / reps * 1e3
+            times.append(ms)
+            cells.append(f"{str(plan):>12}{ms:>9.3f}")
+            del ws
+        lines.append(f"{name:<12}{N:>7}{H:>6}{V:>8}{n_chunk:>8} | " + " | ".join(cells) + f" | {times[0] / min(times):.3f}")
+        log(lines[-1])
+        del x, w, dx, dw
+        torch.cuda.empty_cache()
+    os.makedirs(out, exist_ok=True)
+    path = os.path.join(out, "routes.txt")
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    return path
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--out", required=True)
@@ -303,7 +385,11 @@ def main(argv=None):
     ap.add_argument("--vars", nargs="+", default=["H", "N", "V"], choices=["H", "N", "V"])
     ap.add_argument("--quick", action="store_true", help="every third point, fewer repetitions")
     ap.add_argument("--heads", action="store_true", help="output layers of the sizes of public language models instead")
+    ap.add_argument("--routes", action="store_true", help="the library's choice of route against the alternatives instead")
     args = ap.parse_args(argv)
+    if args.routes:
+        print("wrote", run_routes(args.out, log=lambda m: print(m, flush=True)), flush=True)
+        return 0
     if args.heads:
         print("wrote", run_heads(args.out, log=lambda m: print(m, flush=True)), flush=True)
         return 0
