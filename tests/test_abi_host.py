@@ -558,3 +558,31 @@ def test_one_pass_plan_stays_within_the_bound_and_covers_all_tokens(lib):
         assert lib.lce_check_problem(ctypes.byref(_lib.make_problem(**dict(kw, w_dtype=torch.bfloat16, dw_dtype=torch.bfloat16, route=r)))) == 0
     for r in (3, 7, 8, -1):
         assert lib.lce_check_problem(ctypes.byref(_lib.make_problem(**dict(kw, w_dtype=torch.bfloat16, dw_dtype=torch.bfloat16, route=r)))) == _lib.LCE_EINVAL_ARG
+
+
+def test_plans_of_the_benchmark_configurations(lib):
+    """What lce_forward_backward plans, by itself, for the benchmark's configurations (host-side only): the headline shape
+    in four chunks of 4096 rows with exact fp32 sums of dW; config 3 and every point of config 4 on the one-pass route
+    within their bounds; config 5 (fp32 master weight, fp32 dW) in ten chunks; config 1 (fp32 tensors) on two passes."""
+    from linear_cross_entropy_loss_amd import _lib
+
+    bf, fh, f32 = torch.bfloat16, torch.float16, torch.float32
+
+    def plan(N, H, V, n_chunk, xd, wd, mon=False, route=_lib.ROUTE_AUTO):
+        p = _lib.make_problem(N, H, V, H, V, H, V, xd, wd, xd, wd, -1, 1.0, 0.0, n_chunk, mon, route=route)
+        return _lib.forward_backward_plan(p), _lib.forward_backward_workspace_bytes(p)
+
+    (chunks, rows), ws = plan(16384, 2048, 131072, 4096, bf, bf)
+    assert (chunks, rows) == (4, 4096) and 2048 * 131072 * 2 + 4096 * 131072 * 2 <= ws <= 4096 * 131072 * 4
+    assert plan(16384, 2048, 131072, 4096, bf, bf, route=_lib.ROUTE_AUTO | _lib.ROUTE_EXACT_SUMS)[0] == (4, 4096)
+    (chunks, rows), ws = plan(16384, 4096, 131072, 4096, fh, fh, mon=True)
+    assert (chunks, rows) == (4, 4096) and ws <= 4096 * 131072 * 4
+    (chunks, rows), _ = plan(16384, 4096, 131072, 4096, fh, fh, mon=True, route=_lib.ROUTE_AUTO | _lib.ROUTE_EXACT_SUMS)
+    assert chunks > 4 and rows < 4096  # (exact sums: two bytes per sum in the workspace leave shorter chunks)
+    for V in (32768, 65536, 131072, 262144):
+        for n_chunk in (2048, 4096, 8192):
+            (chunks, rows), ws = plan(16384, 2048, V, n_chunk, bf, bf)
+            assert chunks >= 1 and chunks * rows >= 16384 and ws <= n_chunk * V * 4, (V, n_chunk, chunks, rows, ws)
+    (chunks, rows), ws = plan(65536, 8192, 262144, 8192, fh, f32)
+    assert chunks == 10 and ws <= 8192 * 262144 * 4
+    assert plan(2048, 2048, 16384, 4096, f32, f32)[0] == (0, 0)
