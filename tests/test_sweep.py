@@ -45,3 +45,24 @@ def test_tiny_sweep_end_to_end(tmp_path, monkeypatch):
             assert math.isfinite(v) and v >= 0
             if "Accuracy" in f:
                 assert v < 5e-2
+
+
+@pytest.mark.gpu
+def test_heads_and_routes_tables_end_to_end(tmp_path, monkeypatch):
+    """The two tables that are not the reference's protocols, on shapes small enough for a test: one line per shape, the
+    plan of each column in the routes table, finite times."""
+    print("heads / routes tables", flush=True)
+    monkeypatch.setattr(sweep, "HEADS", [("tiny", 1024, 256, 4096), ("odd", 1000, 264, 5000)])
+    path = sweep.run_heads(str(tmp_path), chunk_sizes=(512, 4096), log=lambda m: None)
+    lines = open(path).read().strip().split("\n")
+    assert len(lines) == 3 and lines[1].startswith("tiny") and lines[2].startswith("odd")
+    for line in lines[1:]:
+        assert "nan" not in line and ("one," in line or "two passes" in line)
+    monkeypatch.setattr(sweep, "ROUTE_SHAPES", [("tiny", 2048, 256, 4096, 512), ("tiny", 1024, 512, 8192, 4096)])
+    path = sweep.run_routes(str(tmp_path), log=lambda m: None)
+    lines = open(path).read().strip().split("\n")
+    assert len(lines) == 3
+    for line in lines[1:]:
+        cells = line.split("|")
+        assert len(cells) == 6 and cells[4].strip().startswith("(0, 0)")  # (the last route column: two passes)
+        assert 1.0 <= float(cells[5]) < 3.0
